@@ -1,0 +1,21 @@
+"""CPU oracle for the ReBeL search hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product package (``poker2_amd``)
+may import, call or link anything in this directory.  The only permitted users
+are ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py``, and there only as the checker or as the timed CPU baseline,
+never as a compute path that ships.
+
+Every function restates, in numpy (plus a small C file for the integer
+ranker), what the reference computes, and cites the reference file:line it
+follows.  How each function is pinned (reference-held vectors, golden fixtures
+written by running the reference's own ``rules.py`` / ``hunl_tensor_env.py`` in
+the build container, closed forms, brute force) is listed per module.
+
+Parity status
+-------------
+* cards, ranker, unblocked mass, showdown, betting tree: pinned (see modules).
+* cfr (multi-iteration numeric values): **parity unpinned** by any
+  reference-held vector; pinned only by per-step identities, game-theoretic
+  invariants and brute force on tiny ranges (see ``oracle/cfr.py``).
+"""
