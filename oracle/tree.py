@@ -200,3 +200,19 @@ def build_tree(roots: list[Node], bins: list[float], depth: int, bb: int = 100) 
     out["showdown_mask"] = out["street"] == 4
     out["showdown_potential"] = out["stacks"] + out["pot"][:, None] - out["starting_stacks"]
     return out
+
+
+def make_root(street: int, pot: int, stack0: int, stack1: int, button: int = 0,
+              bb: int = 100, starting: tuple[int, int] | None = None,
+              scale: float | None = None) -> Node:
+    """A root at the start of a betting round: nothing committed, first to act
+    is the non-button player (``hunl_tensor_env.py:892``).  By default each
+    player is taken to have put half the pot in already."""
+    if starting is None:
+        starting = (stack0 + pot // 2, stack1 + pot // 2)
+    if scale is None:
+        scale = float(starting[0])
+    return Node(to_act=1 - button, button=button, street=street, pot=pot,
+                stacks=[stack0, stack1], committed=[0, 0], min_raise=bb,
+                actions_this_round=0, is_allin=[False, False],
+                starting_stacks=list(starting), scale=scale)
