@@ -1,0 +1,177 @@
+/* libp2hip.so -- C ABI of the MI355X (gfx950) kernels for the ReBeL search hot path.
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; all pointers are DEVICE pointers unless named host_*;
+ *   - H = 1326 hole-card combos, combo (a<b) at index a*(103-a)/2 + (b-a-1); float32
+ *     data rows are H floats, row-major, contiguous; index arrays are int64; masks are
+ *     one byte per element (0 / non-zero); float rows must be 8-byte aligned;
+ *   - work is enqueued on `stream` (a hipStream_t, NULL = default stream); nothing
+ *     synchronises, allocates or keeps a pointer after returning;
+ *   - return value: 0 on success, otherwise a hipError_t (1 = invalid argument).
+ *
+ * The reference (phulin/poker2) has no FFI: the interface each function replaces is the
+ * Python/Triton wrapper cited next to it (paths relative to the reference's src/p2/).
+ */
+#ifndef P2HIP_H
+#define P2HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int p2hip_abi_version(void);
+int p2hip_device_count(void);
+const char* p2hip_error_string(int code);
+
+/* ---- 7-card hand ranker -------------------------------------------------------- */
+
+/* cards [n,7] ids 0..51 of elem_size bytes (1, 2 or 8) -> out[n] packed int32 score
+ * (type nibble << 20 | five kicker nibbles).  Replaces rank_7_cards_single_batch_triton,
+ * env/rules_triton.py:96-117 (kernel :617-632). */
+int p2hip_rank7_cards(const void* cards, int elem_size, int64_t n, int32_t* out, void* stream);
+
+/* cards [n,2,7] -> out[n] in {-1,0,1}, 1 = first hand stronger.  Replaces
+ * compare_7_cards_single_batch_triton, env/rules_triton.py:78-93 (kernel :600-614). */
+int p2hip_compare7_cards(const void* cards, int elem_size, int64_t n, int32_t* out, void* stream);
+
+/* planes [n,4,13] bytes -> packed score.  flush_first = 1: flush suit is the first suit
+ * with >= 5 ranks (env/rules_triton.py:229-242); 0: the fullest suit (env/rules.py:215-219).
+ * Replaces create_comparison_vector + packing, env/rules.py:136-299, :406-407. */
+int p2hip_rank7_planes(const uint8_t* planes, int64_t n, int32_t* out, int flush_first, void* stream);
+
+/* planes [n,2,4,13] bytes -> out[n] in {-1,0,1}.  Replaces compare_7_single_batch
+ * (env/rules.py:390-409) and compare_7_single_batch_triton (env/rules_triton.py:36-51). */
+int p2hip_compare7_planes(const uint8_t* planes, int64_t n, int32_t* out, int flush_first, void* stream);
+
+/* ---- river showdown --------------------------------------------------------------- */
+
+/* Bytes of one per-board strength table (fixed). */
+int64_t p2hip_showdown_table_bytes(void);
+
+/* boards [m,5] ids of elem_size bytes (1,2,4,8).  Any of the three outputs may be NULL.
+ *   mode 0: combos touching the board are ranked as 6-card hands; ranks_out [m,H] int32 =
+ *           dense 1-based strength group ids            (rank_hands, env/rules.py:66-133)
+ *   mode 1: 7 card ids, hole cards first, repeated ids count twice; ranks_out = packed scores
+ *                                                 (rank_hands_triton, env/rules_triton.py:120-148)
+ *   order_out [m,H] int64: stable ascending argsort of the scores;
+ *   table_out [m, p2hip_showdown_table_bytes()]: what p2hip_showdown_both reads; replaces the
+ *           HandRankData built by _init_hand_rank_data, search/cfr_evaluator.py:406-482. */
+int p2hip_showdown_setup(const void* boards, int elem_size, int64_t m, int mode, int32_t* ranks_out,
+                         int64_t* order_out, uint8_t* table_out, void* stream);
+
+/* beliefs [m,2,H] -> out [m,2,H]: blocker-corrected showdown EV of both players per hand,
+ * times potential[m,p] / scale[m].  table_row [m] (or NULL = identity) selects the board
+ * table of each node.  Replaces _showdown_value_both / _showdown_value,
+ * search/cfr_evaluator.py:484-601. */
+int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64_t* table_row,
+                        const float* potential, const float* scale, int64_t m, float* out, void* stream);
+
+/* ---- unblocked (card-compatible) mass --------------------------------------------- */
+
+/* target [rows,H] -> out [rows,H] = max(S - cs[a] - cs[b] + t, 0).  Replaces
+ * calculate_unblocked_mass (env/card_utils.py:196-222) and unblocked_mass_triton
+ * (search/fused_cfr_triton.py:1110-1157). */
+int p2hip_unblocked_mass(const float* target, int64_t rows, float* out, void* stream);
+
+/* beliefs [total,2,H], to_act [total]; out[r] = unblocked(beliefs[r, to_act[r] ^ opponent])
+ * for r < top.  Replaces unblocked_mass_opp_at_parents_triton,
+ * search/fused_cfr_triton.py:1067-1107. */
+int p2hip_unblocked_mass_by_player(const float* beliefs, const int64_t* to_act, int64_t top, int opponent,
+                                   float* out, void* stream);
+
+/* out[c] = d > eps ? unblocked(numer[c]) / d : 0, d = unblocked(denom[parent_index[c]])
+ * (parent_index NULL = identity).  Replaces unblocked_mass_ratio_indirect_triton /
+ * unblocked_mass_ratio_triton, search/fused_cfr_triton.py:1499-1602. */
+int p2hip_unblocked_mass_ratio(const float* numer, const float* denom, const int64_t* parent_index,
+                               int64_t rows, float eps, float* out, void* stream);
+
+/* ---- per-operation CFR kernels (search/fused_cfr_triton.py) ------------------------- */
+/* Scalars that depend on the iteration number are 0-D device tensors (const float*). */
+
+/* fused_dcfr_update_with_tensors_ :200-235 (kernel :71-120).  n = element count (even).
+ * positive_out may be NULL. */
+int p2hip_dcfr_update(float* cumulative_regrets, float* regret_weight_sums, const float* regrets,
+                      const float* t_alpha_num, const float* t_beta_num, const float* t_alpha_den,
+                      const float* t_beta_den, int64_t n, int apply_dcfr, int cfr_plus, float* positive_out,
+                      void* stream);
+
+/* fused_block_and_normalize_beliefs_ :286-335.  target has rows*1 rows of H; row r uses
+ * mask / fallback row r / players_per_row. */
+int p2hip_block_and_normalize(float* target, const uint8_t* allowed, const float* allowed_prob, int64_t rows,
+                              int players_per_row, float eps, void* stream);
+
+/* fused_regret_matching_divide_ :369-399 */
+int p2hip_regret_matching_divide(const float* positive, const float* denom, const float* fallback, float* out,
+                                 int64_t n, float eps, void* stream);
+
+/* fused_weight_child_values :438-477; values/out [m,2,H] */
+int p2hip_weight_child_values(const float* values, const int64_t* prev_actor, const float* policy_hero,
+                              const float* policy_opp, float* out, int64_t m, void* stream);
+
+/* fused_update_average_values_with_tensors_ :538-560 */
+int p2hip_update_average_values(float* values_avg, const float* latest, const float* old_w, const float* new_w,
+                                const float* inv_total, int64_t n, void* stream);
+
+/* fused_avg_values_zero_sum_ :623-668; ignore_mask [nodes] bytes or NULL */
+int p2hip_avg_values_zero_sum(float* values_avg, const float* latest, const float* beliefs,
+                              const uint8_t* ignore_mask, const float* old_w, const float* new_w,
+                              const float* inv_total, int64_t nodes, int enforce_zero_sum, void* stream);
+
+/* fused_regret_tail_ :712-766; writes rows [bottom,total) of regrets */
+int p2hip_regret_tail(float* regrets, const float* values_achieved, const float* actor_values,
+                      const float* src_weights, const int64_t* parent_index, const int64_t* prev_actor,
+                      int64_t bottom, int64_t total, void* stream);
+
+/* fused_average_policy_mix_with_tensors_ :879-914 */
+int p2hip_average_policy_mix(float* policy_probs_avg, const float* policy_probs, const float* self_reach,
+                             const float* self_reach_avg, const int64_t* to_act, const int64_t* parent_index,
+                             const float* old_w, const float* new_w, const float* total_w, int64_t bottom,
+                             int64_t total, float eps, void* stream);
+
+/* fused_parent_sum :1279-1313 -> out [num_parents,H] */
+int p2hip_parent_sum(const float* values, const int64_t* child_offsets, const int64_t* child_count,
+                     int64_t num_parents, float* out, void* stream);
+
+/* fused_sibling_sum :1355-1398 -> out [num_children,H], row = child - bottom */
+int p2hip_sibling_sum(const float* values, const int64_t* child_offsets, const int64_t* child_count,
+                      int64_t num_parents, int64_t bottom, float* out, void* stream);
+
+/* fused_divide_by_parent_sum_ :1316-1352; out may alias pos or fallback */
+int p2hip_divide_by_parent_sum(const float* pos, const float* fallback, const float* parent_sum,
+                               const int64_t* parent_index, float* out, int64_t num_children, float eps,
+                               void* stream);
+
+/* fused_model_values_mix_with_tensors :1658-1680 */
+int p2hip_model_values_mix(const float* hand_values, const float* last_values, const float* onon,
+                           const float* oon, float* out, int64_t n, void* stream);
+
+/* fused_model_values_mix_zero_sum :1739-1775; tensors [rows,2,H] */
+int p2hip_model_values_mix_zero_sum(const float* hand_values, const float* last_values, const float* beliefs,
+                                    const float* onon, const float* oon, float* out, int64_t rows,
+                                    int enforce_zero_sum, void* stream);
+
+/* fused_weighted_parent_sum :1838-1889; child_offsets/count already sliced to the depth */
+int p2hip_weighted_parent_sum(float* values, const int64_t* prev_actor, const float* policy_hero,
+                              const float* policy_opp, const int64_t* child_offsets, const int64_t* child_count,
+                              int64_t num_parents, int64_t parent_base, void* stream);
+
+/* fused_reach_weights_depth_ :1944-1986; rows [start,end) */
+int p2hip_reach_weights_depth(float* reach, const float* policy, const uint8_t* allowed_mask,
+                              const int64_t* parent_index, const int64_t* prev_actor, int64_t start, int64_t end,
+                              void* stream);
+
+/* fused_deep_beliefs_ :2039-2092; rows [n_roots,total) are written */
+int p2hip_deep_beliefs(float* out, const float* root_beliefs, const float* reach, const float* allowed_prob,
+                       const int64_t* root_index, int64_t n_roots, int64_t total, float eps, void* stream);
+
+/* policy_probs_sample <- where(t_sample == *t_now, policy_probs, policy_probs_sample),
+ * search/fused_sparse_cfr_evaluator.py:494-499 */
+int p2hip_sample_snapshot(const float* policy_probs, float* policy_probs_sample, const int64_t* t_sample,
+                          const int64_t* t_now, int64_t total, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* P2HIP_H */

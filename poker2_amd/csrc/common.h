@@ -1,0 +1,108 @@
+// Shared device helpers for the gfx950 kernels: combo tables, wave64 / block
+// reductions and scans, launch checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define P2_H 1326          // hole-card combos
+#define P2_HPAIRS 663      // float2 pairs per 1326-float row (5304 B, 8-byte aligned)
+#define P2_CARDS 52
+#define P2_WAVE 64
+
+// Every entry point returns hipError_t as int; argument errors use this value.
+#define P2_EINVAL 1  // == hipErrorInvalidValue
+
+#define P2_LAUNCH_CHECK()                         \
+  do {                                            \
+    hipError_t e__ = hipGetLastError();           \
+    if (e__ != hipSuccess) return (int)e__;       \
+  } while (0)
+
+// combo index h -> its two cards (a < b), lexicographic order:
+// h = a*(103-a)/2 + (b-a-1)   (src/p2/env/card_utils.py:58-68)
+struct P2ComboTable {
+  uint8_t a[P2_H];
+  uint8_t b[P2_H];
+  uint16_t row_start[P2_CARDS + 1];  // first index of combos whose low card is a
+  constexpr P2ComboTable() : a(), b(), row_start() {
+    int k = 0;
+    for (int c1 = 0; c1 < P2_CARDS; ++c1) {
+      row_start[c1] = (uint16_t)k;
+      for (int c2 = c1 + 1; c2 < P2_CARDS; ++c2) {
+        a[k] = (uint8_t)c1;
+        b[k] = (uint8_t)c2;
+        ++k;
+      }
+    }
+    row_start[P2_CARDS] = (uint16_t)k;
+  }
+};
+
+__device__ const P2ComboTable p2_combo = P2ComboTable();
+
+__device__ __forceinline__ int p2_combo_index(int lo, int hi) {
+  return (lo * (103 - lo)) / 2 + (hi - lo - 1);
+}
+
+// ---- wave64 primitives ------------------------------------------------------
+__device__ __forceinline__ float p2_wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, P2_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ double p2_wave_sum(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, P2_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float p2_wave_scan_incl(float v, int lane) {
+#pragma unroll
+  for (int off = 1; off < P2_WAVE; off <<= 1) {
+    float o = __shfl_up(v, off, P2_WAVE);
+    if (lane >= off) v += o;
+  }
+  return v;
+}
+
+// Block-wide sum of one float per thread; `red` needs >= blockDim/64 floats.
+// All threads get the result.  Contains two barriers.
+template <int NWAVES>
+__device__ __forceinline__ float p2_block_sum(float v, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v = p2_wave_sum(v);
+  __syncthreads();  // protect `red` from a previous use
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int w = 0; w < NWAVES; ++w) s += red[w];
+  return s;
+}
+
+template <int NWAVES>
+__device__ __forceinline__ double p2_block_sum(double v, double* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v = p2_wave_sum(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  double s = 0.0;
+#pragma unroll
+  for (int w = 0; w < NWAVES; ++w) s += red[w];
+  return s;
+}
+
+// 8-byte vector view of a 1326-float row (row stride 5304 B keeps 8-byte alignment
+// as long as the tensor base is 8-byte aligned; the host wrappers check that).
+__device__ __forceinline__ const float2* p2_row2(const float* base, int64_t row) {
+  return reinterpret_cast<const float2*>(base + row * P2_H);
+}
+__device__ __forceinline__ float2* p2_row2(float* base, int64_t row) {
+  return reinterpret_cast<float2*>(base + row * P2_H);
+}
+
+static inline bool p2_aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+static inline bool p2_aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }

@@ -1,0 +1,357 @@
+// River showdown: per-board strength tables (built once per subgame) and the
+// per-iteration blocker-corrected EV of both players.
+//
+// Replaces rank_hands (src/p2/env/rules.py:66-133, rules_triton.py:120-148),
+// _init_hand_rank_data (src/p2/search/cfr_evaluator.py:406-482) and
+// _showdown_value / _showdown_value_both (:484-601).  The reference prefix-sums a
+// [M,1327,52] tensor per call; here each card keeps only its own 51 combos in
+// strength order, so one call is three short LDS scans per player:
+//   P[k]        prefix of the villain range in strength order (k = 0..1326)
+//   Pc[c][j]    prefix over the j weakest of the 51 combos holding card c
+//   hero (a,b) at sorted position k with tie group [L,R):
+//     win = P[L] - Pc[a][iLa] - Pc[b][iLb]
+//     tie = P[R]-P[L] - (Pc[a][iRa]-Pc[a][iLa]) - (Pc[b][iRb]-Pc[b][iLb]) + v[k]
+//     den = max(1 - Pc[a][51] - Pc[b][51] + v[k], 1e-8)
+// where iLa = how many of card a's combos lie strictly below the tie group, etc.
+#include "common.h"
+#include "ranker.hip"
+
+namespace p2 {
+
+// ---- per-board table layout (bytes) ------------------------------------------
+// perm     u16[1326]  sorted position -> combo index; bit 15 = combo blocked by the board
+// lr       u16[1326][2]  tie group [L, R) of the sorted position
+// cidx     u8 [1326][4]  iLa, iRa, iLb, iRb (see above)
+// clist    u16[52][51]   sorted positions of the combos holding card c, ascending;
+//                        all 0xFFFF for a board card (its column is masked out)
+constexpr int SD_OFF_PERM = 0;
+constexpr int SD_OFF_LR = SD_OFF_PERM + P2_H * 2;
+constexpr int SD_OFF_CIDX = SD_OFF_LR + P2_H * 4;
+constexpr int SD_OFF_CLIST = SD_OFF_CIDX + P2_H * 4;
+constexpr int SD_TABLE_USED = SD_OFF_CLIST + P2_CARDS * 51 * 2;  // 18564
+constexpr int SD_TABLE_BYTES = 18688;                             // padded to 256 B
+static_assert(SD_TABLE_USED <= SD_TABLE_BYTES, "table layout");
+
+constexpr int SD_BLOCK = 256;
+constexpr int SD_WAVES = SD_BLOCK / 64;
+constexpr int SORT_N = 2048;
+
+// Block-wide bitonic sort of 2048 uint64 keys in LDS, ascending.
+__device__ void bitonic_sort_2048(unsigned long long* keys) {
+  for (int k = 2; k <= SORT_N; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      __syncthreads();
+      for (int i = threadIdx.x; i < SORT_N; i += SD_BLOCK) {
+        const int ixj = i ^ j;
+        if (ixj > i) {
+          const unsigned long long x = keys[i], y = keys[ixj];
+          const bool up = (i & k) == 0;
+          if ((x > y) == up) { keys[i] = y; keys[ixj] = x; }
+        }
+      }
+    }
+  }
+  __syncthreads();
+}
+
+template <typename T>
+__device__ __forceinline__ int board_card(const void* boards, int64_t m, int j) {
+  return (int)reinterpret_cast<const T*>(boards)[m * 5 + j];
+}
+
+// One workgroup per board.
+//   mode 0: score = union of hole and board planes (a combo touching the board is a
+//           6-card hand), rules.py:86-102; ranks_out = dense 1-based group ids
+//   mode 1: score from the 7 card ids, hole cards first (a repeated id counts twice),
+//           rules_triton.py:139-148; ranks_out = packed scores
+// ranks_out [M,1326] int32, order_out [M,1326] int64 (stable ascending argsort) and
+// table_out are each optional.
+__global__ __launch_bounds__(SD_BLOCK) void showdown_setup_kernel(const void* __restrict__ boards, int elem_size,
+                                                                   int mode, int32_t* __restrict__ ranks_out,
+                                                                   int64_t* __restrict__ order_out,
+                                                                   uint8_t* __restrict__ table_out) {
+  __shared__ unsigned long long keys[SORT_N];
+  __shared__ uint16_t pos_of[P2_H];       // combo -> sorted position
+  __shared__ uint16_t clist[P2_CARDS][52];
+  __shared__ int scan_tmp[SD_WAVES];
+  __shared__ int bcards[5];
+  const int64_t m = blockIdx.x;
+  if (threadIdx.x < 5) {
+    int c = elem_size == 1 ? board_card<int8_t>(boards, m, threadIdx.x)
+          : elem_size == 2 ? board_card<int16_t>(boards, m, threadIdx.x)
+          : elem_size == 4 ? board_card<int32_t>(boards, m, threadIdx.x)
+                           : board_card<int64_t>(boards, m, threadIdx.x);
+    bcards[threadIdx.x] = c;
+  }
+  __syncthreads();
+  uint32_t bs[4] = {0, 0, 0, 0};
+  unsigned long long board_bits = 0;
+  for (int j = 0; j < 5; ++j) {
+    const uint32_t c = (uint32_t)bcards[j];
+    if (c < 52u) { bs[c / 13u] |= 1u << (c % 13u); board_bits |= 1ull << c; }
+  }
+  for (int h = threadIdx.x; h < SORT_N; h += SD_BLOCK) {
+    unsigned long long key = ~0ull;
+    if (h < P2_H) {
+      const int a = p2_combo.a[h], b = p2_combo.b[h];
+      int32_t sc;
+      if (mode == 0) {
+        uint32_t s[4] = {bs[0], bs[1], bs[2], bs[3]};
+        s[a / 13] |= 1u << (a % 13);
+        s[b / 13] |= 1u << (b % 13);
+        sc = score_hand(hand_from_suits(s[0], s[1], s[2], s[3]), false);
+      } else {
+        CardAcc acc;
+        acc.add(a);
+        acc.add(b);
+        for (int j = 0; j < 5; ++j)
+          if ((uint32_t)bcards[j] < 52u) acc.add(bcards[j]);
+        sc = score_hand(acc.finish(), true);
+      }
+      key = ((unsigned long long)(uint32_t)sc << 11) | (unsigned long long)h;
+    }
+    keys[h] = key;
+  }
+  bitonic_sort_2048(keys);  // ties resolve by combo index: a stable argsort
+
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const unsigned long long key = keys[k];
+    const int h = (int)(key & 2047ull);
+    pos_of[h] = (uint16_t)k;
+    if (order_out) order_out[m * P2_H + k] = h;
+    if (mode == 1 && ranks_out) ranks_out[m * P2_H + h] = (int32_t)(key >> 11);
+  }
+  __syncthreads();
+
+  // dense group ids (mode 0): 1 + number of group starts at sorted positions 1..k
+  if (mode == 0 && ranks_out) {
+    // each thread owns 6 consecutive sorted positions (256*6 = 1536 >= 1326)
+    const int k0 = threadIdx.x * 6;
+    int flags[6], local = 0;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      const int k = k0 + i;
+      flags[i] = (k > 0 && k < P2_H && (keys[k] >> 11) != (keys[k - 1] >> 11)) ? 1 : 0;
+      local += flags[i];
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = local;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      int o = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += o;
+    }
+    if (lane == 63) scan_tmp[wave] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += scan_tmp[w];
+    int run = base + incl - local;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      const int k = k0 + i;
+      run += flags[i];
+      if (k < P2_H) ranks_out[m * P2_H + (int)(keys[k] & 2047ull)] = run + 1;
+    }
+  }
+  if (!table_out) return;
+  uint16_t* t_perm = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_PERM);
+  uint16_t* t_lr = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_LR);
+
+  // per-card lists: position of each of the 51 combos of card c, sorted ascending by
+  // counting how many of the other 50 lie below (positions are distinct)
+  for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) {
+    const int c = e / 51, j = e % 51;
+    const int x = j < c ? j : j + 1;
+    const int mine = pos_of[p2_combo_index(x < c ? x : c, x < c ? c : x)];
+    int below = 0;
+    for (int jj = 0; jj < 51; ++jj) {
+      const int y = jj < c ? jj : jj + 1;
+      below += pos_of[p2_combo_index(y < c ? y : c, y < c ? c : y)] < mine ? 1 : 0;
+    }
+    clist[c][below] = (uint16_t)mine;
+  }
+  __syncthreads();
+  uint16_t* t_clist = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_CLIST);
+  for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) {
+    const int c = e / 51, j = e % 51;
+    const bool on_board = (board_bits >> c) & 1ull;
+    t_clist[e] = on_board ? (uint16_t)0xFFFF : clist[c][j];
+  }
+  uint8_t* t_cidx = table_out + m * SD_TABLE_BYTES + SD_OFF_CIDX;
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const unsigned long long key = keys[k];
+    const unsigned long long sc = key >> 11;
+    const int h = (int)(key & 2047ull);
+    // [L, R): first position with this score, first position with a larger one
+    int lo = 0, hi = k;
+    while (lo < hi) { int mid = (lo + hi) >> 1; if ((keys[mid] >> 11) < sc) lo = mid + 1; else hi = mid; }
+    const int L = lo;
+    lo = k + 1; hi = P2_H;
+    while (lo < hi) { int mid = (lo + hi) >> 1; if ((keys[mid] >> 11) <= sc) lo = mid + 1; else hi = mid; }
+    const int R = lo;
+    const int a = p2_combo.a[h], b = p2_combo.b[h];
+    const bool blocked = ((board_bits >> a) | (board_bits >> b)) & 1ull;
+    t_perm[k] = (uint16_t)(h | (blocked ? 0x8000 : 0));
+    t_lr[2 * k] = (uint16_t)L;
+    t_lr[2 * k + 1] = (uint16_t)R;
+    int cnt[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c = q < 2 ? a : b;
+      const int bound = (q & 1) ? R : L;
+      int n = 0;  // entries of card c's list strictly below `bound`
+      int l2 = 0, h2 = 51;
+      while (l2 < h2) { int mid = (l2 + h2) >> 1; if ((int)clist[c][mid] < bound) l2 = mid + 1; else h2 = mid; }
+      n = l2;
+      cnt[q] = n;
+    }
+    t_cidx[4 * k + 0] = (uint8_t)cnt[0];
+    t_cidx[4 * k + 1] = (uint8_t)cnt[1];
+    t_cidx[4 * k + 2] = (uint8_t)cnt[2];
+    t_cidx[4 * k + 3] = (uint8_t)cnt[3];
+  }
+}
+
+// ---- per-call evaluation ---------------------------------------------------------
+// Everything the evaluation of one node needs in LDS.
+struct ShowdownLds {
+  float v[2][P2_H + 2];        // villain-of-hero-p range in strength order: v[p] = beliefs[1-p] sorted
+  float P[2][P2_H + 2];        // exclusive prefix, P[p][k], k = 0..1326
+  float Pc[2][P2_CARDS][52];   // per-card exclusive prefix, Pc[p][c][j], j = 0..51
+  float part[2][SD_WAVES];
+};
+
+// Fill s.v / s.P / s.Pc for the node whose beliefs start at `bel` ([2,H]) using the
+// board table `tab`.  Ends with a barrier.
+__device__ __forceinline__ void showdown_scan(const float* __restrict__ bel, const uint8_t* __restrict__ tab,
+                                              ShowdownLds& s) {
+  const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
+  const uint16_t* clist = reinterpret_cast<const uint16_t*>(tab + SD_OFF_CLIST);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // gather both ranges into strength order; hero p faces villain 1-p
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const int h = perm[k] & 0x7FFF;
+    s.v[0][k] = bel[P2_H + h];
+    s.v[1][k] = bel[h];
+  }
+  __syncthreads();
+  // block scan: thread owns 6 consecutive positions
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int k0 = threadIdx.x * 6;
+    float x[6], local = 0.f;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) { x[i] = (k0 + i < P2_H) ? s.v[p][k0 + i] : 0.f; local += x[i]; }
+    const float incl = p2_wave_scan_incl(local, lane);
+    if (lane == 63) s.part[p][wave] = incl;
+    __syncthreads();
+    float base = 0.f;
+    for (int w = 0; w < wave; ++w) base += s.part[p][w];
+    float run = base + (incl - local);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      if (k0 + i <= P2_H) s.P[p][k0 + i] = run;
+      run += x[i];
+    }
+  }
+  // per-card prefixes: one wave scan per (player, card)
+  for (int q = wave; q < 2 * P2_CARDS; q += SD_WAVES) {
+    const int p = q / P2_CARDS, c = q % P2_CARDS;
+    float x = 0.f;
+    if (lane < 51) {
+      const unsigned pos = clist[c * 51 + lane];
+      x = pos < (unsigned)P2_H ? s.v[p][pos] : 0.f;
+    }
+    const float incl = p2_wave_scan_incl(x, lane);
+    if (lane < 51) s.Pc[p][c][lane + 1] = incl;
+    if (lane == 0) s.Pc[p][c][0] = 0.f;
+  }
+  __syncthreads();
+}
+
+// EV of hero p for the hand at sorted position k (before the potential/scale factor).
+__device__ __forceinline__ float showdown_ev_at(const ShowdownLds& s, int p, int k, int h, int L, int R,
+                                                uchar4 ci) {
+  const int a = p2_combo.a[h], b = p2_combo.b[h];
+  const float vk = s.v[p][k];
+  const float PL = s.P[p][L], PR = s.P[p][R];
+  const float aL = s.Pc[p][a][ci.x], aR = s.Pc[p][a][ci.y];
+  const float bL = s.Pc[p][b][ci.z], bR = s.Pc[p][b][ci.w];
+  const float win = PL - aL - bL;
+  const float tie = (PR - PL) - (aR - aL) - (bR - bL) + vk;
+  float den = 1.0f - s.Pc[p][a][51] - s.Pc[p][b][51] + vk;
+  den = fmaxf(den, 1e-8f);
+  const bool valid = den > 1e-8f;
+  const float wp = valid ? win / den : 0.f;
+  const float tp = valid ? tie / den : 0.f;
+  const float lp = valid ? 1.0f - wp - tp : 0.f;
+  return wp - lp;
+}
+
+// out[n] = showdown EV of both players at node n.
+//   beliefs   [M,2,H]      range pair per node
+//   table_row [M] or null  row of `tables` to use for node n (null: row n)
+//   potential [M,2] float  chips won by player p if he wins; scale [M]
+__global__ __launch_bounds__(SD_BLOCK) void showdown_both_kernel(const float* __restrict__ beliefs,
+                                                                  const uint8_t* __restrict__ tables,
+                                                                  const int64_t* __restrict__ table_row,
+                                                                  const float* __restrict__ potential,
+                                                                  const float* __restrict__ scale,
+                                                                  float* __restrict__ out) {
+  __shared__ ShowdownLds s;
+  const int64_t n = blockIdx.x;
+  const int64_t row = table_row ? table_row[n] : n;
+  const uint8_t* tab = tables + row * SD_TABLE_BYTES;
+  showdown_scan(beliefs + n * 2 * P2_H, tab, s);
+  const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
+  const uint16_t* lr = reinterpret_cast<const uint16_t*>(tab + SD_OFF_LR);
+  const uchar4* cidx = reinterpret_cast<const uchar4*>(tab + SD_OFF_CIDX);
+  const float sc = scale[n];
+  const float pot0 = potential[2 * n], pot1 = potential[2 * n + 1];
+  float* o = out + n * 2 * P2_H;
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const unsigned pk = perm[k];
+    const int h = pk & 0x7FFF;
+    const bool blocked = pk & 0x8000u;
+    const int L = lr[2 * k], R = lr[2 * k + 1];
+    const uchar4 ci = cidx[k];
+    float e0 = showdown_ev_at(s, 0, k, h, L, R, ci);
+    float e1 = showdown_ev_at(s, 1, k, h, L, R, ci);
+    e0 = e0 * (blocked ? 0.f : 1.f);
+    e1 = e1 * (blocked ? 0.f : 1.f);
+    o[h] = e0 * pot0 / sc;
+    o[P2_H + h] = e1 * pot1 / sc;
+  }
+}
+
+}  // namespace p2
+
+extern "C" {
+
+int64_t p2hip_showdown_table_bytes(void) { return p2::SD_TABLE_BYTES; }
+
+int p2hip_showdown_setup(const void* boards, int elem_size, int64_t m, int mode, int32_t* ranks_out,
+                         int64_t* order_out, uint8_t* table_out, void* stream) {
+  if (m < 0 || (m > 0 && !boards)) return P2_EINVAL;
+  if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8) return P2_EINVAL;
+  if (mode != 0 && mode != 1) return P2_EINVAL;
+  if (m == 0) return 0;
+  if (table_out && !p2_aligned8(table_out)) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::showdown_setup_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
+                     boards, elem_size, mode, ranks_out, order_out, table_out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64_t* table_row,
+                        const float* potential, const float* scale, int64_t m, float* out, void* stream) {
+  if (m < 0 || (m > 0 && (!beliefs || !tables || !potential || !scale || !out))) return P2_EINVAL;
+  if (m == 0) return 0;
+  if (!p2_aligned8(tables) || !p2_aligned4(beliefs) || !p2_aligned4(out)) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::showdown_both_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
+                     beliefs, tables, table_row, potential, scale, out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,57 @@
+"""CPU: the C-ABI library loads and exports every symbol include/p2hip.h declares; the
+product package never touches the oracle."""
+import os
+import re
+
+from tests.conftest import ROOT
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "p2hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(p2hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from poker2_amd import _lib
+    lib = _lib.load()
+    syms = header_symbols()
+    assert len(syms) >= 30
+    for name in syms:
+        assert hasattr(lib, name), name
+    assert sorted(_lib.declared_symbols()) == syms
+    assert lib.p2hip_abi_version() >= 1
+    assert lib.p2hip_showdown_table_bytes() % 256 == 0
+
+
+def test_argument_errors_without_a_gpu():
+    from poker2_amd import _lib
+    lib = _lib.load()
+    # negative sizes / null pointers are rejected before any launch
+    assert lib.p2hip_unblocked_mass(None, -1, None, None) == 1
+    assert lib.p2hip_unblocked_mass(None, 3, None, None) == 1
+    assert lib.p2hip_rank7_cards(None, 3, 5, None, None) == 1
+    assert lib.p2hip_dcfr_update(None, None, None, None, None, None, None, 3, 1, 0, None, None) == 1
+    assert lib.p2hip_unblocked_mass(None, 0, None, None) == 0
+
+
+def test_product_never_imports_oracle():
+    pkg = os.path.join(ROOT, "poker2_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(base, f)).read()
+                assert "oracle" not in text.replace("oracle/", "oracle/"), f
+
+
+def test_wrappers_fail_loudly_without_gpu():
+    import pytest
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    from poker2_amd import fused_cfr_hip, rules_hip
+    assert not fused_cfr_hip.triton_is_available()
+    with pytest.raises((RuntimeError, ValueError)):
+        rules_hip.rank_7_cards_single_batch_triton(torch.zeros(4, 7, dtype=torch.int16))
+    with pytest.raises((RuntimeError, ValueError)):
+        fused_cfr_hip.unblocked_mass_triton(torch.zeros(2, 1326))

@@ -1,0 +1,134 @@
+"""GPU parity of the river showdown evaluator against the oracle (cumsum restatement and
+brute force) on the boards the reference's tests use and on seeded random boards."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cards as OC
+from oracle import showdown as OS
+from tests.helpers import H, C, random_boards, random_ranges
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 2e-6
+
+
+@pytest.fixture(scope="module")
+def K():
+    from poker2_amd import rules_hip
+    assert rules_hip.triton_is_available(), "libp2hip.so / GPU missing"
+    return rules_hip
+
+
+def run_hip(K, boards, beliefs, potential, scale, triton_order=True):
+    tables = K.build_showdown_tables(torch.from_numpy(boards).cuda(), triton_order=triton_order)
+    out = K.showdown_value_both(torch.from_numpy(beliefs).cuda(), tables,
+                                torch.from_numpy(potential).cuda(), torch.from_numpy(scale).cuda())
+    return out.cpu().numpy()
+
+
+def oracle_both(boards, beliefs, potential, scale):
+    allowed, _ = OC.allowed_hands_for_boards(boards)
+    hrd = OS.init_hand_rank_data(boards, allowed)
+    return OS.showdown_value_both(beliefs, hrd, potential, scale)
+
+
+NAMED_BOARDS = np.array([
+    [C(12, 3), C(10, 1), C(7, 2), C(5, 0), C(2, 1)],    # Ac Qh 9d 7s 4h
+    [C(12, 2), C(11, 2), C(10, 2), C(9, 2), C(0, 0)],   # Ad Kd Qd Jd 2s
+    [C(12, 1), C(11, 1), C(10, 1), C(9, 1), C(8, 1)],   # Ah Kh Qh Jh Th (everything ties)
+    [C(12, 0), C(9, 1), C(5, 3), C(3, 0), C(0, 2)],     # As Jh 7c 5s 2d
+    [C(8, 3), C(8, 1), C(8, 0), C(5, 2), C(5, 1)],      # Tc Th Ts 7d 7h
+    [C(5, 2), C(4, 2), C(3, 2), C(2, 2), C(1, 2)],      # 7d 6d 5d 4d 3d
+    [C(12, 3), C(11, 2), C(10, 1), C(9, 0), C(7, 3)],   # Ac Kd Qh Js 9c
+], dtype=np.int64)
+
+
+@pytest.mark.parametrize("triton_order", [True, False])
+def test_named_boards_vs_oracle_and_bruteforce(K, triton_order):
+    rng = np.random.default_rng(42)
+    boards = NAMED_BOARDS
+    m = boards.shape[0]
+    bel = random_ranges(rng, boards)
+    pot = np.tile(np.array([[200.0, 200.0]], dtype=np.float32), (m, 1))
+    scale = np.full(m, 1000.0, dtype=np.float32)
+    out = run_hip(K, boards, bel, pot, scale, triton_order)
+    exp = oracle_both(boards, bel, pot, scale)
+    np.testing.assert_allclose(out, exp, rtol=RTOL, atol=ATOL)
+    for i in range(m):
+        for hero in (0, 1):
+            bf = OS.showdown_value_bruteforce(boards[i], bel[i, 1 - hero], 0.2)
+            np.testing.assert_allclose(out[i, hero], bf, rtol=1e-4, atol=3e-6)
+    assert np.abs(out[2]).max() == 0.0  # royal flush on board: all ties
+
+
+def test_uniform_and_delta_ranges(K):
+    boards = NAMED_BOARDS[[0, 1]]
+    allowed, prob = OC.allowed_hands_for_boards(boards)
+    bel = np.stack([prob, prob], axis=1).astype(np.float32)
+    pot = np.array([[150.0, 250.0], [90.0, 90.0]], dtype=np.float32)
+    scale = np.array([1000.0, 450.0], dtype=np.float32)
+    out = run_hip(K, boards, bel, pot, scale)
+    np.testing.assert_allclose(out, oracle_both(boards, bel, pot, scale), rtol=RTOL, atol=ATOL)
+    assert np.all(out[:, 0][~allowed] == 0) and np.all(out[:, 1][~allowed] == 0)
+    assert np.abs(out[0, 0]).max() <= 0.15 + 1e-6 and np.abs(out[0, 1]).max() <= 0.25 + 1e-6
+    # villain holds one known hand (T9 of the board's suit = straight flush on board 1)
+    hero = OC.combo_index(C(8, 2), C(7, 2))
+    bel2 = bel.copy()
+    bel2[1, 1] = 0.0
+    bel2[1, 1, hero] = 1.0
+    out2 = run_hip(K, boards, bel2, pot, scale)
+    ok = allowed[1] & OC.mask_conflicting([C(8, 2), C(7, 2)])
+    np.testing.assert_allclose(out2[1, 0][ok], -90.0 / 450.0, rtol=1e-6)
+    assert np.all(out2[1, 0][~ok] == 0)
+    np.testing.assert_allclose(out2, oracle_both(boards, bel2, pot, scale), rtol=RTOL, atol=ATOL)
+
+
+def test_config2_shape_properties(K):
+    """B=4096 boards, Dirichlet(0.5) ranges, pot 1.0: compare a slice with the oracle and
+    check size-independent properties on all of it."""
+    rng = np.random.default_rng(42)
+    b = 4096
+    boards = random_boards(rng, b)
+    bel = random_ranges(rng, boards)
+    pot = np.ones((b, 2), dtype=np.float32)
+    scale = np.ones(b, dtype=np.float32)
+    out = run_hip(K, boards, bel, pot, scale)
+    sl = slice(0, 96)
+    np.testing.assert_allclose(out[sl], oracle_both(boards[sl], bel[sl], pot[sl], scale[sl]), rtol=RTOL, atol=ATOL)
+    allowed, _ = OC.allowed_hands_for_boards(boards)
+    assert np.isfinite(out).all() and np.abs(out).max() <= 1.0 + 1e-5
+    assert np.all(out[:, 0][~allowed] == 0) and np.all(out[:, 1][~allowed] == 0)
+    # zero-sum: sum_h0 b0[h0] * m1(h0) * EV0[h0] = - sum_h1 b1[h1] * m0(h1) * EV1[h1]
+    from oracle.unblocked import calculate_unblocked_mass
+    m1 = calculate_unblocked_mass(bel[:256, 1])
+    m0 = calculate_unblocked_mass(bel[:256, 0])
+    v0 = (bel[:256, 0] * m1 * out[:256, 0]).sum(-1)
+    v1 = (bel[:256, 1] * m0 * out[:256, 1]).sum(-1)
+    np.testing.assert_allclose(v0, -v1, atol=2e-5)
+    # scaling potential scales the result; table_row indirection gives the same answer
+    tables = K.build_showdown_tables(torch.from_numpy(boards).cuda())
+    idx = torch.arange(b - 1, -1, -1, device="cuda")
+    out_rev = K.showdown_value_both(torch.from_numpy(bel).cuda().flip(0).contiguous(), tables,
+                                    torch.from_numpy(pot * 3).cuda(), torch.from_numpy(scale).cuda(), table_row=idx)
+    np.testing.assert_allclose(out_rev.cpu().numpy()[::-1], out * 3, rtol=1e-6, atol=1e-7)
+
+
+def test_blocked_mass_in_villain_range(K):
+    """Mass on board-blocked combos is tolerated exactly as the reference tolerates it."""
+    rng = np.random.default_rng(9)
+    boards = random_boards(rng, 8)
+    bel = rng.random((8, 2, H)).astype(np.float32)
+    bel /= bel.sum(-1, keepdims=True)
+    pot = np.full((8, 2), 300.0, dtype=np.float32)
+    scale = np.full(8, 900.0, dtype=np.float32)
+    # same ranker on both sides: the two rankers order board-blocked combos differently
+    np.testing.assert_allclose(run_hip(K, boards, bel, pot, scale, triton_order=False),
+                               oracle_both(boards, bel, pot, scale), rtol=RTOL, atol=ATOL)
+
+
+def test_empty(K):
+    tables = K.build_showdown_tables(torch.zeros(0, 5, dtype=torch.long, device="cuda"))
+    out = K.showdown_value_both(torch.zeros(0, 2, H, device="cuda"), tables, torch.zeros(0, 2, device="cuda"),
+                                torch.zeros(0, device="cuda"))
+    assert out.shape == (0, 2, H)
