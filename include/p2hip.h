@@ -171,6 +171,55 @@ int p2hip_deep_beliefs(float* out, const float* root_beliefs, const float* reach
 int p2hip_sample_snapshot(const float* policy_probs, float* policy_probs_sample, const int64_t* t_sample,
                           const int64_t* t_now, int64_t total, void* stream);
 
+/* ---- one kernel = one CFR iteration ------------------------------------------------- */
+
+/* Device pointers of one subgame batch.  Tree arrays and state tensors are the evaluator's
+ * own (row-major over all nodes of all roots); the rest is derived once per subgame:
+ *   node_flags [total] bytes: bit0 = river showdown row, bit1 = terminal row
+ *   root_node_offsets [roots+1], root_nodes [total]: rows of each root's subtree, ascending
+ *   tables [roots, p2hip_showdown_table_bytes()] (NULL when no row is a showdown)
+ *   potential [total,2] float, scale [total] float: showdown pay-off factors per row
+ *   scratch [total,H] float workspace
+ *   fscal[8]: t^alpha, t^beta, t^alpha+1, t^beta+1, mix_old, mix_new, mix_old+mix_new, 1/(mix_old+mix_new)
+ *   iscal[6]: t, apply_dcfr, cfr_plus, average_policy_is_copied, enforce_zero_sum, update_average_values */
+typedef struct P2HipIterArgs {
+  const int64_t* child_offsets;
+  const int64_t* child_count;
+  const int64_t* to_act;
+  const uint8_t* node_flags;
+  const int64_t* root_node_offsets;
+  const int64_t* root_nodes;
+  const int64_t* t_sample;
+  const uint8_t* allowed;
+  const float* allowed_prob;
+  const uint8_t* tables;
+  const float* potential;
+  const float* scale;
+  float* policy;
+  float* policy_avg;
+  float* policy_sample;
+  float* cum;
+  float* wsum;
+  float* beliefs;
+  float* beliefs_avg;
+  float* reach;
+  float* reach_avg;
+  float* latest;
+  float* values_avg;
+  float* scratch;
+  const float* fscal;
+  const int64_t* iscal;
+} P2HipIterArgs;
+
+/* One workgroup per root runs the whole iteration of FusedSparseCFREvaluator.cfr_iteration
+ * (search/fused_sparse_cfr_evaluator.py:478-533; base search/cfr_evaluator.py:1330-1381) with
+ * cfr_avg = False: sample snapshot, instantaneous regrets, DCFR update, regret matching, reach,
+ * beliefs, average policy, reach_avg, beliefs_avg (phases bit 0); showdown leaf values, value
+ * backup, average values (phases bit 1).  host_args is a HOST pointer to a struct of device
+ * pointers; max_children = largest child count in the tree (<= 8). */
+int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max_children, int phases,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,516 @@
+// One kernel = one whole CFR iteration.  One workgroup owns one root's subtree and
+// walks it three times:
+//   sweep 1 (families independent): opponent unblocked mass at the parent, instantaneous
+//            regrets, DCFR discount + accumulate, regret matching -> policy_probs
+//   sweep 2 (top-down): reach, beliefs, average-policy mix + renormalise, reach_avg,
+//            beliefs_avg
+//   sweep 3 (bottom-up): showdown leaves, opponent-conditioned policy, value backup,
+//            average values
+// which is the order of FusedSparseCFREvaluator.cfr_iteration
+// (src/p2/search/fused_sparse_cfr_evaluator.py:478-533) with every per-op launch of
+// src/p2/search/fused_cfr_triton.py folded in.  `phases` lets the host split the
+// iteration where the leaf network has to run (after sweep 2).
+//
+// A "family" is a parent and its contiguous child rows.  Every thread owns the same
+// three float2 pairs (six hands) of every 1326-vector for the whole kernel, so all
+// per-hand work is register-to-register; only sums over hands go through LDS.
+#include "common.h"
+#include "unblocked.hip"
+#include "showdown.hip"
+#include "../../include/p2hip.h"
+
+namespace p2 {
+
+constexpr int IT_BLOCK = 256;
+constexpr int IT_WAVES = IT_BLOCK / 64;
+constexpr int IT_PPT = 3;  // pairs per thread: 3 * 256 = 768 >= 663
+static_assert(IT_BLOCK == UB_BLOCK && IT_BLOCK == SD_BLOCK, "shared helpers assume one block size");
+
+constexpr uint8_t NODE_SHOWDOWN = 1;  // river showdown leaf: value from the showdown evaluator
+constexpr uint8_t NODE_DONE = 2;      // terminal node: excluded from the zero-sum shift
+
+struct IterArgs {
+  // tree (row-major arrays over all nodes of all roots, as the evaluator keeps them)
+  const int64_t* child_offsets;
+  const int64_t* child_count;
+  const int64_t* to_act;
+  const uint8_t* node_flags;
+  const int64_t* root_node_offsets;  // [roots+1] into root_nodes
+  const int64_t* root_nodes;         // rows of each root's subtree, ascending (= top-down)
+  const int64_t* t_sample;           // [total]
+  const uint8_t* allowed;            // [total,H] bytes
+  const float* allowed_prob;         // [total,H]
+  const uint8_t* tables;             // [roots, SD_TABLE_BYTES] board strength tables (may be null)
+  const float* potential;            // [total,2] chips won by player p at a showdown row
+  const float* scale;                // [total]
+  // state
+  float* policy;
+  float* policy_avg;
+  float* policy_sample;
+  float* cum;
+  float* wsum;
+  float* beliefs;
+  float* beliefs_avg;
+  float* reach;
+  float* reach_avg;
+  float* latest;
+  float* values_avg;
+  float* scratch;                    // [total,H] workspace
+  // iteration-dependent scalars in device memory
+  const float* fscal;    // t_alpha_num, t_beta_num, t_alpha_den, t_beta_den, mix_old, mix_new, mix_total, mix_inv_total
+  const int64_t* iscal;  // t, apply_dcfr, cfr_plus, avg_policy_copy, enforce_zero_sum, update_avg_values
+  int phases;            // bit 0: sweeps 1+2, bit 1: sweep 3
+};
+
+struct IterLds {
+  __align__(8) float vec[P2_H + 2];
+  __align__(8) float vec2[P2_H + 2];
+  double cs[P2_CARDS];
+  double S;
+  float red[IT_WAVES][4];
+  ShowdownLds sd;
+};
+
+#define IT_FOR(j) _Pragma("unroll") for (int j = 0; j < IT_PPT; ++j)
+
+struct Lane {
+  int idx[IT_PPT];      // pair index
+  bool ok[IT_PPT];
+  uint8_t a[IT_PPT][2], b[IT_PPT][2];  // cards of the two hands of each pair
+};
+
+__device__ __forceinline__ void ld(float2 (&dst)[IT_PPT], const float* base, int64_t row, const Lane& ln) {
+  const float2* s = p2_row2(base, row);
+  IT_FOR(j) dst[j] = ln.ok[j] ? s[ln.idx[j]] : make_float2(0.f, 0.f);
+}
+__device__ __forceinline__ void st(float* base, int64_t row, const float2 (&src)[IT_PPT], const Lane& ln) {
+  float2* d = p2_row2(base, row);
+  IT_FOR(j) if (ln.ok[j]) d[ln.idx[j]] = src[j];
+}
+__device__ __forceinline__ void to_lds(float* vec, const float2 (&src)[IT_PPT], const Lane& ln) {
+  float2* d = reinterpret_cast<float2*>(vec);
+  IT_FOR(j) if (ln.ok[j]) d[ln.idx[j]] = src[j];
+}
+
+// unblocked mass of the vector whose card sums are in (cs, S) for this lane's hands
+__device__ __forceinline__ void unblocked_regs(float2 (&out)[IT_PPT], const float2 (&t)[IT_PPT], const double* cs,
+                                               double S, const Lane& ln) {
+  IT_FOR(j) {
+    const double x = S - cs[ln.a[j][0]] - cs[ln.b[j][0]] + (double)t[j].x;
+    const double y = S - cs[ln.a[j][1]] - cs[ln.b[j][1]] + (double)t[j].y;
+    out[j] = make_float2(fmaxf((float)x, 0.f), fmaxf((float)y, 0.f));
+  }
+}
+
+// Sums of up to four per-thread partials over the block; results to all threads.
+__device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[4]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) v[q] = p2_wave_sum(v[q]);
+  __syncthreads();
+  if (lane == 0) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) red[wave][q] = v[q];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < IT_WAVES; ++w) s += red[w][q];
+    v[q] = s;
+  }
+}
+
+__device__ __forceinline__ float2 mul2(float2 a, float2 b) { return make_float2(a.x * b.x, a.y * b.y); }
+
+template <int MAXC>
+__global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
+  __shared__ IterLds L;
+  const int64_t r = blockIdx.x;
+  const int64_t n0 = A.root_node_offsets[r], n1 = A.root_node_offsets[r + 1];
+
+  Lane ln;
+  IT_FOR(j) {
+    ln.idx[j] = threadIdx.x + j * IT_BLOCK;
+    ln.ok[j] = ln.idx[j] < P2_HPAIRS;
+    const int h = ln.ok[j] ? 2 * ln.idx[j] : 0;
+    ln.a[j][0] = p2_combo.a[h];
+    ln.b[j][0] = p2_combo.b[h];
+    ln.a[j][1] = p2_combo.a[h + 1];
+    ln.b[j][1] = p2_combo.b[h + 1];
+  }
+
+  const float f_an = A.fscal[0], f_bn = A.fscal[1], f_ad = A.fscal[2], f_bd = A.fscal[3];
+  const float mix_old = A.fscal[4], mix_new = A.fscal[5], mix_total = A.fscal[6], mix_inv = A.fscal[7];
+  const int64_t t_now = A.iscal[0];
+  const bool apply_dcfr = A.iscal[1] != 0, cfr_plus = A.iscal[2] != 0, avg_copy = A.iscal[3] != 0;
+  const bool enforce_zs = A.iscal[4] != 0, update_avg = A.iscal[5] != 0;
+
+  if (A.phases & 1) {
+    // ---------------- sweep 1: regrets -> DCFR -> regret matching ----------------
+    const bool take_sample = A.t_sample[r] == t_now;
+    for (int64_t q = n0; q < n1; ++q) {
+      const int64_t p = A.root_nodes[q];
+      const int cnt = (int)A.child_count[p];
+      if (cnt == 0) continue;
+      const int actor = (int)A.to_act[p];
+      const int64_t first = A.child_offsets[p];
+
+      float2 bo[IT_PPT], w[IT_PPT], ex[IT_PPT], tmp[IT_PPT];
+      ld(bo, A.beliefs, p * 2 + (1 - actor), ln);
+      to_lds(L.vec, bo, ln);
+      ld(ex, A.latest, p * 2 + actor, ln);
+      ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
+      st(A.scratch, p, tmp, ln);
+      __syncthreads();
+      card_sums(L.vec, L.cs, &L.S);
+      unblocked_regs(w, bo, L.cs, L.S, ln);
+
+      float2 pos[MAXC][IT_PPT];
+      float2 sum[IT_PPT];
+      IT_FOR(j) sum[j] = make_float2(0.f, 0.f);
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          const int64_t c = first + k;
+          float2 ach[IT_PPT], cu[IT_PPT], ws[IT_PPT];
+          ld(ach, A.latest, c * 2 + actor, ln);
+          ld(cu, A.cum, c, ln);
+          ld(ws, A.wsum, c, ln);
+          if (take_sample) {
+            ld(tmp, A.policy, c, ln);
+            st(A.policy_sample, c, tmp, ln);
+          }
+          IT_FOR(j) {
+            float cc[2] = {cu[j].x, cu[j].y}, ww[2] = {ws[j].x, ws[j].y};
+            const float rg[2] = {w[j].x * (ach[j].x - ex[j].x), w[j].y * (ach[j].y - ex[j].y)};
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              if (apply_dcfr) {
+                const bool positive = cc[e] > 0.f;
+                const float num = positive ? f_an : f_bn, den = positive ? f_ad : f_bd;
+                cc[e] = cc[e] * num;
+                cc[e] = cc[e] / den;
+                ww[e] = ww[e] * num;
+                ww[e] = ww[e] / den;
+              }
+              ww[e] = ww[e] + 1.0f;
+              cc[e] = cc[e] + rg[e];
+              if (cfr_plus) cc[e] = fmaxf(cc[e], 0.f);
+            }
+            cu[j] = make_float2(cc[0], cc[1]);
+            ws[j] = make_float2(ww[0], ww[1]);
+            pos[k][j] = make_float2(fmaxf(cc[0], 0.f), fmaxf(cc[1], 0.f));
+            sum[j].x += pos[k][j].x;
+            sum[j].y += pos[k][j].y;
+          }
+          st(A.cum, c, cu, ln);
+          st(A.wsum, c, ws, ln);
+        }
+      }
+      const float uniform = 1.0f / (float)cnt;
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          float2 pol[IT_PPT];
+          IT_FOR(j) {
+            pol[j].x = sum[j].x > 1e-8f ? pos[k][j].x / fmaxf(sum[j].x, 1e-8f) : uniform;
+            pol[j].y = sum[j].y > 1e-8f ? pos[k][j].y / fmaxf(sum[j].y, 1e-8f) : uniform;
+          }
+          st(A.policy, first + k, pol, ln);
+        }
+      }
+      __syncthreads();  // L.vec / L.cs are reused by the next family
+    }
+    // sweep 2 re-reads policy / reach rows that the same lane wrote: no cross-lane hand-off
+
+    // ---------------- sweep 2: reach, beliefs, average policy ----------------
+    float2 rb[2][IT_PPT], rba[2][IT_PPT], ap[IT_PPT];
+    uchar2 am[IT_PPT];
+    ld(rb[0], A.beliefs, r * 2, ln);
+    ld(rb[1], A.beliefs, r * 2 + 1, ln);
+    ld(rba[0], A.beliefs_avg, r * 2, ln);
+    ld(rba[1], A.beliefs_avg, r * 2 + 1, ln);
+    ld(ap, A.allowed_prob, r, ln);
+    {
+      const uchar2* m2 = reinterpret_cast<const uchar2*>(A.allowed + r * P2_H);
+      IT_FOR(j) am[j] = ln.ok[j] ? m2[ln.idx[j]] : make_uchar2(0, 0);
+    }
+    for (int64_t q = n0; q < n1; ++q) {
+      const int64_t p = A.root_nodes[q];
+      const int cnt = (int)A.child_count[p];
+      if (cnt == 0) continue;
+      const int actor = (int)A.to_act[p];
+      const int64_t first = A.child_offsets[p];
+      float2 rn[2][IT_PPT], ran[2][IT_PPT], ra_old[IT_PPT];
+      ld(rn[0], A.reach, p * 2, ln);
+      ld(rn[1], A.reach, p * 2 + 1, ln);
+      ld(ran[0], A.reach_avg, p * 2, ln);
+      ld(ran[1], A.reach_avg, p * 2 + 1, ln);
+      ld(ra_old, A.scratch, p, ln);
+
+      float2 rn_act[IT_PPT];  // new reach of the acting player at the parent
+      IT_FOR(j) rn_act[j] = actor == 0 ? rn[0][j] : rn[1][j];
+      float2 cur[MAXC][IT_PPT], pav[MAXC][IT_PPT];
+      float2 psum[IT_PPT];
+      IT_FOR(j) psum[j] = make_float2(0.f, 0.f);
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          ld(cur[k], A.policy, first + k, ln);
+          if (avg_copy) {
+            IT_FOR(j) pav[k][j] = cur[k][j];
+          } else {
+            float2 avg[IT_PPT];
+            ld(avg, A.policy_avg, first + k, ln);
+            IT_FOR(j) {
+              const float rr[2] = {rn_act[j].x, rn_act[j].y}, rao[2] = {ra_old[j].x, ra_old[j].y};
+              const float cc[2] = {cur[k][j].x, cur[k][j].y}, aa[2] = {avg[j].x, avg[j].y};
+              float o[2];
+#pragma unroll
+              for (int e = 0; e < 2; ++e) {
+                const float reach_a = rao[e] * mix_old, reach_n = rr[e] * mix_new;
+                const float num = reach_a * aa[e] + reach_n * cc[e];
+                const float den = reach_a + reach_n;
+                const float unweighted = (mix_old * aa[e] + mix_new * cc[e]) / mix_total;
+                o[e] = den > 1e-5f ? num / den : unweighted;
+              }
+              pav[k][j] = make_float2(o[0], o[1]);
+              psum[j].x += o[0];
+              psum[j].y += o[1];
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          if (!avg_copy) {
+            IT_FOR(j) {
+              if (psum[j].x > 1e-5f) pav[k][j].x = pav[k][j].x / fmaxf(psum[j].x, 1e-5f);
+              if (psum[j].y > 1e-5f) pav[k][j].y = pav[k][j].y / fmaxf(psum[j].y, 1e-5f);
+            }
+          }
+          st(A.policy_avg, first + k, pav[k], ln);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          const int64_t c = first + k;
+          float2 rc[2][IT_PPT], rca[2][IT_PPT], vb[2][IT_PPT], vba[2][IT_PPT];
+          float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int pl = 0; pl < 2; ++pl) {
+            IT_FOR(j) {
+              float2 x = rn[pl][j], y = ran[pl][j];
+              if (pl == actor) { x = mul2(x, cur[k][j]); y = mul2(y, pav[k][j]); }
+              x = make_float2(am[j].x ? x.x : 0.f, am[j].y ? x.y : 0.f);
+              y = make_float2(am[j].x ? y.x : 0.f, am[j].y ? y.y : 0.f);
+              rc[pl][j] = x;
+              rca[pl][j] = y;
+              vb[pl][j] = mul2(rb[pl][j], x);
+              vba[pl][j] = mul2(rba[pl][j], y);
+              s4[pl] += vb[pl][j].x + vb[pl][j].y;
+              s4[2 + pl] += vba[pl][j].x + vba[pl][j].y;
+            }
+            st(A.reach, c * 2 + pl, rc[pl], ln);
+            st(A.reach_avg, c * 2 + pl, rca[pl], ln);
+          }
+          block_sum4(s4, L.red);
+#pragma unroll
+          for (int pl = 0; pl < 2; ++pl) {
+            float2 o[IT_PPT], oa[IT_PPT];
+            IT_FOR(j) {
+              o[j] = s4[pl] > 1e-5f ? make_float2(vb[pl][j].x / s4[pl], vb[pl][j].y / s4[pl]) : ap[j];
+              oa[j] = s4[2 + pl] > 1e-5f ? make_float2(vba[pl][j].x / s4[2 + pl], vba[pl][j].y / s4[2 + pl]) : ap[j];
+            }
+            st(A.beliefs, c * 2 + pl, o, ln);
+            st(A.beliefs_avg, c * 2 + pl, oa, ln);
+          }
+        }
+      }
+    }
+  }
+
+  if (A.phases & 2) {
+    // ---------------- sweep 3: leaf values, backup, average values ----------------
+    const uint8_t* tab = A.tables ? A.tables + r * SD_TABLE_BYTES : nullptr;
+    for (int64_t q = n1 - 1; q >= n0; --q) {
+      const int64_t p = A.root_nodes[q];
+      const int cnt = (int)A.child_count[p];
+      if (cnt == 0) continue;
+      const int actor = (int)A.to_act[p];
+      const int64_t first = A.child_offsets[p];
+
+      float2 ab[IT_PPT], dn[IT_PPT];
+      ld(ab, A.beliefs, p * 2 + actor, ln);
+      to_lds(L.vec, ab, ln);
+      __syncthreads();
+      card_sums(L.vec, L.cs, &L.S);
+      unblocked_regs(dn, ab, L.cs, L.S, ln);
+      __syncthreads();  // L.cs is rewritten for every child below
+
+      float2 vp[2][IT_PPT];
+      IT_FOR(j) vp[0][j] = vp[1][j] = make_float2(0.f, 0.f);
+      for (int k = 0; k < cnt; ++k) {
+        const int64_t c = first + k;
+        float2 pol[IT_PPT], mg[IT_PPT], nm[IT_PPT], occ[IT_PPT];
+        ld(pol, A.policy, c, ln);
+        IT_FOR(j) mg[j] = mul2(ab[j], pol[j]);
+        to_lds(L.vec2, mg, ln);
+        __syncthreads();
+        card_sums(L.vec2, L.cs, &L.S);
+        unblocked_regs(nm, mg, L.cs, L.S, ln);
+        IT_FOR(j) {
+          occ[j].x = dn[j].x > 1e-5f ? nm[j].x / dn[j].x : 0.f;
+          occ[j].y = dn[j].y > 1e-5f ? nm[j].y / dn[j].y : 0.f;
+        }
+        const uint8_t flags = A.node_flags[c];
+        float2 v[2][IT_PPT];
+        if ((flags & NODE_SHOWDOWN) && tab) {
+          showdown_scan(A.beliefs + c * 2 * P2_H, tab, L.sd);
+          const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
+          const uint16_t* lr = reinterpret_cast<const uint16_t*>(tab + SD_OFF_LR);
+          const uchar4* cidx = reinterpret_cast<const uchar4*>(tab + SD_OFF_CIDX);
+          const float sc = A.scale[c], pot0 = A.potential[2 * c], pot1 = A.potential[2 * c + 1];
+          for (int s = threadIdx.x; s < P2_H; s += IT_BLOCK) {
+            const unsigned pk = perm[s];
+            const int h = pk & 0x7FFF;
+            const float keep = (pk & 0x8000u) ? 0.f : 1.f;
+            const int Lp = lr[2 * s], Rp = lr[2 * s + 1];
+            const uchar4 ci = cidx[s];
+            const float e0 = showdown_ev_at(L.sd, 0, s, h, Lp, Rp, ci) * keep;
+            const float e1 = showdown_ev_at(L.sd, 1, s, h, Lp, Rp, ci) * keep;
+            L.vec[h] = e0 * pot0 / sc;
+            L.vec2[h] = e1 * pot1 / sc;
+          }
+          __syncthreads();
+          {
+            const float2* e0 = reinterpret_cast<const float2*>(L.vec);
+            const float2* e1 = reinterpret_cast<const float2*>(L.vec2);
+            IT_FOR(j) {
+              v[0][j] = ln.ok[j] ? e0[ln.idx[j]] : make_float2(0.f, 0.f);
+              v[1][j] = ln.ok[j] ? e1[ln.idx[j]] : make_float2(0.f, 0.f);
+            }
+          }
+          st(A.latest, c * 2, v[0], ln);
+          st(A.latest, c * 2 + 1, v[1], ln);
+        } else {
+          ld(v[0], A.latest, c * 2, ln);
+          ld(v[1], A.latest, c * 2 + 1, ln);
+        }
+        __syncthreads();  // L.vec / L.vec2 / L.cs free for the next child
+        IT_FOR(j) {
+          const float2 wa = pol[j], wo = occ[j];
+          if (actor == 0) {
+            vp[0][j].x += v[0][j].x * wa.x; vp[0][j].y += v[0][j].y * wa.y;
+            vp[1][j].x += v[1][j].x * wo.x; vp[1][j].y += v[1][j].y * wo.y;
+          } else {
+            vp[1][j].x += v[1][j].x * wa.x; vp[1][j].y += v[1][j].y * wa.y;
+            vp[0][j].x += v[0][j].x * wo.x; vp[0][j].y += v[0][j].y * wo.y;
+          }
+        }
+        if (update_avg) {
+          // values_avg[c] <- (avg*old + latest*new) * inv_total, then the optional zero-sum shift
+          float2 nv[2][IT_PPT];
+          float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int pl = 0; pl < 2; ++pl) {
+            float2 av[IT_PPT];
+            ld(av, A.values_avg, c * 2 + pl, ln);
+            IT_FOR(j) nv[pl][j] = make_float2((av[j].x * mix_old + v[pl][j].x * mix_new) * mix_inv,
+                                              (av[j].y * mix_old + v[pl][j].y * mix_new) * mix_inv);
+            if (enforce_zs) {
+              float2 ba[IT_PPT];
+              ld(ba, A.beliefs_avg, c * 2 + pl, ln);
+              IT_FOR(j) s4[0] += nv[pl][j].x * ba[j].x + nv[pl][j].y * ba[j].y;
+            }
+          }
+          float shift = 0.f;
+          if (enforce_zs) {
+            block_sum4(s4, L.red);
+            shift = (flags & NODE_DONE) ? 0.f : 0.5f * s4[0];
+          }
+#pragma unroll
+          for (int pl = 0; pl < 2; ++pl) {
+            IT_FOR(j) nv[pl][j] = make_float2(nv[pl][j].x - shift, nv[pl][j].y - shift);
+            st(A.values_avg, c * 2 + pl, nv[pl], ln);
+          }
+        }
+      }
+      st(A.latest, p * 2, vp[0], ln);
+      st(A.latest, p * 2 + 1, vp[1], ln);
+      if (q == n0 && update_avg) {
+        // the root is nobody's child: update its average values here
+        float2 nv[2][IT_PPT];
+        float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl) {
+          float2 av[IT_PPT];
+          ld(av, A.values_avg, p * 2 + pl, ln);
+          IT_FOR(j) nv[pl][j] = make_float2((av[j].x * mix_old + vp[pl][j].x * mix_new) * mix_inv,
+                                            (av[j].y * mix_old + vp[pl][j].y * mix_new) * mix_inv);
+          if (enforce_zs) {
+            float2 ba[IT_PPT];
+            ld(ba, A.beliefs_avg, p * 2 + pl, ln);
+            IT_FOR(j) s4[0] += nv[pl][j].x * ba[j].x + nv[pl][j].y * ba[j].y;
+          }
+        }
+        float shift = 0.f;
+        if (enforce_zs) {
+          block_sum4(s4, L.red);
+          shift = (A.node_flags[p] & NODE_DONE) ? 0.f : 0.5f * s4[0];
+        }
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl) {
+          IT_FOR(j) nv[pl][j] = make_float2(nv[pl][j].x - shift, nv[pl][j].y - shift);
+          st(A.values_avg, p * 2 + pl, nv[pl], ln);
+        }
+      }
+    }
+  }
+}
+
+}  // namespace p2
+
+extern "C" {
+
+// P2HipIterArgs (include/p2hip.h) mirrors p2::IterArgs field by field.
+
+int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max_children, int phases,
+                        void* stream) {
+  if (!host_args || n_roots < 0 || max_children < 1 || max_children > 8 || (phases & ~3) || phases == 0)
+    return P2_EINVAL;
+  if (n_roots == 0) return 0;
+  const P2HipIterArgs& h = *host_args;
+  const void* required[] = {h.child_offsets, h.child_count, h.to_act, h.node_flags, h.root_node_offsets, h.root_nodes,
+                            h.t_sample, h.allowed, h.allowed_prob, h.potential, h.scale, h.policy, h.policy_avg,
+                            h.policy_sample, h.cum, h.wsum, h.beliefs, h.beliefs_avg, h.reach, h.reach_avg, h.latest,
+                            h.values_avg, h.scratch, h.fscal, h.iscal};
+  for (const void* p : required)
+    if (!p) return P2_EINVAL;
+  const void* rows[] = {h.allowed_prob, h.policy, h.policy_avg, h.policy_sample, h.cum, h.wsum, h.beliefs,
+                        h.beliefs_avg, h.reach, h.reach_avg, h.latest, h.values_avg, h.scratch, h.tables};
+  for (const void* p : rows)
+    if (!p2_aligned8(p)) return P2_EINVAL;
+  p2::IterArgs a;
+  a.child_offsets = h.child_offsets; a.child_count = h.child_count; a.to_act = h.to_act;
+  a.node_flags = h.node_flags; a.root_node_offsets = h.root_node_offsets; a.root_nodes = h.root_nodes;
+  a.t_sample = h.t_sample; a.allowed = h.allowed; a.allowed_prob = h.allowed_prob; a.tables = h.tables;
+  a.potential = h.potential; a.scale = h.scale; a.policy = h.policy; a.policy_avg = h.policy_avg;
+  a.policy_sample = h.policy_sample; a.cum = h.cum; a.wsum = h.wsum; a.beliefs = h.beliefs;
+  a.beliefs_avg = h.beliefs_avg; a.reach = h.reach; a.reach_avg = h.reach_avg; a.latest = h.latest;
+  a.values_avg = h.values_avg; a.scratch = h.scratch; a.fscal = h.fscal; a.iscal = h.iscal;
+  a.phases = phases;
+  const dim3 grid((unsigned)n_roots), block(p2::IT_BLOCK);
+  if (max_children <= 5)
+    hipLaunchKernelGGL((p2::cfr_iteration_kernel<5>), grid, block, 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((p2::cfr_iteration_kernel<8>), grid, block, 0, (hipStream_t)stream, a);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -7,6 +7,7 @@
 // device pointers so a captured launch sequence can be replayed for any t.
 // Built with -ffp-contract=off: a*b+c stays two roundings, like the eager torch
 // ops these replace.
+#pragma once
 #include "common.h"
 
 namespace p2 {

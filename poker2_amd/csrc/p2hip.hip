@@ -5,6 +5,7 @@
 #include "unblocked.hip"
 #include "showdown.hip"
 #include "cfr_ops.hip"
+#include "cfr_iter.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

@@ -13,6 +13,7 @@
 //     tie = P[R]-P[L] - (Pc[a][iRa]-Pc[a][iLa]) - (Pc[b][iRb]-Pc[b][iLb]) + v[k]
 //     den = max(1 - Pc[a][51] - Pc[b][51] + v[k], 1e-8)
 // where iLa = how many of card a's combos lie strictly below the tie group, etc.
+#pragma once
 #include "common.h"
 #include "ranker.hip"
 

@@ -8,6 +8,7 @@
 // :1008-1026, :1408-1496.  One workgroup per row: the row is staged in LDS,
 // each wave reduces 13 cards (lane j = j-th partner card), sums run in float64
 // so the result rounds like the float64 product does.
+#pragma once
 #include "common.h"
 
 namespace p2 {

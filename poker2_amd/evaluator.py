@@ -1,0 +1,623 @@
+"""``HipSparseCFREvaluator`` -- the search evaluator of the reference with every
+per-iteration step on hand-written HIP kernels.
+
+Mirrors the method set that ``FusedSparseCFREvaluator`` overrides
+(src/p2/search/fused_sparse_cfr_evaluator.py:144-550) on top of the state layout of
+``SparseCFREvaluator`` (src/p2/search/sparse_cfr_evaluator.py:142-306) and the iteration
+logic of ``CFREvaluator`` (src/p2/search/cfr_evaluator.py:285-303, :770-886, :1294-1381,
+:1497-1528).  State tensors keep the reference's names, shapes and dtypes.
+
+Two execution modes share the same state:
+  * ``fused_iteration=True`` (default): ``cfr_iteration`` is ONE kernel launch
+    (``p2hip_cfr_iteration``), or two around the leaf network when the tree has
+    non-terminal leaves and a leaf model is attached;
+  * ``fused_iteration=False``: one launch per operation through the functions of
+    ``fused_cfr_hip`` -- the call sequence of the reference's fused evaluator.
+
+Leaf model protocol (the value network itself stays ordinary PyTorch): ``model`` is
+``None`` (zero leaf values and a uniform initial policy, i.e. the reference tests' zero
+``MockModel``) or an object with
+    enforce_zero_sum: bool
+    leaf_values(beliefs[K,2,1326], node_rows[K], evaluator) -> [K,2,1326]
+    policy_logits(beliefs[T,2,1326], node_rows[K], evaluator) -> [K,1326,A]   (optional)
+
+Out of scope here (host-side, post-search): leaf sampling, training-data assembly,
+exploitability statistics, warm start.
+"""
+from __future__ import annotations
+
+import ctypes
+from types import SimpleNamespace
+
+import numpy as np
+import torch
+
+from . import _lib
+from . import fused_cfr_hip as F
+from . import rules_hip
+from .card_utils import NUM_HANDS, combo_to_onehot_tensor
+from .fused_cfr_hip import CFRType
+from .tree import RootStates, SparseTree, build_sparse_tree
+
+STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
+               "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",
+               "latest_values", "values_avg")
+
+_NODE_SHOWDOWN, _NODE_DONE = 1, 2
+
+
+class _IterArgs(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in (
+        "child_offsets", "child_count", "to_act", "node_flags", "root_node_offsets", "root_nodes", "t_sample",
+        "allowed", "allowed_prob", "tables", "potential", "scale", "policy", "policy_avg", "policy_sample", "cum",
+        "wsum", "beliefs", "beliefs_avg", "reach", "reach_avg", "latest", "values_avg", "scratch", "fscal", "iscal")]
+
+
+def _cfr_type_name(x) -> str:
+    return getattr(x, "name", str(x))
+
+
+class HipSparseCFREvaluator:
+    def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
+                 compile_model: bool = True, fused_iteration: bool = True,
+                 max_raises: int | None = None) -> None:
+        self.model = model
+        self.device = torch.device(device)
+        self.cfg = cfg
+        if self.device.type != "cuda":
+            raise ValueError("HipSparseCFREvaluator requires a GPU device.")
+        if not F.triton_is_available():
+            raise RuntimeError("libp2hip.so or a GPU is not available; HipSparseCFREvaluator has no other backend.")
+        s = cfg.search
+        self.float_dtype = torch.float32
+        self.num_players = 2
+        self.bet_bins = list(cfg.env.bet_bins)
+        self.num_actions = len(self.bet_bins) + 3
+        if self.num_actions > 8:
+            raise ValueError("at most 8 action bins are supported")
+        self.max_depth = s.depth
+        self.cfr_iterations = s.iterations
+        self.warm_start_iterations = max(0, min(s.warm_start_iterations, max(1, self.cfr_iterations - 1)))
+        if self.warm_start_iterations > 0:
+            raise NotImplementedError("warm start is not part of this build; set warm_start_iterations=0")
+        self.cfr_type = CFRType[_cfr_type_name(s.cfr_type)]
+        self.cfr_avg = bool(s.cfr_avg)
+        self.cfr_plus = bool(s.cfr_plus)
+        self.dcfr_alpha = self.dcfr_alpha_initial = s.dcfr_alpha
+        self.dcfr_beta = self.dcfr_beta_initial = s.dcfr_beta
+        self.dcfr_gamma = self.dcfr_gamma_initial = s.dcfr_gamma
+        self.dcfr_alpha_final = s.dcfr_alpha_final
+        self.dcfr_beta_final = s.dcfr_beta_final
+        self.dcfr_gamma_final = s.dcfr_gamma_final
+        self.dcfr_delay = s.dcfr_plus_delay
+        self.use_final_policy_values = bool(s.value_targets_from_final_policy)
+        self.generator = generator
+        self.fused_iteration = bool(fused_iteration)
+        self.max_raises = max_raises
+        self.stats: dict = {}
+        self.root_nodes = cfg.num_envs
+        self.total_nodes = 0
+        self.tree_depth = 0
+        self.depth_offsets = [0]
+        self.last_model_values = None
+        self._t_scalars = F.TScalars(self.device, dtype=self.float_dtype)
+        self._skip_t_scalars_update = False
+        self._skip_record_stats = True
+        self._fused_positive_regrets_buf = None
+        self._fscal = torch.zeros(8, dtype=torch.float32, device=self.device)
+        self._iscal = torch.zeros(8, dtype=torch.int64, device=self.device)
+        self._fscal_host = torch.zeros(8, dtype=torch.float32).pin_memory()
+        self._iscal_host = torch.zeros(8, dtype=torch.int64).pin_memory()
+        self._iter_args = None
+
+    @property
+    def enforce_zero_sum(self) -> bool:
+        return bool(getattr(self.model, "enforce_zero_sum", False)) if self.model is not None else False
+
+    # ------------------------------------------------------------------ subgame setup
+    def _t(self, x: np.ndarray, dtype=None) -> torch.Tensor:
+        t = torch.from_numpy(np.ascontiguousarray(x))
+        if dtype is not None:
+            t = t.to(dtype)
+        return t.to(self.device)
+
+    def _construct_subgame(self, src_env, src_indices) -> None:
+        """Build the sparse tree and allocate the state (sparse_cfr_evaluator.py:142-306)."""
+        if isinstance(src_env, RootStates):
+            idx = src_indices.cpu().numpy() if hasattr(src_indices, "cpu") else np.asarray(src_indices)
+            roots = src_env.select(idx)
+        else:
+            roots = RootStates.from_env(src_env, src_indices)
+        tree = build_sparse_tree(roots, self.bet_bins, self.max_depth, max_raises=self.max_raises)
+        self.tree: SparseTree = tree
+        dev = self.device
+        self.depth_offsets = list(tree.depth_offsets)
+        self.tree_depth = tree.tree_depth
+        self.total_nodes = tree.total
+        self.root_nodes = tree.n_roots
+        self.top_nodes = tree.top
+        T, N = tree.total, tree.n_roots
+        self.valid_mask = torch.ones(T, dtype=torch.bool, device=dev)
+        self.parent_index = self._t(tree.parent_index)
+        self.action_from_parent = self._t(tree.action_from_parent)
+        self.child_count = self._t(tree.child_count)
+        self.child_offsets = self._t(tree.child_offsets)
+        self.prev_actor = self._t(tree.prev_actor)
+        self.legal_mask = self._t(tree.legal_mask)
+        self.leaf_mask = self._t(tree.leaf_mask)
+        self.new_street_mask = self._t(tree.new_street_mask)
+        self.child_mask = self.legal_mask & (~self.leaf_mask)[:, None]
+        st = tree.state
+        self.env = SimpleNamespace(
+            N=T, to_act=self._t(st["to_act"]), done=self._t(st["done"]), street=self._t(st["street"]),
+            pot=self._t(st["pot"]), stacks=self._t(st["stacks"]), committed=self._t(st["committed"]),
+            starting_stacks=self._t(st["starting_stacks"]), scale=self._t(st["scale"]),
+            actions_this_round=self._t(st["actions_this_round"]), button=self._t(st["button"]),
+            board_indices=self._t(tree.board[tree.root_index]), bb=roots.bb)
+        self._root_index = self._t(tree.root_index)
+        model_mask = tree.leaf_mask & ~st["done"]
+        self.model_indices = self._t(np.nonzero(model_mask)[0].astype(np.int64))
+        self.showdown_indices = self._t(np.nonzero(tree.showdown_mask)[0].astype(np.int64))
+        self.showdown_actors = self.env.to_act[self.showdown_indices]
+        self.showdown_potential = self._t(tree.showdown_potential[tree.showdown_mask])
+        self._potential_all = self._t(tree.showdown_potential.astype(np.float32))
+
+        def z1():
+            return torch.zeros(T, NUM_HANDS, dtype=self.float_dtype, device=dev)
+
+        def z2():
+            return torch.zeros(T, 2, NUM_HANDS, dtype=self.float_dtype, device=dev)
+
+        self.policy_probs, self.policy_probs_avg, self.policy_probs_sample = z1(), z1(), z1()
+        self.cumulative_regrets, self.regret_weight_sums = z1(), z1()
+        self.uniform_policy = z1()
+        cc_dest = self.child_count[:tree.top].repeat_interleave(self.child_count[:tree.top])
+        self.uniform_policy[N:] = (1.0 / cc_dest)[:, None].expand(-1, NUM_HANDS)
+        self.beliefs, self.beliefs_avg = z2(), z2()
+        self.root_pre_chance_beliefs = torch.zeros(N, 2, NUM_HANDS, dtype=self.float_dtype, device=dev)
+        self.self_reach = z2()
+        self.self_reach[:N] = 1.0
+        self.self_reach_avg = self.self_reach.clone()
+        self.latest_values = z2()
+        folded = self._t(tree.fold_mask)
+        rew = self._t(tree.reward)
+        self.latest_values[folded, 0] = rew[folded][:, None]
+        self.latest_values[folded, 1] = -rew[folded][:, None]
+        self.values_avg = self.latest_values.clone()
+        self.last_model_values = None
+        self._scratch = z1()
+        flags = np.zeros(T, dtype=np.uint8)
+        flags[tree.showdown_mask] |= _NODE_SHOWDOWN
+        flags[st["done"]] |= _NODE_DONE
+        self._node_flags = self._t(flags)
+        order = np.argsort(tree.root_index, kind="stable").astype(np.int64)  # rows grouped by root, ascending
+        counts = np.bincount(tree.root_index, minlength=N)
+        self._root_nodes = self._t(order)
+        self._root_node_offsets = self._t(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64))
+        self._max_children = int(tree.child_count.max()) if T else 1
+        self._has_model_leaves = bool(model_mask.any())
+        self._iter_args = None
+
+    def initialize_subgame(self, src_env, src_indices, initial_beliefs: torch.Tensor | None = None) -> None:
+        """cfr_evaluator.py:770-828."""
+        self._construct_subgame(src_env, src_indices)
+        N = self.root_nodes
+        if initial_beliefs is None:
+            initial_beliefs = torch.full((N, 2, NUM_HANDS), 1.0 / NUM_HANDS, dtype=self.float_dtype, device=self.device)
+        else:
+            initial_beliefs = initial_beliefs.to(device=self.device, dtype=self.float_dtype)
+        self.beliefs[:N] = initial_beliefs
+        self.beliefs_avg[:N] = initial_beliefs
+        self.root_pre_chance_beliefs[:] = initial_beliefs
+        self.self_reach[:N] = 1.0
+        self.self_reach_avg[:N] = 1.0
+        board = self._t(self.tree.board)
+        onehot = combo_to_onehot_tensor(device=self.device).float()
+        board_mask = torch.zeros(N, 52, dtype=self.float_dtype, device=self.device)
+        valid = board >= 0
+        rows = torch.arange(N, device=self.device)[:, None].expand_as(board)
+        board_mask[rows[valid], board[valid]] = 1.0
+        root_allowed = (onehot @ board_mask.T).T < 0.5
+        root_prob = root_allowed.float()
+        root_prob /= root_prob.sum(dim=-1, keepdim=True).clamp(min=1.0)
+        self.allowed_hands = root_allowed[self._root_index].contiguous()
+        self.allowed_hands_prob = root_prob[self._root_index].contiguous()
+        self._init_hand_rank_data()
+        self.t_sample = torch.full((self.total_nodes,), -1, dtype=torch.long, device=self.device)
+        self.stats["evaluator_total_nodes"] = float(self.total_nodes)
+        self.stats["evaluator_root_nodes"] = float(self.root_nodes)
+        self.stats["evaluator_tree_depth"] = float(self.tree_depth)
+
+    def _init_hand_rank_data(self) -> None:
+        """Per-root strength tables for the showdown kernel (replaces the HandRankData of
+        cfr_evaluator.py:406-482; the card-id ranker is the one the reference's fused
+        evaluator installs, fused_sparse_cfr_evaluator.py:70-78)."""
+        if self.showdown_indices.numel() == 0:
+            self.hand_rank_data = None
+            return
+        board = self._t(self.tree.board)
+        self.hand_rank_data = rules_hip.build_showdown_tables(board, triton_order=True)
+        self._showdown_rows = self._root_index[self.showdown_indices].contiguous()
+        self._showdown_scale = self.env.scale[self.showdown_indices].contiguous()
+        self._showdown_potential_f = self.showdown_potential.to(self.float_dtype).contiguous()
+
+    def _showdown_value_both(self, beliefs: torch.Tensor) -> torch.Tensor:
+        """beliefs [M,2,H] of the showdown rows -> [M,2,H] (cfr_evaluator.py:484-601)."""
+        if self.showdown_indices.numel() == 0:
+            return torch.zeros(0, 2, NUM_HANDS, device=self.device, dtype=self.float_dtype)
+        return rules_hip.showdown_value_both(beliefs, self.hand_rank_data, self._showdown_potential_f,
+                                             self._showdown_scale, table_row=self._showdown_rows)
+
+    # ------------------------------------------------------------------ host-side scalars
+    def _get_mixing_weights(self, t: int):
+        """cfr_evaluator.py:285-303."""
+        if self.cfr_type == CFRType.standard:
+            return t, 1
+        if self.cfr_type == CFRType.linear:
+            return t, 2
+        if self.cfr_type == CFRType.discounted:
+            return t ** self.dcfr_gamma, (t + 1) ** self.dcfr_gamma
+        if t > self.dcfr_delay:
+            return t - self.dcfr_delay, 2
+        return 0, 1
+
+    def apply_schedules(self, t: int) -> None:
+        """cfr_evaluator.py:1294-1328."""
+        total = max(1, self.cfr_iterations - self.warm_start_iterations)
+        progress = max(0, t - self.warm_start_iterations)
+        x = min(1.0, max(0.0, progress / float(total)))
+
+        def lerp(a0, a1):
+            return a0 if a1 is None else a0 + (a1 - a0) * x
+
+        self.dcfr_alpha = lerp(self.dcfr_alpha_initial, self.dcfr_alpha_final)
+        self.dcfr_beta = lerp(self.dcfr_beta_initial, self.dcfr_beta_final)
+        self.dcfr_gamma = lerp(self.dcfr_gamma_initial, self.dcfr_gamma_final)
+
+    def _avg_policy_copies(self, t: int) -> bool:
+        return (self.cfr_type in (CFRType.discounted, CFRType.discounted_plus) and t <= self.dcfr_delay) or t == 0
+
+    def prepare_replay(self, t: int) -> None:
+        """Refresh every iteration-dependent device scalar for iteration ``t``; call outside
+        any captured region (fused_sparse_cfr_evaluator.py:535-550)."""
+        self.apply_schedules(t)
+        mix_old, mix_new = self._get_mixing_weights(t)
+        self._t_scalars.update(t=t, dcfr_alpha=self.dcfr_alpha, dcfr_beta=self.dcfr_beta,
+                               mix_old=float(mix_old), mix_new=float(mix_new))
+        apply_dcfr = self.cfr_type in (CFRType.discounted, CFRType.discounted_plus)
+        a, b = float(t ** self.dcfr_alpha), float(t ** self.dcfr_beta)
+        total = float(mix_old) + float(mix_new)
+        f = self._fscal_host
+        f[0], f[1], f[2], f[3] = a, b, a + 1.0, b + 1.0
+        f[4], f[5], f[6] = float(mix_old), float(mix_new), total
+        f[7] = 1.0 / total if total != 0.0 else 1.0
+        i = self._iscal_host
+        i[0], i[1], i[2] = int(t), int(apply_dcfr), int(self.cfr_plus)
+        i[3], i[4], i[5] = int(self._avg_policy_copies(t)), int(self.enforce_zero_sum), int(not self.use_final_policy_values)
+        self._fscal.copy_(f, non_blocking=True)
+        self._iscal.copy_(i, non_blocking=True)
+
+    def _get_sampling_schedule(self) -> torch.Tensor:
+        """cfr_evaluator.py:382-404: per-root iteration at which the policy is snapshotted."""
+        N = self.root_nodes
+        if self.cfr_type == CFRType.discounted_plus:
+            low = max(self.warm_start_iterations, self.dcfr_delay) + 1
+        else:
+            low = self.warm_start_iterations + 1
+        low = min(low, self.cfr_iterations)
+        high = max(self.cfr_iterations, low + 1)
+        if self.cfr_type != CFRType.standard:
+            dist = torch.arange(low, high, dtype=torch.float32) + 1
+        else:
+            dist = torch.ones(high - low)
+        dist /= dist.sum()
+        gen = self.generator if (self.generator is not None and self.generator.device.type == "cpu") else None
+        ts = torch.multinomial(dist, N, replacement=True, generator=gen) + low
+        return ts.to(self.device)[self._root_index].contiguous()
+
+    # ------------------------------------------------------------------ per-op building blocks
+    def _mask_invalid(self, tensor: torch.Tensor) -> None:
+        pass  # every row of the sparse tree is a real node
+
+    def _normalize_beliefs(self, target: torch.Tensor | None = None) -> None:
+        F.fused_block_and_normalize_beliefs_(self.beliefs if target is None else target,
+                                             self.allowed_hands, self.allowed_hands_prob)
+
+    def _calculate_reach_weights(self, target: torch.Tensor, policy: torch.Tensor) -> None:
+        for depth in range(self.tree_depth):
+            F.fused_reach_weights_depth_(reach=target, policy=policy, allowed_mask=self.allowed_hands,
+                                         parent_index=self.parent_index, prev_actor=self.prev_actor,
+                                         start=self.depth_offsets[depth + 1], end=self.depth_offsets[depth + 2])
+
+    def _get_root_index(self) -> torch.Tensor:
+        return self._root_index
+
+    def _propagate_all_beliefs(self, target: torch.Tensor | None = None,
+                               reach_weights: torch.Tensor | None = None) -> None:
+        target = self.beliefs if target is None else target
+        reach_weights = self.self_reach if reach_weights is None else reach_weights
+        F.fused_deep_beliefs_(out=target, root_beliefs=target, reach_weights=reach_weights,
+                              allowed_prob=self.allowed_hands_prob, root_index=self._root_index,
+                              num_roots=self.root_nodes)
+
+    def update_policy(self, t: int) -> None:
+        """fused_sparse_cfr_evaluator.py:201-236."""
+        bottom, top = self.depth_offsets[1], self.depth_offsets[-2]
+        if self._fused_positive_regrets_buf is None or \
+                self._fused_positive_regrets_buf.shape != self.cumulative_regrets.shape:
+            self._fused_positive_regrets_buf = torch.empty_like(self.cumulative_regrets)
+        pos = self._fused_positive_regrets_buf
+        torch.clamp(self.cumulative_regrets, min=0.0, out=pos)
+        parent_sum = F.fused_parent_sum(pos, self.child_offsets[:top].contiguous(),
+                                        self.child_count[:top].contiguous(), max_children=self.num_actions)
+        F.fused_divide_by_parent_sum_(pos=pos[bottom:], fallback=self.uniform_policy[bottom:], parent_sum=parent_sum,
+                                      parent_index=self.parent_index[bottom:].contiguous(),
+                                      out=self.policy_probs[bottom:])
+        self._calculate_reach_weights(self.self_reach, self.policy_probs)
+        self._propagate_all_beliefs(self.beliefs, self.self_reach)
+        self.update_average_policy(t)
+        self._calculate_reach_weights(self.self_reach_avg, self.policy_probs_avg)
+        self._propagate_all_beliefs(self.beliefs_avg, self.self_reach_avg)
+
+    def update_average_policy(self, t: int) -> None:
+        """fused_sparse_cfr_evaluator.py:355-398."""
+        if self._avg_policy_copies(t):
+            self.policy_probs_avg[:] = self.policy_probs
+            return
+        N, top = self.root_nodes, self.depth_offsets[-2]
+        F.fused_average_policy_mix_with_tensors_(
+            policy_probs_avg=self.policy_probs_avg, policy_probs=self.policy_probs, self_reach=self.self_reach,
+            self_reach_avg=self.self_reach_avg, to_act=self.env.to_act, parent_index=self.parent_index,
+            old=self._t_scalars.mix_old, new=self._t_scalars.mix_new, total_weight=self._t_scalars.mix_total,
+            bottom=N)
+        parent_sum = F.fused_parent_sum(self.policy_probs_avg, self.child_offsets[:top].contiguous(),
+                                        self.child_count[:top].contiguous(), max_children=self.num_actions)
+        child = self.policy_probs_avg[N:]
+        F.fused_divide_by_parent_sum_(pos=child, fallback=child, parent_sum=parent_sum,
+                                      parent_index=self.parent_index[N:].contiguous(), out=child, eps=1e-5)
+        self.policy_probs_avg[:N] = 0.0
+
+    def compute_instantaneous_regrets(self, values_achieved: torch.Tensor,
+                                      values_expected: torch.Tensor | None = None) -> torch.Tensor:
+        """fused_sparse_cfr_evaluator.py:312-349."""
+        if values_expected is None:
+            values_expected = values_achieved
+        bottom, top = self.depth_offsets[1], self.depth_offsets[-2]
+        beliefs = self.beliefs_avg if self.cfr_avg else self.beliefs
+        regrets = torch.zeros_like(self.policy_probs)
+        src_weights = F.unblocked_mass_opp_at_parents_triton(beliefs, self.env.to_act, top)
+        rows = torch.arange(top, device=self.device)
+        actor_values = values_expected[:top][rows, self.env.to_act[:top], :].contiguous()
+        F.fused_regret_tail_(regrets=regrets, values_achieved=values_achieved.contiguous(), actor_values=actor_values,
+                             src_weights=src_weights, parent_index=self.parent_index, prev_actor=self.prev_actor,
+                             bottom=bottom)
+        return regrets
+
+    def compute_expected_values(self, policy=None, beliefs=None, leaf_values=None, values=None) -> None:
+        """fused_sparse_cfr_evaluator.py:242-306."""
+        policy = self.policy_probs if policy is None else policy
+        beliefs = self.beliefs if beliefs is None else beliefs
+        leaf_values = self.latest_values if leaf_values is None else leaf_values
+        values = leaf_values if values is None else values
+        if leaf_values is not values:
+            torch.where(self.leaf_mask[:, None, None], leaf_values, torch.zeros_like(values), out=values)
+        bottom, top = self.depth_offsets[1], self.depth_offsets[-2]
+        rows = torch.arange(top, device=self.device)
+        actor_beliefs = beliefs[:top][rows, self.env.to_act[:top], :].contiguous()
+        marginal = actor_beliefs.index_select(0, self.parent_index[bottom:]) * policy[bottom:]
+        occ = torch.zeros_like(policy)
+        occ[bottom:] = F.unblocked_mass_ratio_indirect_triton(
+            numer_target=marginal.contiguous(), denom_target=actor_beliefs,
+            parent_index=self.parent_index[bottom:].contiguous())
+        for depth in range(self.tree_depth - 1, -1, -1):
+            base, end = self.depth_offsets[depth], self.depth_offsets[depth + 1]
+            F.fused_weighted_parent_sum(values=values, prev_actor=self.prev_actor, policy_hero=policy, policy_opp=occ,
+                                        child_offsets=self.child_offsets[base:end].contiguous(),
+                                        child_count=self.child_count[base:end].contiguous(), parent_base=base,
+                                        max_children=self.num_actions)
+
+    def update_average_values(self, t: int) -> None:
+        """fused_sparse_cfr_evaluator.py:404-414."""
+        F.fused_avg_values_zero_sum_(values_avg=self.values_avg, latest_values=self.latest_values,
+                                     beliefs=self.beliefs_avg, old=self._t_scalars.mix_old,
+                                     new=self._t_scalars.mix_new, inv_total=self._t_scalars.mix_inv_total,
+                                     enforce_zero_sum=self.enforce_zero_sum, ignore_mask=self.env.done)
+
+    # ------------------------------------------------------------------ leaf values
+    def _model_leaf_values(self, beliefs: torch.Tensor) -> torch.Tensor | None:
+        if self.model_indices.numel() == 0:
+            return None
+        if self.model is None:
+            return torch.zeros(self.model_indices.numel(), 2, NUM_HANDS, dtype=self.float_dtype, device=self.device)
+        return self.model.leaf_values(beliefs[self.model_indices], self.model_indices, self).to(self.float_dtype)
+
+    def _set_model_values_impl(self, t: int, beliefs: torch.Tensor) -> None:
+        """fused_sparse_cfr_evaluator.py:420-445 (CFR-AVG de-averaging included)."""
+        hv = self._model_leaf_values(beliefs)
+        if hv is None:
+            return
+        if (not self.cfr_avg) or t <= 1 or self.last_model_values is None:
+            self.latest_values.index_copy_(0, self.model_indices, hv)
+        else:
+            unmixed = torch.empty_like(hv)
+            F.fused_model_values_mix_zero_sum(hv.contiguous(), self.last_model_values.contiguous(),
+                                              beliefs[self.model_indices].contiguous(), self._t_scalars.mix_onon,
+                                              self._t_scalars.mix_oon, unmixed, self.enforce_zero_sum)
+            self.latest_values.index_copy_(0, self.model_indices, unmixed)
+        self.last_model_values = hv
+
+    @torch.no_grad()
+    def set_leaf_values(self, t: int, beliefs: torch.Tensor | None = None, *, showdown: bool = True) -> None:
+        """fused_sparse_cfr_evaluator.py:447-472: model rows through PyTorch, showdown rows
+        through the showdown kernel; fold rows are constants set at construction."""
+        if beliefs is None:
+            beliefs = self.beliefs_avg if self.cfr_avg else self.beliefs
+        self._set_model_values_impl(t, beliefs)
+        if showdown and self.showdown_indices.numel():
+            self.latest_values[self.showdown_indices] = self._showdown_value_both(beliefs[self.showdown_indices])
+
+    # ------------------------------------------------------------------ iteration
+    def _build_iter_args(self) -> _IterArgs:
+        a = _IterArgs()
+        p = _lib.ptr
+        a.child_offsets, a.child_count, a.to_act = p(self.child_offsets), p(self.child_count), p(self.env.to_act)
+        a.node_flags, a.root_node_offsets, a.root_nodes = p(self._node_flags), p(self._root_node_offsets), p(self._root_nodes)
+        a.t_sample, a.allowed, a.allowed_prob = p(self.t_sample), p(self.allowed_hands), p(self.allowed_hands_prob)
+        a.tables = p(self.hand_rank_data) if self.hand_rank_data is not None else None
+        a.potential, a.scale = p(self._potential_all), p(self.env.scale)
+        a.policy, a.policy_avg, a.policy_sample = p(self.policy_probs), p(self.policy_probs_avg), p(self.policy_probs_sample)
+        a.cum, a.wsum = p(self.cumulative_regrets), p(self.regret_weight_sums)
+        a.beliefs, a.beliefs_avg = p(self.beliefs), p(self.beliefs_avg)
+        a.reach, a.reach_avg = p(self.self_reach), p(self.self_reach_avg)
+        a.latest, a.values_avg, a.scratch = p(self.latest_values), p(self.values_avg), p(self._scratch)
+        a.fscal, a.iscal = p(self._fscal), p(self._iscal)
+        return a
+
+    def _launch_iteration(self, phases: int) -> None:
+        if self._iter_args is None:
+            self._iter_args = self._build_iter_args()
+        if self.cfr_avg:
+            raise NotImplementedError("the one-kernel iteration covers cfr_avg=False; use fused_iteration=False")
+        code = _lib.load().p2hip_cfr_iteration(ctypes.byref(self._iter_args), self.root_nodes, self._max_children,
+                                               phases, _lib.stream_ptr())
+        _lib.check(code, "p2hip_cfr_iteration")
+
+    def cfr_iteration(self, t: int) -> None:
+        """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533)."""
+        if not self._skip_t_scalars_update:
+            self.prepare_replay(t)
+        if self.cfr_type == CFRType.linear and self.fused_iteration:
+            raise NotImplementedError("linear CFR runs through fused_iteration=False")
+        if self.fused_iteration:
+            if self._has_model_leaves and self.model is not None:
+                self._launch_iteration(1)
+                self.set_leaf_values(t, showdown=False)
+                self._launch_iteration(2)
+            else:
+                self._launch_iteration(3)
+            return
+        F.fused_sample_snapshot_(self.policy_probs_sample, self.policy_probs, self.t_sample, self._t_scalars.t_tensor)
+        regrets = self.compute_instantaneous_regrets(self.latest_values)
+        if self.cfr_type == CFRType.linear:
+            regrets.masked_fill_(self.prev_actor[:, None] == t % self.num_players, 0.0)
+            self.regret_weight_sums += 1
+            self.cumulative_regrets += regrets
+        else:
+            F.fused_dcfr_update_with_tensors_(
+                cumulative_regrets=self.cumulative_regrets, regret_weight_sums=self.regret_weight_sums,
+                regrets=regrets, t_alpha_num=self._t_scalars.t_alpha_num, t_beta_num=self._t_scalars.t_beta_num,
+                t_alpha_den=self._t_scalars.t_alpha_den, t_beta_den=self._t_scalars.t_beta_den,
+                apply_dcfr=self.cfr_type in (CFRType.discounted, CFRType.discounted_plus), cfr_plus=self.cfr_plus)
+        self.update_policy(t)
+        self.set_leaf_values(t)
+        self.compute_expected_values()
+        if not self.use_final_policy_values:
+            self.update_average_values(t)
+
+    # ------------------------------------------------------------------ whole search
+    @torch.no_grad()
+    def initialize_policy_and_beliefs(self) -> None:
+        """cfr_evaluator.py:830-886: initial policy from the model's logits (uniform over the
+        legal actions without a model), beliefs pushed down level by level."""
+        self.policy_probs.zero_()
+        if self.tree_depth == 0:
+            self._normalize_beliefs()
+        for depth in range(self.tree_depth):
+            o, on, onn = self.depth_offsets[depth], self.depth_offsets[depth + 1], self.depth_offsets[depth + 2]
+            rows = torch.arange(o, on, device=self.device)
+            if self.model is not None and hasattr(self.model, "policy_logits"):
+                logits = self.model.policy_logits(self.beliefs, rows, self).to(self.float_dtype)
+            else:
+                logits = torch.zeros(on - o, NUM_HANDS, self.num_actions, dtype=self.float_dtype, device=self.device)
+            legal = self.legal_mask[o:on][:, None, :]
+            probs = torch.softmax(logits.masked_fill(~legal, float("-inf")), dim=-1)
+            probs = torch.nan_to_num(probs, nan=0.0)
+            probs.masked_fill_((self.child_count[o:on] == 0)[:, None, None], 0.0)
+            src = probs.permute(0, 2, 1)  # [K, A, H]
+            self.policy_probs[on:onn] = src[self.parent_index[on:onn] - o, self.action_from_parent[on:onn]]
+            child = self.beliefs[self.parent_index[on:onn]].clone()
+            idx = torch.arange(onn - on, device=self.device)
+            child[idx, self.prev_actor[on:onn]] *= self.policy_probs[on:onn]
+            self.beliefs[on:onn] = child
+            self._normalize_beliefs()
+        self._calculate_reach_weights(self.self_reach, self.policy_probs)
+        self.policy_probs_avg[:] = self.policy_probs
+        self.self_reach_avg[:] = self.self_reach
+        self.beliefs_avg[:] = self.beliefs
+
+    def prepare_search(self, t_sample: torch.Tensor | None = None) -> None:
+        """Everything ``evaluate_cfr`` does before its loop (cfr_evaluator.py:1505-1515)."""
+        self.initialize_policy_and_beliefs()
+        self.prepare_replay(0)
+        self.set_leaf_values(0)
+        self.compute_expected_values()
+        self.values_avg[:] = self.latest_values
+        if t_sample is None:
+            t_sample = self._get_sampling_schedule()
+        self.t_sample.copy_(t_sample.to(self.device))
+
+    def evaluate_cfr(self, training_mode: bool = True) -> None:
+        """cfr_evaluator.py:1497-1528 without the post-search leaf sampling and statistics."""
+        self.prepare_search()
+        for t in range(self.warm_start_iterations, self.cfr_iterations):
+            self.cfr_iteration(t)
+        if self.use_final_policy_values:
+            self.update_average_values_final()
+
+    def update_average_values_final(self) -> None:
+        """cfr_evaluator.py:1276-1292."""
+        self.set_leaf_values(0, beliefs=self.beliefs_avg)
+        self.compute_expected_values(self.policy_probs_avg, self.beliefs_avg, self.latest_values, self.values_avg)
+        if self.enforce_zero_sum:
+            s = (self.values_avg * self.beliefs_avg).sum(dim=2, keepdim=True).mean(dim=1, keepdim=True)
+            s.masked_fill_(self.env.done[:, None, None], 0.0)
+            self.values_avg -= s
+
+    def state_dict(self) -> dict:
+        return {n: getattr(self, n) for n in STATE_NAMES}
+
+
+class GraphedCFRIteration:
+    """Captures ``evaluator.cfr_iteration`` into a HIP graph and replays it for any ``t``
+    (src/p2/search/fused_cfr_triton.py:2359-2451).  The iteration-dependent scalars live in
+    device memory and are refreshed by ``prepare_replay`` outside the graph."""
+
+    def __init__(self, evaluator: HipSparseCFREvaluator) -> None:
+        if evaluator.device.type != "cuda":
+            raise ValueError("GraphedCFRIteration requires a GPU evaluator.")
+        self.evaluator = evaluator
+        self._graph = None
+        self._captured_t = None
+
+    def capture(self, t_capture: int, num_warmup: int = 2) -> None:
+        ev = self.evaluator
+        for i in range(num_warmup):
+            ev.cfr_iteration(t_capture + i)
+        ev.prepare_replay(t_capture)
+        prev = ev._skip_t_scalars_update
+        ev._skip_t_scalars_update = True
+        try:
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                ev.cfr_iteration(t_capture)
+            torch.cuda.current_stream().wait_stream(s)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=s):
+                ev.cfr_iteration(t_capture)
+        finally:
+            ev._skip_t_scalars_update = prev
+        self._graph = graph
+        self._captured_t = t_capture
+
+    def replay(self, t: int | None = None) -> None:
+        if self._graph is None:
+            raise RuntimeError("capture() must be called before replay().")
+        if t is not None:
+            self.evaluator.prepare_replay(t)
+        self._graph.replay()
+
+    @property
+    def captured_t(self):
+        return self._captured_t

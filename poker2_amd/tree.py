@@ -1,0 +1,293 @@
+"""Sparse betting-tree construction on the host (numpy, all roots at once).
+
+Produces the tree layout every kernel consumes -- the one the reference builds in
+``SparseCFREvaluator._construct_subgame`` (src/p2/search/sparse_cfr_evaluator.py:142-306)
+by stepping its tensor env: rows are level-major, the children of one parent are
+contiguous and ordered by action bin, and a child's row holds the quantities "for
+the action that leads to it".
+
+The betting rules are those of src/p2/env/hunl_tensor_env.py (legality :348-423,
+bet / fold reward :684-724, step and round closure :766-897): integer chips, a
+pot-fraction bet is ``trunc(float32(fraction) * float32(pot))`` on top of the call,
+all-in always available, a betting round closes after two actions when the
+commitments match (or an all-in is covered), the river closes into a showdown.
+
+``max_raises`` is an extension for synthetic benchmark trees (the reference caps by
+ply depth only): once that many bets/raises were made in the round, only fold and
+call remain.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+
+H = 1326
+
+
+@dataclass
+class RootStates:
+    """Public state of N subgame roots (numpy arrays of length N)."""
+    street: np.ndarray
+    to_act: np.ndarray
+    button: np.ndarray
+    pot: np.ndarray
+    stacks: np.ndarray            # [N,2]
+    committed: np.ndarray         # [N,2]
+    min_raise: np.ndarray
+    actions_this_round: np.ndarray
+    is_allin: np.ndarray          # [N,2] bool
+    starting_stacks: np.ndarray   # [N,2]
+    scale: np.ndarray             # [N] float32
+    board: np.ndarray             # [N,5] int64, -1 = not dealt
+    done: np.ndarray = None       # [N] bool
+    bb: int = 100
+
+    def __post_init__(self):
+        if self.done is None:
+            self.done = np.zeros(self.street.shape[0], dtype=bool)
+
+    @property
+    def n(self) -> int:
+        return int(self.street.shape[0])
+
+    def select(self, idx) -> "RootStates":
+        """Rows ``idx`` as a new RootStates."""
+        idx = np.asarray(idx)
+        kw = {}
+        for name in self.__dataclass_fields__:
+            v = getattr(self, name)
+            kw[name] = v[idx] if isinstance(v, np.ndarray) else v
+        return RootStates(**kw)
+
+    @classmethod
+    def at_round_start(cls, street, pot, stacks, board, button=0, bb: int = 100,
+                       starting_stacks=None, scale=None) -> "RootStates":
+        """Roots at the start of a betting round: nothing committed, the non-button player
+        acts first.  By default each player is taken to have paid half the pot already."""
+        pot = np.atleast_1d(np.asarray(pot, dtype=np.int64))
+        n = pot.shape[0]
+        stacks = np.broadcast_to(np.asarray(stacks, dtype=np.int64), (n, 2)).copy()
+        button = np.broadcast_to(np.asarray(button, dtype=np.int64), (n,)).copy()
+        street = np.broadcast_to(np.asarray(street, dtype=np.int64), (n,)).copy()
+        if starting_stacks is None:
+            starting_stacks = stacks + (pot // 2)[:, None]
+        starting_stacks = np.broadcast_to(np.asarray(starting_stacks, dtype=np.int64), (n, 2)).copy()
+        if scale is None:
+            scale = starting_stacks[:, 0].astype(np.float32)
+        scale = np.broadcast_to(np.asarray(scale, dtype=np.float32), (n,)).copy()
+        board = np.asarray(board, dtype=np.int64)
+        if board.ndim == 1:
+            board = np.broadcast_to(board, (n, board.shape[0]))
+        full = np.full((n, 5), -1, dtype=np.int64)
+        full[:, : board.shape[1]] = board
+        return cls(street=street, to_act=1 - button, button=button, pot=pot, stacks=stacks,
+                   committed=np.zeros((n, 2), np.int64), min_raise=np.full(n, bb, np.int64),
+                   actions_this_round=np.zeros(n, np.int64), is_allin=np.zeros((n, 2), bool),
+                   starting_stacks=starting_stacks, scale=scale, board=full, bb=bb)
+
+    @classmethod
+    def from_env(cls, env, indices) -> "RootStates":
+        """Copy rows of an object exposing the reference env's attribute names
+        (``HUNLTensorEnv``: button, street, to_act, pot, stacks, committed, min_raise,
+        actions_this_round, is_allin, starting_stacks, scale, board_indices, done, bb)."""
+        def g(name):
+            x = getattr(env, name)
+            x = x.detach().cpu().numpy() if hasattr(x, "detach") else np.asarray(x)
+            return x[np.asarray(indices)]
+        idx = indices.detach().cpu().numpy() if hasattr(indices, "detach") else np.asarray(indices)
+        indices = idx
+        return cls(street=g("street").astype(np.int64), to_act=g("to_act").astype(np.int64),
+                   button=g("button").astype(np.int64), pot=g("pot").astype(np.int64),
+                   stacks=g("stacks").astype(np.int64), committed=g("committed").astype(np.int64),
+                   min_raise=g("min_raise").astype(np.int64),
+                   actions_this_round=g("actions_this_round").astype(np.int64),
+                   is_allin=g("is_allin").astype(bool), starting_stacks=g("starting_stacks").astype(np.int64),
+                   scale=g("scale").astype(np.float32), board=g("board_indices").astype(np.int64),
+                   done=g("done").astype(bool), bb=int(getattr(env, "bb", 100)))
+
+
+_STATE_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",
+                 "is_allin", "starting_stacks", "scale", "done", "raises")
+
+
+def _legal_mask(s: dict, bins: list[float], max_raises: int | None) -> tuple[np.ndarray, np.ndarray]:
+    n = s["pot"].shape[0]
+    nb = len(bins) + 3
+    rows = np.arange(n)
+    me, opp = s["to_act"], 1 - s["to_act"]
+    me_stack, opp_stack = s["stacks"][rows, me], s["stacks"][rows, opp]
+    to_call = s["committed"][rows, opp] - s["committed"][rows, me]
+    amounts = np.full((n, nb), -1, dtype=np.int64)
+    mask = np.zeros((n, nb), dtype=bool)
+    mask[:, 0] = to_call > 0
+    mask[:, 1] = True
+    fr = np.asarray(bins, dtype=np.float32)
+    additional = (fr[None, :] * s["pot"].astype(np.float32)[:, None]).astype(np.int64)  # truncates
+    amt = to_call[:, None] + additional
+    can = (me_stack > 0) & (opp_stack > 0)
+    amounts[:, 2:-1] = amt
+    mask[:, 2:-1] = can[:, None] & (amt <= me_stack[:, None]) & (additional >= s["min_raise"][:, None])
+    amounts[:, nb - 1] = me_stack
+    mask[:, nb - 1] = me_stack > 0
+    if max_raises is not None:
+        capped = s["raises"] >= max_raises
+        mask[capped, 2:] = False
+    opp_allin = s["is_allin"][rows, opp]
+    mask[opp_allin, 0:2] = True
+    mask[opp_allin, 2:] = False
+    me_allin = s["is_allin"][rows, me]
+    mask[me_allin, :] = False
+    mask[me_allin, 1] = True
+    mask &= ~s["done"][:, None]
+    return amounts, mask
+
+
+def _step(parent: dict, prow: np.ndarray, bins_taken: np.ndarray, amounts: np.ndarray, nb: int, bb: int):
+    """Children of ``parent`` rows ``prow`` after taking ``bins_taken``; returns (state, fold reward)."""
+    c = {k: parent[k][prow].copy() for k in _STATE_FIELDS}
+    m = prow.shape[0]
+    rows = np.arange(m)
+    me, opp = c["to_act"].copy(), 1 - c["to_act"]
+    to_call = c["committed"][rows, opp] - c["committed"][rows, me]
+    me_stack = c["stacks"][rows, me]
+    fold = bins_taken == 0
+    call = bins_taken == 1
+    allin = bins_taken == nb - 1
+    bet = ~(fold | call | allin)
+    chips = np.zeros(m, dtype=np.int64)
+    chips[call] = np.minimum(to_call, me_stack)[call]
+    chips[allin] = me_stack[allin]
+    chips[bet] = amounts[prow, bins_taken][bet]
+    c["stacks"][rows, me] -= chips
+    c["committed"][rows, me] += chips
+    c["pot"] += chips
+    c["is_allin"][rows[allin], me[allin]] = True
+    c["min_raise"][bet] = np.maximum(c["min_raise"], chips - to_call)[bet]
+    c["raises"] = c["raises"] + (bet | allin).astype(np.int64)
+    # fold: the other player takes the pot; value for player 0 in units of `scale`
+    reward = np.zeros(m, dtype=np.float32)
+    f32 = np.float32
+    share = np.where(opp == 0, c["pot"].astype(f32), f32(0.0))
+    r = (c["stacks"][:, 0].astype(f32) + share - c["starting_stacks"][:, 0].astype(f32)) / c["scale"]
+    reward[fold] = r[fold]
+    c["done"] = c["done"] | fold
+    c["to_act"] = 1 - c["to_act"]
+    c["actions_this_round"] = c["actions_this_round"] + 1
+    equal = c["committed"][:, 0] == c["committed"][:, 1]
+    a0, a1 = c["is_allin"][:, 0], c["is_allin"][:, 1]
+    covered = (a0 & a1) | (a0 & (c["committed"][:, 0] <= c["committed"][:, 1])) | \
+        (a1 & (c["committed"][:, 1] <= c["committed"][:, 0]))
+    closed = ~c["done"] & (equal | covered) & (c["actions_this_round"] >= 2)
+    c["committed"][closed] = 0
+    c["actions_this_round"][closed] = 0
+    c["raises"][closed] = 0
+    c["to_act"][closed] = 1 - c["button"][closed]
+    c["min_raise"][closed] = bb
+    c["done"] = c["done"] | (closed & (c["street"] == 3))  # river closes into a showdown
+    c["street"] = c["street"] + closed.astype(np.int64)
+    return c, reward
+
+
+@dataclass
+class SparseTree:
+    depth_offsets: list
+    n_roots: int
+    total: int
+    num_actions: int
+    bet_bins: list
+    parent_index: np.ndarray
+    action_from_parent: np.ndarray
+    child_count: np.ndarray
+    child_offsets: np.ndarray
+    prev_actor: np.ndarray
+    root_index: np.ndarray
+    legal_mask: np.ndarray
+    leaf_mask: np.ndarray
+    new_street_mask: np.ndarray
+    fold_mask: np.ndarray
+    showdown_mask: np.ndarray
+    reward: np.ndarray
+    state: dict = field(repr=False)
+    board: np.ndarray = None      # [n_roots,5]
+
+    @property
+    def tree_depth(self) -> int:
+        return max(0, len(self.depth_offsets) - 2)
+
+    @property
+    def top(self) -> int:
+        return self.depth_offsets[-2] if len(self.depth_offsets) > 1 else self.n_roots
+
+    def __getattr__(self, name):
+        st = object.__getattribute__(self, "state")
+        if name in st:
+            return st[name]
+        raise AttributeError(name)
+
+    @property
+    def showdown_potential(self) -> np.ndarray:
+        """[total,2] chips player p nets by winning the pot (sparse_cfr_evaluator.py:249-253)."""
+        return self.state["stacks"] + self.state["pot"][:, None] - self.state["starting_stacks"]
+
+
+def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
+                      max_raises: int | None = None) -> SparseTree:
+    """Breadth-first expansion to ``depth`` plies.  Below the root level a node whose betting
+    round has just closed (``actions_this_round == 0``, which includes showdowns) is not
+    expanded (sparse_cfr_evaluator.py:167-197)."""
+    assert roots.n > 0, "must supply at least one root state"
+    bins = [float(b) for b in bet_bins]
+    nb = len(bins) + 3
+    n = roots.n
+    s0 = {k: np.array(getattr(roots, k)) for k in _STATE_FIELDS if k != "raises"}
+    s0["raises"] = np.zeros(n, dtype=np.int64)
+    levels = [s0]
+    parents = [np.full(n, -1, dtype=np.int64)]
+    actions = [np.full(n, -1, dtype=np.int64)]
+    rewards = [np.zeros(n, dtype=np.float32)]
+    offsets = [0, n]
+    d = 0
+    while d < depth:
+        par = levels[-1]
+        amounts, legal = _legal_mask(par, bins, max_raises)
+        if d > 0:
+            legal &= (par["actions_this_round"] != 0)[:, None]
+        prow, taken = np.nonzero(legal)  # parent-major, action-ascending
+        if prow.size == 0:
+            break
+        child, rew = _step(par, prow, taken, amounts, nb, roots.bb)
+        levels.append(child)
+        parents.append(prow + offsets[-2])
+        actions.append(taken.astype(np.int64))
+        rewards.append(rew)
+        offsets.append(offsets[-1] + prow.size)
+        d += 1
+    state = {k: np.concatenate([lv[k] for lv in levels]) for k in _STATE_FIELDS}
+    total = offsets[-1]
+    parent_index = np.concatenate(parents)
+    action = np.concatenate(actions)
+    reward = np.concatenate(rewards)
+    _, legal = _legal_mask(state, bins, max_raises)
+    is_root = np.zeros(total, dtype=bool)
+    is_root[:n] = True
+    new_street = (state["actions_this_round"] == 0) & ~is_root
+    leaf = state["done"] | new_street
+    leaf[offsets[-2]:] = True
+    child_mask = legal & ~leaf[:, None]
+    child_count = child_mask.sum(axis=1).astype(np.int64)
+    assert total == n + int(child_count.sum())
+    assert (child_count[~leaf] > 0).all() and not leaf[:n].any()
+    child_offsets = (offsets[1] + np.cumsum(child_count) - child_count).astype(np.int64)
+    prev_actor = np.full(total, -1, dtype=np.int64)
+    prev_actor[n:] = state["to_act"][parent_index[n:]]
+    root_index = np.arange(total, dtype=np.int64)
+    for lv in range(len(offsets) - 2):
+        s, e = offsets[lv + 1], offsets[lv + 2]
+        root_index[s:e] = root_index[parent_index[s:e]]
+    return SparseTree(depth_offsets=list(offsets), n_roots=n, total=total, num_actions=nb, bet_bins=bins,
+                      parent_index=parent_index, action_from_parent=action, child_count=child_count,
+                      child_offsets=child_offsets, prev_actor=prev_actor, root_index=root_index,
+                      legal_mask=legal, leaf_mask=leaf, new_street_mask=new_street,
+                      fold_mask=(action == 0) & state["done"], showdown_mask=state["street"] == 4,
+                      reward=reward, state=state, board=np.array(roots.board))

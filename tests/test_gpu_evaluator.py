@@ -1,0 +1,149 @@
+"""GPU parity of the whole CFR iteration: the one-kernel path and the per-operation path of
+HipSparseCFREvaluator against the numpy oracle on seeded river subgames."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cfr as OCFR
+from tests.helpers import random_boards, random_ranges
+
+pytestmark = pytest.mark.gpu
+
+
+def tree_as_dict(t):
+    d = {k: getattr(t, k) for k in ("depth_offsets", "parent_index", "action_from_parent", "child_count",
+                                    "child_offsets", "prev_actor", "legal_mask", "leaf_mask", "new_street_mask",
+                                    "fold_mask", "showdown_mask", "reward")}
+    d.update({k: t.state[k] for k in ("to_act", "done", "scale")})
+    d["showdown_potential"] = t.showdown_potential
+    return d
+
+
+def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discounted", delay=0, cfr_plus=False,
+              enforce_zs=False, stacks=(800, 800), pot=200, t_sample=None, bins=(0.5, 1.0)):
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(seed)
+    boards = random_boards(rng, n_roots)
+    beliefs = random_ranges(rng, boards)
+    pots = np.full(n_roots, pot, dtype=np.int64)
+    buttons = np.arange(n_roots) % 2
+    roots = RootStates.at_round_start(3, pots, np.tile(np.array([stacks]), (n_roots, 1)), boards, button=buttons)
+    cfg = river_dcfr_config(n_roots, iterations=iters, depth=depth, dcfr_delay=delay)
+    cfg.search.cfr_type = CFRType[cfr_type]
+    cfg.search.cfr_plus = cfr_plus
+    cfg.env.bet_bins = list(bins)
+    model = None
+    if enforce_zs:
+        class ZeroModel:
+            enforce_zero_sum = True
+
+            def leaf_values(self, beliefs, rows, ev):
+                return torch.zeros_like(beliefs)
+        model = ZeroModel()
+    ev = HipSparseCFREvaluator(model, torch.device("cuda"), cfg, fused_iteration=fused, max_raises=max_raises)
+    ev.initialize_subgame(roots, np.arange(n_roots), torch.from_numpy(beliefs))
+    if t_sample is None:
+        t_sample = np.full(n_roots, -1, dtype=np.int64)
+    from oracle.ranker import rank_hands_cards
+
+    def ranker(board):  # same ranker as the product's showdown tables (card-id semantics)
+        packed, order = rank_hands_cards(board)
+        return packed, order
+    orc = OCFR.OracleCFR(tree_as_dict(ev.tree), boards, beliefs, cfr_type=cfr_type, dcfr_alpha=1.5, dcfr_beta=0.0,
+                         dcfr_gamma=2.0, dcfr_delay=delay, cfr_plus=cfr_plus, cfr_iterations=iters,
+                         enforce_zero_sum=enforce_zs, t_sample_roots=t_sample, ranker=ranker)
+    ev.prepare_search(t_sample=torch.from_numpy(np.asarray(t_sample))[torch.from_numpy(ev.tree.root_index)])
+    orc.prepare()
+    return ev, orc
+
+
+def compare(ev, orc, rtol, atol, names=None):
+    worst = {}
+    for name in names or OCFR.OracleCFR.STATE_NAMES:
+        a = getattr(ev, name).cpu().numpy()
+        b = getattr(orc, name)
+        err = np.abs(a - b) - (atol + rtol * np.abs(b))
+        worst[name] = float(np.abs(a - b).max())
+        assert (err <= 0).all(), f"{name}: max abs diff {np.abs(a - b).max():.3e}, violations {(err > 0).sum()}"
+    return worst
+
+
+def test_prepare_matches_oracle():
+    ev, orc = make_pair(3, 2, None, seed=1, fused=True, iters=4)
+    compare(ev, orc, rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("depth,max_raises", [(2, None), (16, 1), (16, 2)])
+def test_iterations_match_oracle(fused, depth, max_raises):
+    iters = 8
+    ev, orc = make_pair(3, depth, max_raises, seed=11 + depth, fused=fused, iters=iters,
+                        t_sample=np.array([2, 5, 100]))
+    for t in range(iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+        compare(ev, orc, rtol=2e-4, atol=2e-5)
+    # the snapshot of root 0 was taken at t = 2, of root 1 at t = 5, root 2 never
+    assert ev.policy_probs_sample[ev._root_index == 2].abs().max().item() == 0.0
+    assert ev.policy_probs_sample[ev._root_index == 0].abs().max().item() > 0.0
+
+
+@pytest.mark.parametrize("cfr_type,delay,cfr_plus,zs", [("discounted", 3, False, False),
+                                                         ("discounted_plus", 2, True, False),
+                                                         ("standard", 0, False, True)])
+def test_variants_fused_vs_oracle(cfr_type, delay, cfr_plus, zs):
+    iters = 7
+    ev, orc = make_pair(2, 2, None, seed=5, fused=True, iters=iters, cfr_type=cfr_type, delay=delay,
+                        cfr_plus=cfr_plus, enforce_zs=zs, stacks=(500, 900), pot=300, bins=(0.33, 0.75, 1.5))
+    for t in range(iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+    compare(ev, orc, rtol=2e-4, atol=2e-5)
+
+
+def test_fused_and_per_op_paths_agree_and_graph_replay():
+    from poker2_amd.evaluator import GraphedCFRIteration
+    iters = 12
+    ev_f, _ = make_pair(4, 2, None, seed=21, fused=True, iters=iters)
+    ev_p, _ = make_pair(4, 2, None, seed=21, fused=False, iters=iters)
+    ev_g, _ = make_pair(4, 2, None, seed=21, fused=True, iters=iters)
+    for t in range(3):
+        ev_g.cfr_iteration(t)
+    snap = {k: v.clone() for k, v in ev_g.state_dict().items()}
+    runner = GraphedCFRIteration(ev_g)
+    runner.capture(t_capture=3, num_warmup=0)
+    for k, v in snap.items():
+        ev_g.state_dict()[k].copy_(v)  # capture ran iteration 3 twice: rewind to the state after t = 2
+    for t in range(iters):
+        ev_f.cfr_iteration(t)
+        ev_p.cfr_iteration(t)
+        if t >= 3:
+            runner.replay(t)
+            torch.cuda.synchronize()
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        a, b, g = getattr(ev_f, name), getattr(ev_p, name), getattr(ev_g, name)
+        torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-5, msg=lambda m: f"{name}: {m}")
+        assert torch.equal(a, g), f"graph replay differs on {name}"
+
+
+def test_structural_invariants_after_many_iterations():
+    iters = 60
+    ev, _ = make_pair(8, 16, 1, seed=3, fused=True, iters=iters)
+    for t in range(iters):
+        ev.cfr_iteration(t)
+    top, n = ev.depth_offsets[-2], ev.root_nodes
+    for pol in (ev.policy_probs, ev.policy_probs_avg):
+        s = torch.zeros(top, 1326, device="cuda").index_add_(0, ev.parent_index[n:], pol[n:])
+        torch.testing.assert_close(s, torch.ones_like(s), rtol=0, atol=1e-5)
+    for b in (ev.beliefs, ev.beliefs_avg):
+        torch.testing.assert_close(b.sum(-1), torch.ones_like(b.sum(-1)), rtol=0, atol=1e-5)
+    par = ev.parent_index[n:]
+    assert (ev.self_reach[n:] <= ev.self_reach[par] + 1e-7).all()
+    assert torch.isfinite(ev.values_avg).all() and ev.values_avg.abs().max() <= 1.0 + 1e-4
+    # blocked hands never carry reach below the root
+    assert (ev.self_reach[n:][~ev.allowed_hands[n:]][:, None].expand(-1, 1) == 0).all() if False else True
+    blocked = ~ev.allowed_hands[n:]
+    assert (ev.self_reach[n:, 0][blocked] == 0).all() and (ev.self_reach[n:, 1][blocked] == 0).all()

@@ -1,0 +1,79 @@
+"""CPU: the product's vectorised tree builder and the oracle's scalar one against the
+fixture written by the reference's own HUNLTensorEnv, and against each other."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import tree as OT
+from poker2_amd.tree import RootStates, build_sparse_tree
+
+STATE_KEYS = ["to_act", "street", "pot", "min_raise", "actions_this_round", "done", "stacks", "committed",
+              "is_allin", "starting_stacks", "scale"]
+
+
+def cases(golden_dir):
+    g = np.load(os.path.join(golden_dir, "tree_golden.npz"))
+    for name in sorted({k.split("/")[0] for k in g.files}):
+        yield name, {k.split("/")[1]: g[k] for k in g.files if k.startswith(name + "/")}
+
+
+def roots_of(case):
+    r = case["roots"]
+    pot, stacks, button = r[:, 0], r[:, 1:3], r[:, 3]
+    street = int(case["root_street"])
+    prod = RootStates.at_round_start(street, pot, stacks, np.full((len(r), 5), -1), button=button)
+    orac = [OT.make_root(street, int(p), int(s[0]), int(s[1]), button=int(b)) for p, s, b in zip(pot, stacks, button)]
+    return prod, orac
+
+
+def test_builders_match_reference_env_fixture(golden_dir):
+    n = 0
+    for name, case in cases(golden_dir):
+        bins = [float(x) for x in case["bins"]]
+        depth = int(case["depth"])
+        prod, orac = roots_of(case)
+        t = build_sparse_tree(prod, bins, depth)
+        o = OT.build_tree(orac, bins, depth)
+        assert t.depth_offsets == list(case["depth_offsets"]) == o["depth_offsets"], name
+        assert np.array_equal(t.parent_index, case["parent_index"]) and np.array_equal(o["parent_index"], case["parent_index"])
+        assert np.array_equal(t.action_from_parent, case["action_from_parent"])
+        assert np.array_equal(o["action_from_parent"], case["action_from_parent"])
+        for k in STATE_KEYS:
+            assert np.array_equal(t.state[k], case[k].astype(t.state[k].dtype)), (name, k)
+            assert np.array_equal(o[k], case[k].astype(o[k].dtype)), (name, k)
+        assert np.array_equal(t.legal_mask, case["legal_mask"]) and np.array_equal(o["legal_mask"], case["legal_mask"])
+        fm = t.fold_mask
+        assert np.array_equal(fm, o["fold_mask"])
+        assert np.array_equal(t.reward[fm], case["reward"][fm]) and np.array_equal(o["reward"][fm], case["reward"][fm])
+        for k in ("child_count", "child_offsets", "prev_actor", "leaf_mask", "new_street_mask", "showdown_mask"):
+            assert np.array_equal(getattr(t, k), o[k]), (name, k)
+        assert np.array_equal(t.showdown_potential, o["showdown_potential"])
+        n += 1
+    assert n >= 6
+
+
+def test_hand_derived_river_tree():
+    # pot 200, stacks 800/800, bins {0.5, 1}: root 4 children, then 4, 5, 5, 2 -> 21 nodes
+    roots = RootStates.at_round_start(3, [200], [[800, 800]], np.arange(5)[None])
+    t = build_sparse_tree(roots, [0.5, 1.0], 2)
+    assert t.depth_offsets == [0, 1, 5, 21]
+    assert t.child_count[:5].tolist() == [4, 4, 5, 5, 2]
+    assert t.action_from_parent[1:5].tolist() == [1, 2, 3, 4]
+    assert t.root_index.tolist() == [0] * 21
+    # check-check is a showdown worth half the pot to either player
+    sd = np.nonzero(t.showdown_mask)[0]
+    assert 5 in sd and t.showdown_potential[5].tolist() == [100, 100]
+    # folding to the half-pot bet: player 0 (first to act when button = 0 ... to_act = 1) loses nothing more
+    assert t.fold_mask.sum() == 3
+
+
+def test_full_river_tree_is_terminal_and_max_raises_extension():
+    roots = RootStates.at_round_start(3, [200], [[800, 800]], np.arange(5)[None])
+    full = build_sparse_tree(roots, [0.5, 1.0], 16)
+    assert full.state["done"][full.leaf_mask].all()  # every leaf is a fold or a showdown
+    capped = build_sparse_tree(roots, [0.5, 1.0], 16, max_raises=3)
+    assert capped.state["done"][capped.leaf_mask].all()
+    assert capped.total < full.total
+    with pytest.raises(AssertionError):
+        build_sparse_tree(RootStates.at_round_start(3, np.zeros(0), np.zeros((0, 2)), np.zeros((0, 5))), [0.5], 2)
