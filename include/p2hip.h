@@ -220,6 +220,11 @@ typedef struct P2HipIterArgs {
 int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max_children, int phases,
                         void* stream);
 
+/* Copy 8 floats and 8 int64 from HOST arrays into the device arrays fscal[8] / iscal[8] read by
+ * p2hip_cfr_iteration.  The values travel as kernel arguments: the host arrays may be reused as
+ * soon as the call returns.  Plays the role of TScalars.update, search/fused_cfr_triton.py:2131-2158. */
+int p2hip_write_scalars(float* fscal, int64_t* iscal, const float* host_f, const int64_t* host_i, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,8 +82,17 @@ class OracleCFR:
         policy_logits_fn: Callable | None = None,
         t_sample_roots: np.ndarray | None = None,
         ranker=None,
+        fused_variant: bool = False,
     ) -> None:
         assert cfr_type in CFR_TYPES
+        # fused_variant=True follows FusedSparseCFREvaluator where it departs from the base
+        # class on rows / hands that carry no probability mass:
+        #   * root rows of self_reach(_avg) stay 1.0 on board-blocked hands (the fused reach
+        #     kernel only writes child rows, fused_sparse_cfr_evaluator.py:153-172);
+        #   * root rows of beliefs(_avg) are not re-normalised every iteration (the fused
+        #     belief kernel skips them, fused_cfr_triton.py:2008-2011);
+        #   * average values use (a*old + v*new) * (1/(old+new)) (fused_cfr_triton.py:604-605).
+        self.fused_variant = fused_variant
         self.tree = tree
         self.depth_offsets = list(tree["depth_offsets"])
         self.tree_depth = max(0, len(self.depth_offsets) - 2)
@@ -207,11 +216,18 @@ class OracleCFR:
             rows = np.arange(e - s)
             dest[rows, self.prev_actor[s:e]] *= policy[s:e]
             target[s:e] = dest
-        self.block_beliefs(target)
+        if self.fused_variant:
+            n = self.root_nodes
+            target[n:][np.broadcast_to(~self.allowed_hands[n:, None, :], target[n:].shape)] = 0.0
+        else:
+            self.block_beliefs(target)
 
     def propagate_all_beliefs(self, target: np.ndarray, reach: np.ndarray) -> None:
-        target[:] = self.fan_out_deep(target[: self.root_nodes].copy()) * reach
+        roots = target[: self.root_nodes].copy()
+        target[:] = self.fan_out_deep(roots) * reach
         self.normalize_beliefs(target)
+        if self.fused_variant:
+            target[: self.root_nodes] = roots
 
     # ---- schedules / weights --------------------------------------------------
     def mixing_weights(self, t: int):
@@ -392,9 +408,13 @@ class OracleCFR:
 
     def update_average_values(self, t: int) -> None:
         old, new = self.mixing_weights(t)
-        self.values_avg *= F32(old)
-        self.values_avg += F32(new) * self.latest_values
-        self.values_avg /= F32(old + new)
+        if self.fused_variant:
+            inv = F32(1.0 / (float(old) + float(new)))
+            self.values_avg[:] = (self.values_avg * F32(old) + self.latest_values * F32(new)) * inv
+        else:
+            self.values_avg *= F32(old)
+            self.values_avg += F32(new) * self.latest_values
+            self.values_avg /= F32(old + new)
         self.values_avg[:] = self.maybe_enforce_zero_sum(self.values_avg, self.beliefs_avg, ignore_mask=self.done)
 
     # ---- one iteration (cfr_evaluator.py:1330-1381) -----------------------------

@@ -150,6 +150,25 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
   if (A.phases & 1) {
     // ---------------- sweep 1: regrets -> DCFR -> regret matching ----------------
     const bool take_sample = A.t_sample[r] == t_now;
+    {
+      // The root row takes part in the flat DCFR update like every other row: its regret is
+      // zero (never positive), so only its weight sum moves.
+      float2 ws[IT_PPT];
+      ld(ws, A.wsum, r, ln);
+      IT_FOR(j) {
+        float ww[2] = {ws[j].x, ws[j].y};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          if (apply_dcfr) {
+            ww[e] = ww[e] * f_bn;
+            ww[e] = ww[e] / f_bd;
+          }
+          ww[e] = ww[e] + 1.0f;
+        }
+        ws[j] = make_float2(ww[0], ww[1]);
+      }
+      st(A.wsum, r, ws, ln);
+    }
     for (int64_t q = n0; q < n1; ++q) {
       const int64_t p = A.root_nodes[q];
       const int cnt = (int)A.child_count[p];
@@ -473,9 +492,35 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
   }
 }
 
+struct ScalarPack {
+  float f[8];
+  int64_t i[8];
+};
+
+// The values travel as kernel arguments, so the host may reuse its buffers at once.
+__global__ void write_scalars_kernel(float* __restrict__ fscal, int64_t* __restrict__ iscal, ScalarPack v) {
+  const int k = threadIdx.x;
+  if (k < 8) {
+    fscal[k] = v.f[k];
+    iscal[k] = v.i[k];
+  }
+}
+
 }  // namespace p2
 
 extern "C" {
+
+int p2hip_write_scalars(float* fscal, int64_t* iscal, const float* host_f, const int64_t* host_i, void* stream) {
+  if (!fscal || !iscal || !host_f || !host_i) return P2_EINVAL;
+  p2::ScalarPack v;
+  for (int k = 0; k < 8; ++k) {
+    v.f[k] = host_f[k];
+    v.i[k] = host_i[k];
+  }
+  hipLaunchKernelGGL(p2::write_scalars_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, fscal, iscal, v);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
 
 // P2HipIterArgs (include/p2hip.h) mirrors p2::IterArgs field by field.
 

@@ -106,8 +106,8 @@ class HipSparseCFREvaluator:
         self._fused_positive_regrets_buf = None
         self._fscal = torch.zeros(8, dtype=torch.float32, device=self.device)
         self._iscal = torch.zeros(8, dtype=torch.int64, device=self.device)
-        self._fscal_host = torch.zeros(8, dtype=torch.float32).pin_memory()
-        self._iscal_host = torch.zeros(8, dtype=torch.int64).pin_memory()
+        self._fscal_host = (ctypes.c_float * 8)()
+        self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
 
     @property
@@ -294,8 +294,8 @@ class HipSparseCFREvaluator:
         i = self._iscal_host
         i[0], i[1], i[2] = int(t), int(apply_dcfr), int(self.cfr_plus)
         i[3], i[4], i[5] = int(self._avg_policy_copies(t)), int(self.enforce_zero_sum), int(not self.use_final_policy_values)
-        self._fscal.copy_(f, non_blocking=True)
-        self._iscal.copy_(i, non_blocking=True)
+        _lib.call("p2hip_write_scalars", _lib.ptr(self._fscal), _lib.ptr(self._iscal),
+                  ctypes.cast(f, ctypes.c_void_p), ctypes.cast(i, ctypes.c_void_p), _lib.stream_ptr())
 
     def _get_sampling_schedule(self) -> torch.Tensor:
         """cfr_evaluator.py:382-404: per-root iteration at which the policy is snapshotted."""
