@@ -148,6 +148,7 @@ def test_structural_invariants_after_many_iterations():
     top, n = ev.depth_offsets[-2], ev.root_nodes
     for pol in (ev.policy_probs, ev.policy_probs_avg):
         s = torch.zeros(top, 1326, device="cuda").index_add_(0, ev.parent_index[n:], pol[n:])
+        s = s[ev.child_count[:top] > 0]  # leaves at intermediate depths have no policy
         torch.testing.assert_close(s, torch.ones_like(s), rtol=0, atol=1e-5)
     for b in (ev.beliefs, ev.beliefs_avg):
         torch.testing.assert_close(b.sum(-1), torch.ones_like(b.sum(-1)), rtol=0, atol=1e-5)
@@ -155,6 +156,5 @@ def test_structural_invariants_after_many_iterations():
     assert (ev.self_reach[n:] <= ev.self_reach[par] + 1e-7).all()
     assert torch.isfinite(ev.values_avg).all() and ev.values_avg.abs().max() <= 1.0 + 1e-4
     # blocked hands never carry reach below the root
-    assert (ev.self_reach[n:][~ev.allowed_hands[n:]][:, None].expand(-1, 1) == 0).all() if False else True
     blocked = ~ev.allowed_hands[n:]
     assert (ev.self_reach[n:, 0][blocked] == 0).all() and (ev.self_reach[n:, 1][blocked] == 0).all()
