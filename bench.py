@@ -148,6 +148,9 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy three times (reference point for "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: every box of this build has one GPU and the path shards by root "
@@ -158,6 +161,13 @@ def main() -> None:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU fallback exists for the product path).", file=sys.stderr)
         sys.exit(1)
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     ev, _, _ = make_evaluator(args.roots, args.tree, args.seed, iterations=args.warmup + args.steps + 1)
     nodes_per_root = ev.total_nodes // ev.root_nodes
     t = 0
