@@ -176,7 +176,8 @@ int p2hip_sample_snapshot(const float* policy_probs, float* policy_probs_sample,
 /* Device pointers of one subgame batch.  Tree arrays and state tensors are the evaluator's
  * own (row-major over all nodes of all roots); the rest is derived once per subgame:
  *   node_flags [total] bytes: bit0 = river showdown row, bit1 = terminal row
- *   root_node_offsets [roots+1], root_nodes [total]: rows of each root's subtree, ascending
+ *   root_parent_offsets [roots+1], root_parents: rows that have children, per root, ascending
+ *   root_showdown_offsets [roots+1], root_showdown_nodes: river showdown rows per root
  *   tables [roots, p2hip_showdown_table_bytes()] (NULL when no row is a showdown)
  *   potential [total,2] float, scale [total] float: showdown pay-off factors per row
  *   scratch [total,H] float workspace
@@ -187,8 +188,10 @@ typedef struct P2HipIterArgs {
   const int64_t* child_count;
   const int64_t* to_act;
   const uint8_t* node_flags;
-  const int64_t* root_node_offsets;
-  const int64_t* root_nodes;
+  const int64_t* root_parent_offsets;
+  const int64_t* root_parents;
+  const int64_t* root_showdown_offsets;
+  const int64_t* root_showdown_nodes;
   const int64_t* t_sample;
   const uint8_t* allowed;
   const float* allowed_prob;

@@ -4,8 +4,8 @@
 //            regrets, DCFR discount + accumulate, regret matching -> policy_probs
 //   sweep 2 (top-down): reach, beliefs, average-policy mix + renormalise, reach_avg,
 //            beliefs_avg
-//   sweep 3 (bottom-up): showdown leaves, opponent-conditioned policy, value backup,
-//            average values
+//   sweep 3: showdown leaves first (their values depend only on the new beliefs), then
+//            bottom-up: opponent-conditioned policy, value backup, average values
 // which is the order of FusedSparseCFREvaluator.cfr_iteration
 // (src/p2/search/fused_sparse_cfr_evaluator.py:478-533) with every per-op launch of
 // src/p2/search/fused_cfr_triton.py folded in.  `phases` lets the host split the
@@ -24,10 +24,18 @@ namespace p2 {
 constexpr int IT_BLOCK = 256;
 constexpr int IT_WAVES = IT_BLOCK / 64;
 constexpr int IT_PPT = 3;  // pairs per thread: 3 * 256 = 768 >= 663
+#ifndef P2_IT_MIN_WAVES
+#define P2_IT_MIN_WAVES 3
+#endif
+constexpr int IT_MIN_WAVES = P2_IT_MIN_WAVES;  // waves per SIMD the register budget is capped for
 static_assert(IT_BLOCK == UB_BLOCK && IT_BLOCK == SD_BLOCK, "shared helpers assume one block size");
 
 constexpr uint8_t NODE_SHOWDOWN = 1;  // river showdown leaf: value from the showdown evaluator
 constexpr uint8_t NODE_DONE = 2;      // terminal node: excluded from the zero-sum shift
+// vectors card-summed per batch: what the LDS union holds next to the showdown buffers, and
+// never less than one family (parent + children)
+template <int MAXC>
+struct ItChunk { static constexpr int value = (MAXC + 1) > 8 ? (MAXC + 1) : 8; };
 
 struct IterArgs {
   // tree (row-major arrays over all nodes of all roots, as the evaluator keeps them)
@@ -35,8 +43,10 @@ struct IterArgs {
   const int64_t* child_count;
   const int64_t* to_act;
   const uint8_t* node_flags;
-  const int64_t* root_node_offsets;  // [roots+1] into root_nodes
-  const int64_t* root_nodes;         // rows of each root's subtree, ascending (= top-down)
+  const int64_t* root_parent_offsets;    // [roots+1] into root_parents
+  const int64_t* root_parents;           // rows with children of each root's subtree, ascending (= top-down)
+  const int64_t* root_showdown_offsets;  // [roots+1] into root_showdown_nodes
+  const int64_t* root_showdown_nodes;    // river showdown rows of each root's subtree
   const int64_t* t_sample;           // [total]
   const uint8_t* allowed;            // [total,H] bytes
   const float* allowed_prob;         // [total,H]
@@ -62,16 +72,30 @@ struct IterArgs {
   int phases;            // bit 0: sweeps 1+2, bit 1: sweep 3
 };
 
+constexpr int IT_VSTRIDE = P2_H + 2;  // floats between vectors staged in LDS
+
+template <int CH>
 struct IterLds {
-  __align__(8) float vec[P2_H + 2];
-  __align__(8) float vec2[P2_H + 2];
-  double cs[P2_CARDS];
-  double S;
+  union {
+    float vecs[CH][IT_VSTRIDE];  // vectors whose card sums are being taken
+    ShowdownLds sd;              // showdown scans (never live at the same time)
+  } u;
+  double cs[CH * P2_CARDS];
   float red[IT_WAVES][4];
-  ShowdownLds sd;
 };
 
 #define IT_FOR(j) _Pragma("unroll") for (int j = 0; j < IT_PPT; ++j)
+
+// Section timing for tuning builds only (-DP2_ITER_PROFILE); compiled out of the library.
+#ifdef P2_ITER_PROFILE
+__device__ long long g_iter_prof[8192][8];
+#define PROF_BEGIN(var) const long long var = wall_clock64()
+#define PROF_END(slot, var) \
+  do { if (threadIdx.x == 0) g_iter_prof[blockIdx.x & 8191][slot] += wall_clock64() - (var); } while (0)
+#else
+#define PROF_BEGIN(var)
+#define PROF_END(slot, var)
+#endif
 
 struct Lane {
   int idx[IT_PPT];      // pair index
@@ -107,12 +131,12 @@ __device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[4]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int q = 0; q < 4; ++q) v[q] = p2_wave_sum(v[q]);
-  __syncthreads();
+  p2_sync_lds();
   if (lane == 0) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) red[wave][q] = v[q];
   }
-  __syncthreads();
+  p2_sync_lds();
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     float s = 0.f;
@@ -125,10 +149,11 @@ __device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[4]) {
 __device__ __forceinline__ float2 mul2(float2 a, float2 b) { return make_float2(a.x * b.x, a.y * b.y); }
 
 template <int MAXC>
-__global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
-  __shared__ IterLds L;
+__global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(IterArgs A) {
+  constexpr int IT_CHUNK = ItChunk<MAXC>::value;
+  __shared__ IterLds<IT_CHUNK> L;
   const int64_t r = blockIdx.x;
-  const int64_t n0 = A.root_node_offsets[r], n1 = A.root_node_offsets[r + 1];
+  const int64_t pp0 = A.root_parent_offsets[r], pp1 = A.root_parent_offsets[r + 1];
 
   Lane ln;
   IT_FOR(j) {
@@ -149,6 +174,7 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
 
   if (A.phases & 1) {
     // ---------------- sweep 1: regrets -> DCFR -> regret matching ----------------
+    PROF_BEGIN(t_s1);
     const bool take_sample = A.t_sample[r] == t_now;
     {
       // The root row takes part in the flat DCFR update like every other row: its regret is
@@ -169,82 +195,101 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
       }
       st(A.wsum, r, ws, ln);
     }
-    for (int64_t q = n0; q < n1; ++q) {
-      const int64_t p = A.root_nodes[q];
-      const int cnt = (int)A.child_count[p];
-      if (cnt == 0) continue;
-      const int actor = (int)A.to_act[p];
-      const int64_t first = A.child_offsets[p];
-
-      float2 bo[IT_PPT], w[IT_PPT], ex[IT_PPT], tmp[IT_PPT];
-      ld(bo, A.beliefs, p * 2 + (1 - actor), ln);
-      to_lds(L.vec, bo, ln);
-      ld(ex, A.latest, p * 2 + actor, ln);
-      ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
-      st(A.scratch, p, tmp, ln);
-      __syncthreads();
-      card_sums(L.vec, L.cs, &L.S);
-      unblocked_regs(w, bo, L.cs, L.S, ln);
-
-      float2 pos[MAXC][IT_PPT];
-      float2 sum[IT_PPT];
-      IT_FOR(j) sum[j] = make_float2(0.f, 0.f);
+    for (int64_t i0 = pp0; i0 < pp1; i0 += IT_CHUNK) {
+      const int nch = (int)((pp1 - i0) < IT_CHUNK ? (pp1 - i0) : IT_CHUNK);
+      // opponent beliefs of every parent of the chunk: staged together, card-summed in one pass
+      PROF_BEGIN(t_c1);
 #pragma unroll
-      for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
-          const int64_t c = first + k;
-          float2 ach[IT_PPT], cu[IT_PPT], ws[IT_PPT];
-          ld(ach, A.latest, c * 2 + actor, ln);
-          ld(cu, A.cum, c, ln);
-          ld(ws, A.wsum, c, ln);
-          if (take_sample) {
-            ld(tmp, A.policy, c, ln);
-            st(A.policy_sample, c, tmp, ln);
-          }
-          IT_FOR(j) {
-            float cc[2] = {cu[j].x, cu[j].y}, ww[2] = {ws[j].x, ws[j].y};
-            const float rg[2] = {w[j].x * (ach[j].x - ex[j].x), w[j].y * (ach[j].y - ex[j].y)};
+      for (int u = 0; u < IT_CHUNK; ++u) {
+        if (u < nch) {
+          const int64_t p = A.root_parents[i0 + u];
+          const int actor = (int)A.to_act[p];
+          float2 bo[IT_PPT], tmp[IT_PPT];
+          ld(bo, A.beliefs, p * 2 + (1 - actor), ln);
+          ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
+          to_lds(L.u.vecs[u], bo, ln);
+          st(A.scratch, p, tmp, ln);
+        }
+      }
+      p2_sync_lds();
+      card_sums_multi(L.u.vecs[0], IT_VSTRIDE, nch, L.cs);
+      PROF_END(4, t_c1);
+      for (int u = 0; u < nch; ++u) {
+        const int64_t p = A.root_parents[i0 + u];
+        const int cnt = (int)A.child_count[p];
+        const int actor = (int)A.to_act[p];
+        const int64_t first = A.child_offsets[p];
+        float2 bo[IT_PPT], w[IT_PPT], ex[IT_PPT];
+        ld(ex, A.latest, p * 2 + actor, ln);
+        {
+          const float2* v2 = reinterpret_cast<const float2*>(L.u.vecs[u]);
+          IT_FOR(j) bo[j] = ln.ok[j] ? v2[ln.idx[j]] : make_float2(0.f, 0.f);
+        }
+        unblocked_regs(w, bo, L.cs + u * P2_CARDS, card_total(L.cs + u * P2_CARDS), ln);
+
+        float2 pos[MAXC][IT_PPT];
+        float2 sum[IT_PPT];
+        IT_FOR(j) sum[j] = make_float2(0.f, 0.f);
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-              if (apply_dcfr) {
-                const bool positive = cc[e] > 0.f;
-                const float num = positive ? f_an : f_bn, den = positive ? f_ad : f_bd;
-                cc[e] = cc[e] * num;
-                cc[e] = cc[e] / den;
-                ww[e] = ww[e] * num;
-                ww[e] = ww[e] / den;
-              }
-              ww[e] = ww[e] + 1.0f;
-              cc[e] = cc[e] + rg[e];
-              if (cfr_plus) cc[e] = fmaxf(cc[e], 0.f);
+        for (int k = 0; k < MAXC; ++k) {
+          if (k < cnt) {
+            const int64_t c = first + k;
+            float2 ach[IT_PPT], cu[IT_PPT], ws[IT_PPT];
+            ld(ach, A.latest, c * 2 + actor, ln);
+            ld(cu, A.cum, c, ln);
+            ld(ws, A.wsum, c, ln);
+            if (take_sample) {
+              float2 tmp[IT_PPT];
+              ld(tmp, A.policy, c, ln);
+              st(A.policy_sample, c, tmp, ln);
             }
-            cu[j] = make_float2(cc[0], cc[1]);
-            ws[j] = make_float2(ww[0], ww[1]);
-            pos[k][j] = make_float2(fmaxf(cc[0], 0.f), fmaxf(cc[1], 0.f));
-            sum[j].x += pos[k][j].x;
-            sum[j].y += pos[k][j].y;
-          }
-          st(A.cum, c, cu, ln);
-          st(A.wsum, c, ws, ln);
-        }
-      }
-      const float uniform = 1.0f / (float)cnt;
+            IT_FOR(j) {
+              float cc[2] = {cu[j].x, cu[j].y}, ww[2] = {ws[j].x, ws[j].y};
+              const float rg[2] = {w[j].x * (ach[j].x - ex[j].x), w[j].y * (ach[j].y - ex[j].y)};
 #pragma unroll
-      for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
-          float2 pol[IT_PPT];
-          IT_FOR(j) {
-            pol[j].x = sum[j].x > 1e-8f ? pos[k][j].x / fmaxf(sum[j].x, 1e-8f) : uniform;
-            pol[j].y = sum[j].y > 1e-8f ? pos[k][j].y / fmaxf(sum[j].y, 1e-8f) : uniform;
+              for (int e = 0; e < 2; ++e) {
+                if (apply_dcfr) {
+                  const bool positive = cc[e] > 0.f;
+                  const float num = positive ? f_an : f_bn, den = positive ? f_ad : f_bd;
+                  cc[e] = cc[e] * num;
+                  cc[e] = cc[e] / den;
+                  ww[e] = ww[e] * num;
+                  ww[e] = ww[e] / den;
+                }
+                ww[e] = ww[e] + 1.0f;
+                cc[e] = cc[e] + rg[e];
+                if (cfr_plus) cc[e] = fmaxf(cc[e], 0.f);
+              }
+              cu[j] = make_float2(cc[0], cc[1]);
+              ws[j] = make_float2(ww[0], ww[1]);
+              pos[k][j] = make_float2(fmaxf(cc[0], 0.f), fmaxf(cc[1], 0.f));
+              sum[j].x += pos[k][j].x;
+              sum[j].y += pos[k][j].y;
+            }
+            st(A.cum, c, cu, ln);
+            st(A.wsum, c, ws, ln);
           }
-          st(A.policy, first + k, pol, ln);
+        }
+        const float uniform = 1.0f / (float)cnt;
+#pragma unroll
+        for (int k = 0; k < MAXC; ++k) {
+          if (k < cnt) {
+            float2 pol[IT_PPT];
+            IT_FOR(j) {
+              pol[j].x = sum[j].x > 1e-8f ? pos[k][j].x / fmaxf(sum[j].x, 1e-8f) : uniform;
+              pol[j].y = sum[j].y > 1e-8f ? pos[k][j].y / fmaxf(sum[j].y, 1e-8f) : uniform;
+            }
+            st(A.policy, first + k, pol, ln);
+          }
         }
       }
-      __syncthreads();  // L.vec / L.cs are reused by the next family
+      p2_sync_lds();  // the staged vectors and L.cs are rewritten by the next chunk
     }
-    // sweep 2 re-reads policy / reach rows that the same lane wrote: no cross-lane hand-off
+    PROF_END(0, t_s1);
+    PROF_BEGIN(t_s2);
 
     // ---------------- sweep 2: reach, beliefs, average policy ----------------
+    // (re-reads policy / reach rows that the same lane wrote: no cross-lane hand-off)
     float2 rb[2][IT_PPT], rba[2][IT_PPT], ap[IT_PPT];
     uchar2 am[IT_PPT];
     ld(rb[0], A.beliefs, r * 2, ln);
@@ -256,10 +301,9 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
       const uchar2* m2 = reinterpret_cast<const uchar2*>(A.allowed + r * P2_H);
       IT_FOR(j) am[j] = ln.ok[j] ? m2[ln.idx[j]] : make_uchar2(0, 0);
     }
-    for (int64_t q = n0; q < n1; ++q) {
-      const int64_t p = A.root_nodes[q];
+    for (int64_t i = pp0; i < pp1; ++i) {
+      const int64_t p = A.root_parents[i];
       const int cnt = (int)A.child_count[p];
-      if (cnt == 0) continue;
       const int actor = (int)A.to_act[p];
       const int64_t first = A.child_offsets[p];
       float2 rn[2][IT_PPT], ran[2][IT_PPT], ra_old[IT_PPT];
@@ -337,7 +381,9 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
             st(A.reach, c * 2 + pl, rc[pl], ln);
             st(A.reach_avg, c * 2 + pl, rca[pl], ln);
           }
+          PROF_BEGIN(t_b2);
           block_sum4(s4, L.red);
+          PROF_END(6, t_b2);
 #pragma unroll
           for (int pl = 0; pl < 2; ++pl) {
             float2 o[IT_PPT], oa[IT_PPT];
@@ -351,78 +397,101 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
         }
       }
     }
+    PROF_END(1, t_s2);
   }
 
   if (A.phases & 2) {
-    // ---------------- sweep 3: leaf values, backup, average values ----------------
-    const uint8_t* tab = A.tables ? A.tables + r * SD_TABLE_BYTES : nullptr;
-    for (int64_t q = n1 - 1; q >= n0; --q) {
-      const int64_t p = A.root_nodes[q];
+    // ---------------- sweep 3a: showdown leaves ----------------
+    PROF_BEGIN(t_s3);
+    const int64_t sd0 = A.root_showdown_offsets[r], sd1 = A.root_showdown_offsets[r + 1];
+    if (sd1 > sd0 && A.tables) {
+      PROF_BEGIN(t_sd);
+      ShowdownRegs sdr;
+      showdown_load_regs(A.tables + r * SD_TABLE_BYTES, sdr);
+      // beliefs written in sweep 2 are gathered by other lanes here: the one hand-off through
+      // global memory, hence a full barrier
+      __syncthreads();
+      float vk[2][SD_PPT];
+      showdown_gather(A.beliefs + A.root_showdown_nodes[sd0] * 2 * P2_H, sdr, vk);
+      for (int64_t i = sd0; i < sd1; ++i) {
+        const int64_t c = A.root_showdown_nodes[i];
+        float vnext[2][SD_PPT];
+        if (i + 1 < sd1) showdown_gather(A.beliefs + A.root_showdown_nodes[i + 1] * 2 * P2_H, sdr, vnext);
+        // the EVs land in the sorted-range buffers, which the evaluation no longer needs by then
+        showdown_eval(vk, sdr, L.u.sd, L.u.sd.v[0], L.u.sd.v[1], A.potential[2 * c], A.potential[2 * c + 1],
+                      A.scale[c]);
+        p2_sync_lds();
+        float2 v[2][IT_PPT];
+        {
+          const float2* e0 = reinterpret_cast<const float2*>(L.u.sd.v[0]);
+          const float2* e1 = reinterpret_cast<const float2*>(L.u.sd.v[1]);
+          IT_FOR(j) {
+            v[0][j] = ln.ok[j] ? e0[ln.idx[j]] : make_float2(0.f, 0.f);
+            v[1][j] = ln.ok[j] ? e1[ln.idx[j]] : make_float2(0.f, 0.f);
+          }
+        }
+        st(A.latest, c * 2, v[0], ln);
+        st(A.latest, c * 2 + 1, v[1], ln);
+        p2_sync_lds();  // the next evaluation overwrites the buffers just read
+        if (i + 1 < sd1) {
+#pragma unroll
+          for (int q = 0; q < SD_PPT; ++q) { vk[0][q] = vnext[0][q]; vk[1][q] = vnext[1][q]; }
+        }
+      }
+      PROF_END(3, t_sd);
+    }
+
+    // ---------------- sweep 3b: backup, bottom-up ----------------
+    for (int64_t i = pp1 - 1; i >= pp0; --i) {
+      const int64_t p = A.root_parents[i];
       const int cnt = (int)A.child_count[p];
-      if (cnt == 0) continue;
       const int actor = (int)A.to_act[p];
       const int64_t first = A.child_offsets[p];
 
-      float2 ab[IT_PPT], dn[IT_PPT];
+      // actor beliefs at the parent and the marginal of every action, card-summed in one pass
+      PROF_BEGIN(t_c3);
+      float2 ab[IT_PPT], dn[IT_PPT], polk[MAXC][IT_PPT];
       ld(ab, A.beliefs, p * 2 + actor, ln);
-      to_lds(L.vec, ab, ln);
-      __syncthreads();
-      card_sums(L.vec, L.cs, &L.S);
-      unblocked_regs(dn, ab, L.cs, L.S, ln);
-      __syncthreads();  // L.cs is rewritten for every child below
+      to_lds(L.u.vecs[0], ab, ln);
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          float2 mg[IT_PPT];
+          ld(polk[k], A.policy, first + k, ln);
+          IT_FOR(j) mg[j] = mul2(ab[j], polk[k][j]);
+          to_lds(L.u.vecs[1 + k], mg, ln);
+        }
+      }
+      p2_sync_lds();
+      card_sums_multi(L.u.vecs[0], IT_VSTRIDE, cnt + 1, L.cs);
+      unblocked_regs(dn, ab, L.cs, card_total(L.cs), ln);
+      PROF_END(5, t_c3);
 
       float2 vp[2][IT_PPT];
       IT_FOR(j) vp[0][j] = vp[1][j] = make_float2(0.f, 0.f);
-      for (int k = 0; k < cnt; ++k) {
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k >= cnt) continue;
         const int64_t c = first + k;
-        float2 pol[IT_PPT], mg[IT_PPT], nm[IT_PPT], occ[IT_PPT];
-        ld(pol, A.policy, c, ln);
-        IT_FOR(j) mg[j] = mul2(ab[j], pol[j]);
-        to_lds(L.vec2, mg, ln);
-        __syncthreads();
-        card_sums(L.vec2, L.cs, &L.S);
-        unblocked_regs(nm, mg, L.cs, L.S, ln);
+        float2 v[2][IT_PPT], av[2][IT_PPT];
+        ld(v[0], A.latest, c * 2, ln);
+        ld(v[1], A.latest, c * 2 + 1, ln);
+        if (update_avg) {
+          ld(av[0], A.values_avg, c * 2, ln);
+          ld(av[1], A.values_avg, c * 2 + 1, ln);
+        }
+        float2 nm[IT_PPT], occ[IT_PPT];
+        {
+          float2 mg[IT_PPT];
+          IT_FOR(j) mg[j] = mul2(ab[j], polk[k][j]);
+          unblocked_regs(nm, mg, L.cs + (1 + k) * P2_CARDS, card_total(L.cs + (1 + k) * P2_CARDS), ln);
+        }
         IT_FOR(j) {
           occ[j].x = dn[j].x > 1e-5f ? nm[j].x / dn[j].x : 0.f;
           occ[j].y = dn[j].y > 1e-5f ? nm[j].y / dn[j].y : 0.f;
         }
-        const uint8_t flags = A.node_flags[c];
-        float2 v[2][IT_PPT];
-        if ((flags & NODE_SHOWDOWN) && tab) {
-          showdown_scan(A.beliefs + c * 2 * P2_H, tab, L.sd);
-          const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
-          const uint16_t* lr = reinterpret_cast<const uint16_t*>(tab + SD_OFF_LR);
-          const uchar4* cidx = reinterpret_cast<const uchar4*>(tab + SD_OFF_CIDX);
-          const float sc = A.scale[c], pot0 = A.potential[2 * c], pot1 = A.potential[2 * c + 1];
-          for (int s = threadIdx.x; s < P2_H; s += IT_BLOCK) {
-            const unsigned pk = perm[s];
-            const int h = pk & 0x7FFF;
-            const float keep = (pk & 0x8000u) ? 0.f : 1.f;
-            const int Lp = lr[2 * s], Rp = lr[2 * s + 1];
-            const uchar4 ci = cidx[s];
-            const float e0 = showdown_ev_at(L.sd, 0, s, h, Lp, Rp, ci) * keep;
-            const float e1 = showdown_ev_at(L.sd, 1, s, h, Lp, Rp, ci) * keep;
-            L.vec[h] = e0 * pot0 / sc;
-            L.vec2[h] = e1 * pot1 / sc;
-          }
-          __syncthreads();
-          {
-            const float2* e0 = reinterpret_cast<const float2*>(L.vec);
-            const float2* e1 = reinterpret_cast<const float2*>(L.vec2);
-            IT_FOR(j) {
-              v[0][j] = ln.ok[j] ? e0[ln.idx[j]] : make_float2(0.f, 0.f);
-              v[1][j] = ln.ok[j] ? e1[ln.idx[j]] : make_float2(0.f, 0.f);
-            }
-          }
-          st(A.latest, c * 2, v[0], ln);
-          st(A.latest, c * 2 + 1, v[1], ln);
-        } else {
-          ld(v[0], A.latest, c * 2, ln);
-          ld(v[1], A.latest, c * 2 + 1, ln);
-        }
-        __syncthreads();  // L.vec / L.vec2 / L.cs free for the next child
         IT_FOR(j) {
-          const float2 wa = pol[j], wo = occ[j];
+          const float2 wa = polk[k][j], wo = occ[j];
           if (actor == 0) {
             vp[0][j].x += v[0][j].x * wa.x; vp[0][j].y += v[0][j].y * wa.y;
             vp[1][j].x += v[1][j].x * wo.x; vp[1][j].y += v[1][j].y * wo.y;
@@ -437,10 +506,8 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
           float s4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int pl = 0; pl < 2; ++pl) {
-            float2 av[IT_PPT];
-            ld(av, A.values_avg, c * 2 + pl, ln);
-            IT_FOR(j) nv[pl][j] = make_float2((av[j].x * mix_old + v[pl][j].x * mix_new) * mix_inv,
-                                              (av[j].y * mix_old + v[pl][j].y * mix_new) * mix_inv);
+            IT_FOR(j) nv[pl][j] = make_float2((av[pl][j].x * mix_old + v[pl][j].x * mix_new) * mix_inv,
+                                              (av[pl][j].y * mix_old + v[pl][j].y * mix_new) * mix_inv);
             if (enforce_zs) {
               float2 ba[IT_PPT];
               ld(ba, A.beliefs_avg, c * 2 + pl, ln);
@@ -450,7 +517,7 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
           float shift = 0.f;
           if (enforce_zs) {
             block_sum4(s4, L.red);
-            shift = (flags & NODE_DONE) ? 0.f : 0.5f * s4[0];
+            shift = (A.node_flags[c] & NODE_DONE) ? 0.f : 0.5f * s4[0];
           }
 #pragma unroll
           for (int pl = 0; pl < 2; ++pl) {
@@ -461,7 +528,7 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
       }
       st(A.latest, p * 2, vp[0], ln);
       st(A.latest, p * 2 + 1, vp[1], ln);
-      if (q == n0 && update_avg) {
+      if (i == pp0 && update_avg) {
         // the root is nobody's child: update its average values here
         float2 nv[2][IT_PPT];
         float s4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -488,7 +555,9 @@ __global__ __launch_bounds__(IT_BLOCK) void cfr_iteration_kernel(IterArgs A) {
           st(A.values_avg, p * 2 + pl, nv[pl], ln);
         }
       }
+      p2_sync_lds();  // the staged vectors and L.cs are rewritten by the next family
     }
+    PROF_END(2, t_s3);
   }
 }
 
@@ -510,6 +579,18 @@ __global__ void write_scalars_kernel(float* __restrict__ fscal, int64_t* __restr
 
 extern "C" {
 
+#ifdef P2_ITER_PROFILE
+int p2hip_iter_prof_read(long long* host, int reset) {
+  hipError_t e = hipMemcpyFromSymbol(host, HIP_SYMBOL(p2::g_iter_prof), sizeof(long long) * 8192 * 8);
+  if (e != hipSuccess) return (int)e;
+  if (reset) {
+    static long long zeros[8192 * 8];
+    e = hipMemcpyToSymbol(HIP_SYMBOL(p2::g_iter_prof), zeros, sizeof(zeros));
+  }
+  return (int)e;
+}
+#endif
+
 int p2hip_write_scalars(float* fscal, int64_t* iscal, const float* host_f, const int64_t* host_i, void* stream) {
   if (!fscal || !iscal || !host_f || !host_i) return P2_EINVAL;
   p2::ScalarPack v;
@@ -530,7 +611,8 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max
     return P2_EINVAL;
   if (n_roots == 0) return 0;
   const P2HipIterArgs& h = *host_args;
-  const void* required[] = {h.child_offsets, h.child_count, h.to_act, h.node_flags, h.root_node_offsets, h.root_nodes,
+  const void* required[] = {h.child_offsets, h.child_count, h.to_act, h.node_flags, h.root_parent_offsets, h.root_parents,
+                            h.root_showdown_offsets, h.root_showdown_nodes,
                             h.t_sample, h.allowed, h.allowed_prob, h.potential, h.scale, h.policy, h.policy_avg,
                             h.policy_sample, h.cum, h.wsum, h.beliefs, h.beliefs_avg, h.reach, h.reach_avg, h.latest,
                             h.values_avg, h.scratch, h.fscal, h.iscal};
@@ -542,7 +624,8 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max
     if (!p2_aligned8(p)) return P2_EINVAL;
   p2::IterArgs a;
   a.child_offsets = h.child_offsets; a.child_count = h.child_count; a.to_act = h.to_act;
-  a.node_flags = h.node_flags; a.root_node_offsets = h.root_node_offsets; a.root_nodes = h.root_nodes;
+  a.node_flags = h.node_flags; a.root_parent_offsets = h.root_parent_offsets; a.root_parents = h.root_parents;
+  a.root_showdown_offsets = h.root_showdown_offsets; a.root_showdown_nodes = h.root_showdown_nodes;
   a.t_sample = h.t_sample; a.allowed = h.allowed; a.allowed_prob = h.allowed_prob; a.tables = h.tables;
   a.potential = h.potential; a.scale = h.scale; a.policy = h.policy; a.policy_avg = h.policy_avg;
   a.policy_sample = h.policy_sample; a.cum = h.cum; a.wsum = h.wsum; a.beliefs = h.beliefs;

@@ -46,10 +46,29 @@ __device__ __forceinline__ int p2_combo_index(int lo, int hi) {
 }
 
 // ---- wave64 primitives ------------------------------------------------------
-__device__ __forceinline__ float p2_wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, P2_WAVE);
+// DPP move with zero fill: lanes without a source (row edge, masked row) read 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float p2_dpp0(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+
+// Inclusive prefix sum over the 64 lanes: four row shifts inside each 16-lane row, then two
+// row broadcasts carry the row totals across (six VALU ops, no LDS traffic).
+__device__ __forceinline__ float p2_wave_scan_incl(float v) {
+  v += p2_dpp0<0x111, 0xF>(v);  // row_shr:1
+  v += p2_dpp0<0x112, 0xF>(v);  // row_shr:2
+  v += p2_dpp0<0x114, 0xF>(v);  // row_shr:4
+  v += p2_dpp0<0x118, 0xF>(v);  // row_shr:8
+  v += p2_dpp0<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+  v += p2_dpp0<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+__device__ __forceinline__ float p2_wave_scan_incl(float v, int /*lane*/) { return p2_wave_scan_incl(v); }
+
+__device__ __forceinline__ float p2_wave_sum(float v) {
+  v = p2_wave_scan_incl(v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 __device__ __forceinline__ double p2_wave_sum(double v) {
@@ -58,13 +77,12 @@ __device__ __forceinline__ double p2_wave_sum(double v) {
   return v;
 }
 
-__device__ __forceinline__ float p2_wave_scan_incl(float v, int lane) {
-#pragma unroll
-  for (int off = 1; off < P2_WAVE; off <<= 1) {
-    float o = __shfl_up(v, off, P2_WAVE);
-    if (lane >= off) v += o;
-  }
-  return v;
+// Workgroup barrier that orders LDS traffic only: outstanding global loads and stores are
+// NOT waited for, so it must not be used to hand global data between lanes.
+__device__ __forceinline__ void p2_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // Block-wide sum of one float per thread; `red` needs >= blockDim/64 floats.
@@ -73,9 +91,9 @@ template <int NWAVES>
 __device__ __forceinline__ float p2_block_sum(float v, float* red) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   v = p2_wave_sum(v);
-  __syncthreads();  // protect `red` from a previous use
+  p2_sync_lds();  // protect `red` from a previous use
   if (lane == 0) red[wave] = v;
-  __syncthreads();
+  p2_sync_lds();
   float s = 0.f;
 #pragma unroll
   for (int w = 0; w < NWAVES; ++w) s += red[w];
@@ -86,9 +104,9 @@ template <int NWAVES>
 __device__ __forceinline__ double p2_block_sum(double v, double* red) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   v = p2_wave_sum(v);
-  __syncthreads();
+  p2_sync_lds();
   if (lane == 0) red[wave] = v;
-  __syncthreads();
+  p2_sync_lds();
   double s = 0.0;
 #pragma unroll
   for (int w = 0; w < NWAVES; ++w) s += red[w];

@@ -214,79 +214,139 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_setup_kernel(const void* __
 }
 
 // ---- per-call evaluation ---------------------------------------------------------
+constexpr int SD_PPT = 6;  // consecutive sorted positions per thread: 256 * 6 = 1536 >= 1326
+
 // Everything the evaluation of one node needs in LDS.
 struct ShowdownLds {
-  float v[2][P2_H + 2];        // villain-of-hero-p range in strength order: v[p] = beliefs[1-p] sorted
+  __align__(8) float v[2][P2_H + 2];        // villain-of-hero-p range in strength order: v[p] = beliefs[1-p] sorted
   float P[2][P2_H + 2];        // exclusive prefix, P[p][k], k = 0..1326
   float Pc[2][P2_CARDS][52];   // per-card exclusive prefix, Pc[p][c][j], j = 0..51
   float part[2][SD_WAVES];
 };
 
-// Fill s.v / s.P / s.Pc for the node whose beliefs start at `bel` ([2,H]) using the
-// board table `tab`.  Ends with a barrier.
-__device__ __forceinline__ void showdown_scan(const float* __restrict__ bel, const uint8_t* __restrict__ tab,
-                                              ShowdownLds& s) {
+// The slice of one board's table that a lane needs, kept in registers for as long as the
+// board is in use (every showdown leaf of one root shares it).
+struct ShowdownRegs {
+  uint32_t perm[SD_PPT];   // combo index, bit 15 = blocked by the board; 0xFFFFFFFF past the end
+  uint32_t lr[SD_PPT];     // L | R << 16
+  uint32_t cidx[SD_PPT];   // iLa | iRa << 8 | iLb << 16 | iRb << 24
+  uint32_t ab[SD_PPT];     // the combo's two cards, a | b << 8
+  uint32_t clist[13];      // lane j < 51: sorted position of the j-th weakest combo of card wave + 4*i
+};
+
+__device__ __forceinline__ void showdown_load_regs(const uint8_t* __restrict__ tab, ShowdownRegs& R) {
   const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
+  const uint32_t* lr = reinterpret_cast<const uint32_t*>(tab + SD_OFF_LR);
+  const uint32_t* cidx = reinterpret_cast<const uint32_t*>(tab + SD_OFF_CIDX);
   const uint16_t* clist = reinterpret_cast<const uint16_t*>(tab + SD_OFF_CLIST);
+  const int k0 = threadIdx.x * SD_PPT;
+#pragma unroll
+  for (int i = 0; i < SD_PPT; ++i) {
+    const int k = k0 + i;
+    const bool ok = k < P2_H;
+    R.perm[i] = ok ? perm[k] : 0xFFFFFFFFu;
+    R.lr[i] = ok ? lr[k] : 0u;
+    R.cidx[i] = ok ? cidx[k] : 0u;
+  }
+#pragma unroll
+  for (int i = 0; i < SD_PPT; ++i) {
+    const int h = (R.perm[i] == 0xFFFFFFFFu) ? 0 : (int)(R.perm[i] & 0x7FFFu);
+    R.ab[i] = (uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8);
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // gather both ranges into strength order; hero p faces villain 1-p
-  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
-    const int h = perm[k] & 0x7FFF;
-    s.v[0][k] = bel[P2_H + h];
-    s.v[1][k] = bel[h];
-  }
-  __syncthreads();
-  // block scan: thread owns 6 consecutive positions
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int k0 = threadIdx.x * 6;
-    float x[6], local = 0.f;
-#pragma unroll
-    for (int i = 0; i < 6; ++i) { x[i] = (k0 + i < P2_H) ? s.v[p][k0 + i] : 0.f; local += x[i]; }
-    const float incl = p2_wave_scan_incl(local, lane);
-    if (lane == 63) s.part[p][wave] = incl;
-    __syncthreads();
-    float base = 0.f;
-    for (int w = 0; w < wave; ++w) base += s.part[p][w];
-    float run = base + (incl - local);
-#pragma unroll
-    for (int i = 0; i < 6; ++i) {
-      if (k0 + i <= P2_H) s.P[p][k0 + i] = run;
-      run += x[i];
-    }
-  }
-  // per-card prefixes: one wave scan per (player, card)
-  for (int q = wave; q < 2 * P2_CARDS; q += SD_WAVES) {
-    const int p = q / P2_CARDS, c = q % P2_CARDS;
-    float x = 0.f;
-    if (lane < 51) {
-      const unsigned pos = clist[c * 51 + lane];
-      x = pos < (unsigned)P2_H ? s.v[p][pos] : 0.f;
-    }
-    const float incl = p2_wave_scan_incl(x, lane);
-    if (lane < 51) s.Pc[p][c][lane + 1] = incl;
-    if (lane == 0) s.Pc[p][c][0] = 0.f;
-  }
-  __syncthreads();
+  for (int i = 0; i < 13; ++i) R.clist[i] = lane < 51 ? clist[(wave + 4 * i) * 51 + lane] : 0xFFFFu;
 }
 
-// EV of hero p for the hand at sorted position k (before the potential/scale factor).
-__device__ __forceinline__ float showdown_ev_at(const ShowdownLds& s, int p, int k, int h, int L, int R,
-                                                uchar4 ci) {
-  const int a = p2_combo.a[h], b = p2_combo.b[h];
-  const float vk = s.v[p][k];
-  const float PL = s.P[p][L], PR = s.P[p][R];
-  const float aL = s.Pc[p][a][ci.x], aR = s.Pc[p][a][ci.y];
-  const float bL = s.Pc[p][b][ci.z], bR = s.Pc[p][b][ci.w];
-  const float win = PL - aL - bL;
-  const float tie = (PR - PL) - (aR - aL) - (bR - bL) + vk;
-  float den = 1.0f - s.Pc[p][a][51] - s.Pc[p][b][51] + vk;
-  den = fmaxf(den, 1e-8f);
-  const bool valid = den > 1e-8f;
-  const float wp = valid ? win / den : 0.f;
-  const float tp = valid ? tie / den : 0.f;
-  const float lp = valid ? 1.0f - wp - tp : 0.f;
-  return wp - lp;
+// Gather both ranges of the node whose beliefs start at `bel` ([2,H]) into strength order:
+// vk[p][i] = villain-of-hero-p mass at this lane's i-th sorted position.
+__device__ __forceinline__ void showdown_gather(const float* __restrict__ bel, const ShowdownRegs& R,
+                                                float (&vk)[2][SD_PPT]) {
+#pragma unroll
+  for (int i = 0; i < SD_PPT; ++i) {
+    const bool ok = R.perm[i] != 0xFFFFFFFFu;
+    const int h = (int)(R.perm[i] & 0x7FFFu);
+    vk[0][i] = ok ? bel[P2_H + h] : 0.f;
+    vk[1][i] = ok ? bel[h] : 0.f;
+  }
+}
+
+// Showdown EV of both players from gathered ranges, written in combo order to ev0 / ev1 (LDS,
+// 1326 floats each) already multiplied by mul0 / mul1 and divided by `div`; 0 for combos blocked
+// by the board.  ev0 / ev1 may be s.v[0] / s.v[1] (dead by the time they are written).  Uses LDS
+// barriers only; the caller puts an LDS barrier before reading ev0 / ev1 and another before the
+// next call.
+__device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s,
+                                              float* ev0, float* ev1, float mul0, float mul1, float div) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int k0 = threadIdx.x * SD_PPT;
+  float local[2], incl[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    local[p] = 0.f;
+#pragma unroll
+    for (int i = 0; i < SD_PPT; ++i) {
+      if (k0 + i < P2_H) s.v[p][k0 + i] = vk[p][i];
+      local[p] += vk[p][i];
+    }
+    incl[p] = p2_wave_scan_incl(local[p]);
+    if (lane == 63) s.part[p][wave] = incl[p];
+  }
+  p2_sync_lds();
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    float base = 0.f;
+    for (int w = 0; w < wave; ++w) base += s.part[p][w];
+    float run = base + (incl[p] - local[p]);
+#pragma unroll
+    for (int i = 0; i < SD_PPT; ++i) {
+      if (k0 + i <= P2_H) s.P[p][k0 + i] = run;
+      run += vk[p][i];
+    }
+  }
+  // per-card prefixes: one wave scan per (player, card); this wave owns cards wave, wave+4, ...
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+#pragma unroll
+    for (int i = 0; i < 13; ++i) {
+      const int c = wave + 4 * i;
+      const uint32_t pos = R.clist[i];
+      const float x = pos < (uint32_t)P2_H ? s.v[p][pos] : 0.f;
+      const float sc = p2_wave_scan_incl(x);
+      if (lane < 51) s.Pc[p][c][lane + 1] = sc;
+      if (lane == 0) s.Pc[p][c][0] = 0.f;
+    }
+  }
+  p2_sync_lds();
+#pragma unroll
+  for (int i = 0; i < SD_PPT; ++i) {
+    if (R.perm[i] == 0xFFFFFFFFu) continue;
+    const int h = (int)(R.perm[i] & 0x7FFFu);
+    const float keep = (R.perm[i] & 0x8000u) ? 0.f : 1.f;
+    const int L = (int)(R.lr[i] & 0xFFFFu), Rr = (int)(R.lr[i] >> 16);
+    const int a = (int)(R.ab[i] & 0xFFu), b = (int)(R.ab[i] >> 8);
+    const int iLa = (int)(R.cidx[i] & 0xFFu), iRa = (int)((R.cidx[i] >> 8) & 0xFFu);
+    const int iLb = (int)((R.cidx[i] >> 16) & 0xFFu), iRb = (int)(R.cidx[i] >> 24);
+    float e[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const float v0 = vk[p][i];
+      const float PL = s.P[p][L], PR = s.P[p][Rr];
+      const float aL = s.Pc[p][a][iLa], aR = s.Pc[p][a][iRa];
+      const float bL = s.Pc[p][b][iLb], bR = s.Pc[p][b][iRb];
+      const float win = PL - aL - bL;
+      const float tie = (PR - PL) - (aR - aL) - (bR - bL) + v0;
+      float den = 1.0f - s.Pc[p][a][51] - s.Pc[p][b][51] + v0;
+      den = fmaxf(den, 1e-8f);
+      const bool valid = den > 1e-8f;
+      const float wp = valid ? win / den : 0.f;
+      const float tp = valid ? tie / den : 0.f;
+      const float lp = valid ? 1.0f - wp - tp : 0.f;
+      e[p] = (wp - lp) * keep;
+    }
+    ev0[h] = e[0] * mul0 / div;
+    ev1[h] = e[1] * mul1 / div;
+  }
 }
 
 // out[n] = showdown EV of both players at node n.
@@ -302,26 +362,20 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_both_kernel(const float* __
   __shared__ ShowdownLds s;
   const int64_t n = blockIdx.x;
   const int64_t row = table_row ? table_row[n] : n;
-  const uint8_t* tab = tables + row * SD_TABLE_BYTES;
-  showdown_scan(beliefs + n * 2 * P2_H, tab, s);
-  const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
-  const uint16_t* lr = reinterpret_cast<const uint16_t*>(tab + SD_OFF_LR);
-  const uchar4* cidx = reinterpret_cast<const uchar4*>(tab + SD_OFF_CIDX);
-  const float sc = scale[n];
-  const float pot0 = potential[2 * n], pot1 = potential[2 * n + 1];
-  float* o = out + n * 2 * P2_H;
-  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
-    const unsigned pk = perm[k];
-    const int h = pk & 0x7FFF;
-    const bool blocked = pk & 0x8000u;
-    const int L = lr[2 * k], R = lr[2 * k + 1];
-    const uchar4 ci = cidx[k];
-    float e0 = showdown_ev_at(s, 0, k, h, L, R, ci);
-    float e1 = showdown_ev_at(s, 1, k, h, L, R, ci);
-    e0 = e0 * (blocked ? 0.f : 1.f);
-    e1 = e1 * (blocked ? 0.f : 1.f);
-    o[h] = e0 * pot0 / sc;
-    o[P2_H + h] = e1 * pot1 / sc;
+  ShowdownRegs R;
+  showdown_load_regs(tables + row * SD_TABLE_BYTES, R);
+  // the EVs are written over the sorted ranges, which are dead once the card scans are done
+  float vk[2][SD_PPT];
+  showdown_gather(beliefs + n * 2 * P2_H, R, vk);
+  showdown_eval(vk, R, s, s.v[0], s.v[1], potential[2 * n], potential[2 * n + 1], scale[n]);
+  p2_sync_lds();
+  float2* o0 = p2_row2(out, n * 2);
+  float2* o1 = p2_row2(out, n * 2 + 1);
+  const float2* e0 = reinterpret_cast<const float2*>(s.v[0]);
+  const float2* e1 = reinterpret_cast<const float2*>(s.v[1]);
+  for (int i = threadIdx.x; i < P2_HPAIRS; i += SD_BLOCK) {
+    o0[i] = e0[i];
+    o1[i] = e1[i];
   }
 }
 
@@ -348,7 +402,7 @@ int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64
                         const float* potential, const float* scale, int64_t m, float* out, void* stream) {
   if (m < 0 || (m > 0 && (!beliefs || !tables || !potential || !scale || !out))) return P2_EINVAL;
   if (m == 0) return 0;
-  if (!p2_aligned8(tables) || !p2_aligned4(beliefs) || !p2_aligned4(out)) return P2_EINVAL;
+  if (!p2_aligned8(tables) || !p2_aligned4(beliefs) || !p2_aligned8(out)) return P2_EINVAL;
   hipLaunchKernelGGL(p2::showdown_both_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
                      beliefs, tables, table_row, potential, scale, out);
   P2_LAUNCH_CHECK();

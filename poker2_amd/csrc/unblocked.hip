@@ -16,26 +16,44 @@ namespace p2 {
 constexpr int UB_BLOCK = 256;
 constexpr int UB_WAVES = UB_BLOCK / 64;
 
-// Card sums of the row held in `t` (LDS, 1326 floats) -> cs[52], S.  Two barriers.
-__device__ __forceinline__ void card_sums(const float* t, double* cs, double* s_out) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int c = wave; c < P2_CARDS; c += UB_WAVES) {
+// Card sums of `nvec` vectors held in LDS (vector v starts at t + v*stride):
+// cs[v*52 + c] = sum of the 51 combos of vector v that hold card c, in float64.
+// Four lanes share one (vector, card) task: each adds 13 partner cards, two shuffles
+// combine them.  Every thread must call it after an LDS barrier that covers the staged
+// vectors; it ends with an LDS barrier.
+__device__ __forceinline__ void card_sums_multi(const float* t, int stride, int nvec, double* cs) {
+  const int sub = threadIdx.x & 3;
+  const int ntask = nvec * P2_CARDS;
+  for (int base = 0; base < ntask; base += UB_BLOCK / 4) {
+    const int task = base + (threadIdx.x >> 2);
+    const bool valid = task < ntask;
     double v = 0.0;
-    if (lane < 51) {
-      const int x = lane < c ? lane : lane + 1;  // partner card
-      const int lo = x < c ? x : c, hi = x < c ? c : x;
-      v = (double)t[p2_combo_index(lo, hi)];
+    if (valid) {
+      const int vec = task / P2_CARDS, c = task - vec * P2_CARDS;
+      const float* tv = t + vec * stride;
+#pragma unroll
+      for (int i = 0; i < 13; ++i) {
+        const int j = sub + 4 * i;
+        if (j < 51) {
+          const int x = j < c ? j : j + 1;  // partner card
+          const int lo = x < c ? x : c, hi = x < c ? c : x;
+          v += (double)tv[p2_combo_index(lo, hi)];
+        }
+      }
     }
-    v = p2_wave_sum(v);
-    if (lane == 0) cs[c] = v;
+    v += __shfl_xor(v, 1, P2_WAVE);
+    v += __shfl_xor(v, 2, P2_WAVE);
+    if (valid && sub == 0) cs[task] = v;
   }
-  __syncthreads();
-  if (threadIdx.x < 64) {
-    double v = threadIdx.x < P2_CARDS ? cs[threadIdx.x] : 0.0;
-    v = p2_wave_sum(v);
-    if (threadIdx.x == 0) *s_out = 0.5 * v;  // every combo is counted under both of its cards
-  }
-  __syncthreads();
+  p2_sync_lds();
+}
+
+// Total mass of a vector from its 52 card sums (every combo is counted under both of its
+// cards).  Wave-level: every lane of every wave gets the value; no barrier.
+__device__ __forceinline__ double card_total(const double* cs52) {
+  const int lane = threadIdx.x & 63;
+  const double x = lane < P2_CARDS ? cs52[lane] : 0.0;
+  return 0.5 * p2_wave_sum(x);
 }
 
 __device__ __forceinline__ float unblocked_at(const float* t, const double* cs, double S, int h) {
@@ -57,14 +75,13 @@ __global__ __launch_bounds__(UB_BLOCK) void unblocked_mass_kernel(const float* _
                                                                    float* __restrict__ out) {
   __shared__ __align__(8) float t[P2_H + 2];
   __shared__ double cs[P2_CARDS];
-  __shared__ double S;
   const int64_t r = blockIdx.x;
   int64_t src = r;
   if (to_act) src = 2 * r + ((int)to_act[r] ^ flip);
   load_row(target + src * P2_H, t);
-  __syncthreads();
-  card_sums(t, cs, &S);
-  const double s = S;
+  p2_sync_lds();
+  card_sums_multi(t, 0, 1, cs);
+  const double s = card_total(cs);
   float2* o2 = p2_row2(out, r);
   for (int i = threadIdx.x; i < P2_HPAIRS; i += UB_BLOCK) {
     float2 v;
@@ -79,18 +96,19 @@ __global__ __launch_bounds__(UB_BLOCK) void unblocked_ratio_kernel(const float* 
                                                                     const float* __restrict__ denom,
                                                                     const int64_t* __restrict__ parent_index,
                                                                     float eps, float* __restrict__ out) {
-  __shared__ __align__(8) float tn[P2_H + 2];
-  __shared__ __align__(8) float td[P2_H + 2];
-  __shared__ double csn[P2_CARDS], csd[P2_CARDS];
-  __shared__ double Sn, Sd;
+  __shared__ __align__(8) float tt[2][P2_H + 2];  // numerator row, denominator row
+  __shared__ double cs2[2 * P2_CARDS];
+  float* tn = tt[0];
+  float* td = tt[1];
+  const double* csn = cs2;
+  const double* csd = cs2 + P2_CARDS;
   const int64_t c = blockIdx.x;
   const int64_t p = parent_index ? parent_index[c] : c;
   load_row(numer + c * P2_H, tn);
   load_row(denom + p * P2_H, td);
-  __syncthreads();
-  card_sums(tn, csn, &Sn);
-  card_sums(td, csd, &Sd);
-  const double sn = Sn, sd = Sd;
+  p2_sync_lds();
+  card_sums_multi(tt[0], P2_H + 2, 2, cs2);
+  const double sn = card_total(csn), sd = card_total(csd);
   float2* o2 = p2_row2(out, c);
   for (int i = threadIdx.x; i < P2_HPAIRS; i += UB_BLOCK) {
     float r[2];

@@ -48,7 +48,8 @@ _NODE_SHOWDOWN, _NODE_DONE = 1, 2
 
 class _IterArgs(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in (
-        "child_offsets", "child_count", "to_act", "node_flags", "root_node_offsets", "root_nodes", "t_sample",
+        "child_offsets", "child_count", "to_act", "node_flags", "root_parent_offsets", "root_parents",
+        "root_showdown_offsets", "root_showdown_nodes", "t_sample",
         "allowed", "allowed_prob", "tables", "potential", "scale", "policy", "policy_avg", "policy_sample", "cum",
         "wsum", "beliefs", "beliefs_avg", "reach", "reach_avg", "latest", "values_avg", "scratch", "fscal", "iscal")]
 
@@ -190,10 +191,17 @@ class HipSparseCFREvaluator:
         flags[tree.showdown_mask] |= _NODE_SHOWDOWN
         flags[st["done"]] |= _NODE_DONE
         self._node_flags = self._t(flags)
-        order = np.argsort(tree.root_index, kind="stable").astype(np.int64)  # rows grouped by root, ascending
-        counts = np.bincount(tree.root_index, minlength=N)
-        self._root_nodes = self._t(order)
-        self._root_node_offsets = self._t(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64))
+        def per_root(mask):
+            """Rows selected by ``mask`` grouped by root (ascending inside a root) + offsets [N+1]."""
+            rows = np.nonzero(mask)[0]
+            roots_of = tree.root_index[rows]
+            order = np.argsort(roots_of, kind="stable")
+            counts = np.bincount(roots_of, minlength=N)
+            return (self._t(rows[order].astype(np.int64)),
+                    self._t(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)))
+
+        self._root_parents, self._root_parent_offsets = per_root(tree.child_count > 0)
+        self._root_showdown_nodes, self._root_showdown_offsets = per_root(tree.showdown_mask)
         self._max_children = int(tree.child_count.max()) if T else 1
         self._has_model_leaves = bool(model_mask.any())
         self._iter_args = None
@@ -461,7 +469,9 @@ class HipSparseCFREvaluator:
         a = _IterArgs()
         p = _lib.ptr
         a.child_offsets, a.child_count, a.to_act = p(self.child_offsets), p(self.child_count), p(self.env.to_act)
-        a.node_flags, a.root_node_offsets, a.root_nodes = p(self._node_flags), p(self._root_node_offsets), p(self._root_nodes)
+        a.node_flags = p(self._node_flags)
+        a.root_parent_offsets, a.root_parents = p(self._root_parent_offsets), p(self._root_parents)
+        a.root_showdown_offsets, a.root_showdown_nodes = p(self._root_showdown_offsets), p(self._root_showdown_nodes)
         a.t_sample, a.allowed, a.allowed_prob = p(self.t_sample), p(self.allowed_hands), p(self.allowed_hands_prob)
         a.tables = p(self.hand_rank_data) if self.hand_rank_data is not None else None
         a.potential, a.scale = p(self._potential_all), p(self.env.scale)
