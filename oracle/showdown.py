@@ -20,7 +20,9 @@ is what torch's CPU cumsum does for float32 input.
 
 Pinned by: brute force over all hero x villain pairs (several boards from the
 reference's tests), all-tie board -> 0, delta villain -> +-potential,
-villain-range scale invariance under renormalisation, |EV| <= potential/scale.
+zero-sum identity over compatible pairs, |EV| <= potential/scale.  The formula takes
+the villain range as normalised and zero on board-blocked hands (the constant 1 in
+``den``), as the evaluator guarantees; it is not invariant to rescaling the range.
 """
 from __future__ import annotations
 
