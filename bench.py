@@ -31,6 +31,10 @@ H = 1326
 BYTES_PER_NODE_ITER = 29 * H * 4          # 17 vectors written + 12 read per node per iteration
 HBM_PEAK_GBS = 8000.0
 TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2)}
+# HBM bytes per launch of the iteration kernel from two rocprofv3 --pmc passes (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy): an offline
+# measurement per workload, quoted in the JSON line; None where no counter run exists.
+MEASURED_TRAFFIC_BYTES = {("depth2", 4096): 6.03e9 + 6.81e9}
 
 
 def synth_roots(n: int, seed: int):
@@ -212,7 +216,8 @@ def main() -> None:
                    "roots": args.roots, "nodes_per_root": nodes_per_root, "total_nodes": ev.total_nodes,
                    "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots)),
                      "kernel": "cfr_iteration_kernel", "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes},
     }

@@ -1,0 +1,137 @@
+"""Per-operator timings on the workloads of the reference's three micro-benchmarks
+(benchmarks/bench_fused_cfr_triton.py:53-351, bench_rules_triton.py:25-126,
+bench_calculate_unblocked_mass.py:24-60), through this package's drop-in functions.
+
+    python -m poker2_amd.bench_ops [--repeats 100] [--json]
+
+Each line: mean time per call (HIP events around `repeats` calls after 10 warm-ups), the
+algorithmic bytes of the call (every input read once, every output written once) and the
+resulting GB/s.  Inputs are seeded and resident in HBM before timing.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+
+import numpy as np
+import torch
+
+from . import fused_cfr_hip as F
+from . import rules_hip as R
+from .card_utils import hand_combos_tensor
+
+H = 1326
+
+
+def timed(fn, repeats: int, warmup: int = 10) -> float:
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(repeats):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / repeats * 1e-3
+
+
+def random_hands(n: int, seed: int) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return np.argsort(rng.random((n, 52)), axis=1)[:, :7]
+
+
+def cases(repeats: int):
+    dev = torch.device("cuda")
+    g = torch.Generator(device="cpu").manual_seed(42)
+
+    # --- DCFR discount + accumulate, [10 000, 1326] (bench_fused_cfr_triton.py:53-121)
+    for rows in (10_000, 86_016):
+        cum = torch.randn(rows, H, generator=g).to(dev)
+        wsum = (torch.rand(rows, H, generator=g) * 5).to(dev)
+        reg = (torch.randn(rows, H, generator=g) * 0.1).to(dev)
+        yield (f"dcfr_update rows={rows}", 5 * rows * H * 4,
+               lambda cum=cum, wsum=wsum, reg=reg: F.fused_dcfr_update_(cum, wsum, reg, 7, F.CFRType.discounted, 1.5, 0.0, False))
+
+    # --- sibling sum / parent sum + divide, 30 000 parents x ~5 children (:193-326)
+    parents = 30_000
+    rng = np.random.default_rng(42)
+    child_count = torch.from_numpy(np.clip(5 + rng.integers(-1, 2, parents), 1, None)).to(dev)
+    n_children = int(child_count.sum())
+    child_offsets = (torch.cumsum(child_count, 0) - child_count + parents).contiguous()
+    parent_index = torch.arange(parents, device=dev).repeat_interleave(child_count)
+    values = torch.zeros(parents + n_children, H, device=dev)
+    values[parents:] = torch.rand(n_children, H, device=dev)
+    yield ("sibling_sum parents=30000", 2 * n_children * H * 4,
+           lambda: F.fused_sibling_sum(values, child_offsets, child_count, parents, n_children))
+    pos = torch.rand(n_children, H, device=dev)
+    fallback = torch.rand(n_children, H, device=dev)
+    out = torch.empty_like(pos)
+    full_pos = torch.zeros(parents + n_children, H, device=dev)
+    full_pos[parents:] = pos
+
+    def parent_sum_then_divide():
+        ps = F.fused_parent_sum(full_pos, child_offsets, child_count)
+        F.fused_divide_by_parent_sum_(pos, fallback, ps, parent_index, out)
+    yield ("parent_sum + divide parents=30000", (4 * n_children + 2 * parents) * H * 4, parent_sum_then_divide)
+
+    # --- unblocked mass (bench_calculate_unblocked_mass.py:24-42, bench_fused_cfr_triton.py:329-351)
+    for rows in (10_000, 400_000):
+        t = torch.rand(rows, H, generator=g)
+        t = (t / t.sum(-1, keepdim=True)).to(dev)
+        yield (f"unblocked_mass rows={rows}", 2 * rows * H * 4, lambda t=t: F.unblocked_mass_triton(t))
+        del t
+
+    # --- 7-card ranker (bench_rules_triton.py:25-126)
+    for n in (1024, 8192, 65536, 1 << 20):
+        a, b = random_hands(n, 7 + n), random_hands(n, 8 + n)
+        cards = torch.from_numpy(np.stack([a, b], 1).astype(np.int16)).to(dev)
+        planes = torch.zeros(n, 2, 4, 13, dtype=torch.bool, device=dev)
+        idx = torch.arange(n, device=dev)[:, None]
+        for p in range(2):
+            c = cards[:, p].long()
+            planes[idx, p, c // 13, c % 13] = True
+        yield (f"compare_7 planes n={n}", n * (104 + 4), lambda planes=planes: R.compare_7_single_batch_triton(planes))
+        yield (f"compare_7 cards(int16) n={n}", n * (28 + 4),
+               lambda cards=cards: R.compare_7_cards_single_batch_triton(cards))
+        one = cards[:, 0].to(torch.int8).contiguous()
+        yield (f"rank_7 cards(int8) n={n}", n * (7 + 4), lambda one=one: R.rank_7_cards_single_batch_triton(one))
+
+    # --- river showdown, 4096 public states
+    m = 4096
+    boards = torch.from_numpy(np.argsort(rng.random((m, 52)), axis=1)[:, :5].astype(np.int64)).to(dev)
+    combos = hand_combos_tensor(dev)
+    on_board = torch.zeros(m, 52, dtype=torch.bool, device=dev)
+    on_board.scatter_(1, boards, True)
+    allowed = ~(on_board[:, combos[:, 0]] | on_board[:, combos[:, 1]])
+    bel = torch.from_numpy(rng.gamma(0.5, size=(m, 2, H)).astype(np.float32)).to(dev) * allowed[:, None, :]
+    bel = bel / bel.sum(-1, keepdim=True)
+    yield ("rank_hands (tables) boards=4096", m * (5 * 8 + R.showdown_table_bytes()),
+           lambda: R.build_showdown_tables(boards))
+    tables = R.build_showdown_tables(boards)
+    pot = torch.ones(m, 2, device=dev)
+    sc = torch.ones(m, device=dev)
+    res = torch.empty_like(bel)
+    yield ("showdown_value_both states=4096", 4 * m * H * 4,
+           lambda: R.showdown_value_both(bel, tables, pot, sc, out=res))
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--repeats", type=int, default=100)
+    ap.add_argument("--json", action="store_true")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("bench_ops needs a GPU (the product path has no CPU fallback)")
+    rows = []
+    for name, nbytes, fn in cases(args.repeats):
+        sec = timed(fn, args.repeats)
+        rows.append({"op": name, "us": sec * 1e6, "algorithmic_bytes": nbytes, "GBps": nbytes / sec / 1e9})
+        if not args.json:
+            print(f"{name:40s} {sec * 1e6:10.1f} us  {nbytes / 1e6:10.1f} MB  {nbytes / sec / 1e9:8.1f} GB/s", flush=True)
+    if args.json:
+        print(json.dumps(rows))
+
+
+if __name__ == "__main__":
+    main()
