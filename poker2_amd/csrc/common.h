@@ -66,6 +66,17 @@ __device__ __forceinline__ float p2_wave_scan_incl(float v) {
 }
 __device__ __forceinline__ float p2_wave_scan_incl(float v, int /*lane*/) { return p2_wave_scan_incl(v); }
 
+// Two independent scans in lockstep: each DPP step of one fills the two wait states the other
+// needs between writing a register and reading it through DPP.
+__device__ __forceinline__ void p2_wave_scan_incl2(float& a, float& b) {
+  a += p2_dpp0<0x111, 0xF>(a); b += p2_dpp0<0x111, 0xF>(b);
+  a += p2_dpp0<0x112, 0xF>(a); b += p2_dpp0<0x112, 0xF>(b);
+  a += p2_dpp0<0x114, 0xF>(a); b += p2_dpp0<0x114, 0xF>(b);
+  a += p2_dpp0<0x118, 0xF>(a); b += p2_dpp0<0x118, 0xF>(b);
+  a += p2_dpp0<0x142, 0xA>(a); b += p2_dpp0<0x142, 0xA>(b);
+  a += p2_dpp0<0x143, 0xC>(a); b += p2_dpp0<0x143, 0xC>(b);
+}
+
 __device__ __forceinline__ float p2_wave_sum(float v) {
   v = p2_wave_scan_incl(v);
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));

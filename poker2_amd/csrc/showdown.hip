@@ -234,24 +234,35 @@ struct ShowdownRegs {
   uint32_t clist[13];      // lane j < 51: sorted position of the j-th weakest combo of card wave + 4*i
 };
 
-__device__ __forceinline__ void showdown_load_regs(const uint8_t* __restrict__ tab, ShowdownRegs& R) {
-  const uint16_t* perm = reinterpret_cast<const uint16_t*>(tab + SD_OFF_PERM);
-  const uint32_t* lr = reinterpret_cast<const uint32_t*>(tab + SD_OFF_LR);
-  const uint32_t* cidx = reinterpret_cast<const uint32_t*>(tab + SD_OFF_CIDX);
+struct __attribute__((packed, aligned(4))) SdU3 { uint32_t x, y, z; };
+
+// Table slice of this lane's six consecutive sorted positions.  1326 = 221 * 6, so a lane is
+// either entirely inside the table or entirely past its end and the 12 / 24 / 24 bytes it owns
+// are fetched as three-dword loads (the table sections are 4-byte aligned).
+// `ab_lds` (optional): a | b << 8 per combo, staged in LDS by the caller; null reads the
+// constant table in global memory instead.
+__device__ __forceinline__ void showdown_load_regs(const uint8_t* __restrict__ tab, ShowdownRegs& R,
+                                                   const uint16_t* ab_lds = nullptr) {
   const uint16_t* clist = reinterpret_cast<const uint16_t*>(tab + SD_OFF_CLIST);
-  const int k0 = threadIdx.x * SD_PPT;
+  const bool ok = threadIdx.x * SD_PPT < P2_H;
+  if (ok) {
+    const SdU3 pm = *reinterpret_cast<const SdU3*>(tab + SD_OFF_PERM + threadIdx.x * (SD_PPT * 2));
+    const SdU3* lr = reinterpret_cast<const SdU3*>(tab + SD_OFF_LR + threadIdx.x * (SD_PPT * 4));
+    const SdU3* cx = reinterpret_cast<const SdU3*>(tab + SD_OFF_CIDX + threadIdx.x * (SD_PPT * 4));
+    const SdU3 l0 = lr[0], l1 = lr[1], c0 = cx[0], c1 = cx[1];
+    R.perm[0] = pm.x & 0xFFFFu; R.perm[1] = pm.x >> 16;
+    R.perm[2] = pm.y & 0xFFFFu; R.perm[3] = pm.y >> 16;
+    R.perm[4] = pm.z & 0xFFFFu; R.perm[5] = pm.z >> 16;
+    R.lr[0] = l0.x; R.lr[1] = l0.y; R.lr[2] = l0.z; R.lr[3] = l1.x; R.lr[4] = l1.y; R.lr[5] = l1.z;
+    R.cidx[0] = c0.x; R.cidx[1] = c0.y; R.cidx[2] = c0.z; R.cidx[3] = c1.x; R.cidx[4] = c1.y; R.cidx[5] = c1.z;
+  } else {
 #pragma unroll
-  for (int i = 0; i < SD_PPT; ++i) {
-    const int k = k0 + i;
-    const bool ok = k < P2_H;
-    R.perm[i] = ok ? perm[k] : 0xFFFFFFFFu;
-    R.lr[i] = ok ? lr[k] : 0u;
-    R.cidx[i] = ok ? cidx[k] : 0u;
+    for (int i = 0; i < SD_PPT; ++i) { R.perm[i] = 0xFFFFFFFFu; R.lr[i] = 0u; R.cidx[i] = 0u; }
   }
 #pragma unroll
   for (int i = 0; i < SD_PPT; ++i) {
-    const int h = (R.perm[i] == 0xFFFFFFFFu) ? 0 : (int)(R.perm[i] & 0x7FFFu);
-    R.ab[i] = (uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8);
+    const int h = ok ? (int)(R.perm[i] & 0x7FFFu) : 0;
+    R.ab[i] = ab_lds ? (uint32_t)ab_lds[h] : ((uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8));
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -276,8 +287,9 @@ __device__ __forceinline__ void showdown_gather(const float* __restrict__ bel, c
 // by the board.  ev0 / ev1 may be s.v[0] / s.v[1] (dead by the time they are written).  Uses LDS
 // barriers only; the caller puts an LDS barrier before reading ev0 / ev1 and another before the
 // next call.
-__device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s,
-                                              float* ev0, float* ev1, float mul0, float mul1, float div) {
+// First half of showdown_eval: sorted ranges, their prefix and the per-card prefixes into LDS.
+// Ends with an LDS barrier.
+__device__ __forceinline__ void showdown_scans(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int k0 = threadIdx.x * SD_PPT;
   float local[2], incl[2];
@@ -305,19 +317,32 @@ __device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], cons
     }
   }
   // per-card prefixes: one wave scan per (player, card); this wave owns cards wave, wave+4, ...
+  // Both players' lists of a card share the positions, so they are scanned in lockstep.
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
-#pragma unroll
-    for (int i = 0; i < 13; ++i) {
-      const int c = wave + 4 * i;
-      const uint32_t pos = R.clist[i];
-      const float x = pos < (uint32_t)P2_H ? s.v[p][pos] : 0.f;
-      const float sc = p2_wave_scan_incl(x);
-      if (lane < 51) s.Pc[p][c][lane + 1] = sc;
-      if (lane == 0) s.Pc[p][c][0] = 0.f;
+  for (int i = 0; i < 13; ++i) {
+    const int c = wave + 4 * i;
+    const uint32_t pos = R.clist[i];
+    const bool in = pos < (uint32_t)P2_H;
+    float x0 = in ? s.v[0][pos] : 0.f;
+    float x1 = in ? s.v[1][pos] : 0.f;
+    p2_wave_scan_incl2(x0, x1);
+    if (lane < 51) {
+      s.Pc[0][c][lane + 1] = x0;
+      s.Pc[1][c][lane + 1] = x1;
+    }
+    if (lane == 0) {
+      s.Pc[0][c][0] = 0.f;
+      s.Pc[1][c][0] = 0.f;
     }
   }
   p2_sync_lds();
+}
+
+// Second half: six LDS reads per hand and player, EVs written in combo order to ev0 / ev1.
+__device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], const ShowdownRegs& R,
+                                                const ShowdownLds& s, float* ev0, float* ev1, float mul0, float mul1,
+                                                float div) {
+  const float r0 = mul0 / div, r1 = mul1 / div;  // potential / scale of the node, one division each
 #pragma unroll
   for (int i = 0; i < SD_PPT; ++i) {
     if (R.perm[i] == 0xFFFFFFFFu) continue;
@@ -338,44 +363,77 @@ __device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], cons
       const float tie = (PR - PL) - (aR - aL) - (bR - bL) + v0;
       float den = 1.0f - s.Pc[p][a][51] - s.Pc[p][b][51] + v0;
       den = fmaxf(den, 1e-8f);
+      // The kernel is VALU-issue bound and an IEEE division is about ten instructions, so both
+      // quotients share one hardware reciprocal and are corrected by one fused residual step
+      // each, which keeps x/x == 1 and 0/x == 0 exact (an all-tie board stays exactly zero).
       const bool valid = den > 1e-8f;
-      const float wp = valid ? win / den : 0.f;
-      const float tp = valid ? tie / den : 0.f;
+      const float inv = valid ? __builtin_amdgcn_rcpf(den) : 0.f;
+      float wp = win * inv, tp = tie * inv;
+      wp = __builtin_fmaf(__builtin_fmaf(-wp, den, win), inv, wp);
+      tp = __builtin_fmaf(__builtin_fmaf(-tp, den, tie), inv, tp);
       const float lp = valid ? 1.0f - wp - tp : 0.f;
       e[p] = (wp - lp) * keep;
     }
-    ev0[h] = e[0] * mul0 / div;
-    ev1[h] = e[1] * mul1 / div;
+    ev0[h] = e[0] * r0;
+    ev1[h] = e[1] * r1;
   }
+}
+
+__device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s,
+                                              float* ev0, float* ev1, float mul0, float mul1, float div) {
+  showdown_scans(vk, R, s);
+  showdown_finish(vk, R, s, ev0, ev1, mul0, mul1, div);
 }
 
 // out[n] = showdown EV of both players at node n.
 //   beliefs   [M,2,H]      range pair per node
 //   table_row [M] or null  row of `tables` to use for node n (null: row n)
 //   potential [M,2] float  chips won by player p if he wins; scale [M]
-__global__ __launch_bounds__(SD_BLOCK) void showdown_both_kernel(const float* __restrict__ beliefs,
-                                                                  const uint8_t* __restrict__ tables,
-                                                                  const int64_t* __restrict__ table_row,
-                                                                  const float* __restrict__ potential,
-                                                                  const float* __restrict__ scale,
-                                                                  float* __restrict__ out) {
+// Workgroups walk the nodes with a grid stride; the table slice of the next node is requested
+// before the scans of the current one and its ranges are gathered between the scans and the
+// final pass, so the two dependent global round trips of a node overlap the LDS work of the
+// previous one.
+__global__ __launch_bounds__(SD_BLOCK, 3) void showdown_both_kernel(const float* __restrict__ beliefs,
+                                                                     const uint8_t* __restrict__ tables,
+                                                                     const int64_t* __restrict__ table_row,
+                                                                     const float* __restrict__ potential,
+                                                                     const float* __restrict__ scale, int64_t m,
+                                                                     float* __restrict__ out) {
   __shared__ ShowdownLds s;
-  const int64_t n = blockIdx.x;
-  const int64_t row = table_row ? table_row[n] : n;
-  ShowdownRegs R;
-  showdown_load_regs(tables + row * SD_TABLE_BYTES, R);
-  // the EVs are written over the sorted ranges, which are dead once the card scans are done
-  float vk[2][SD_PPT];
-  showdown_gather(beliefs + n * 2 * P2_H, R, vk);
-  showdown_eval(vk, R, s, s.v[0], s.v[1], potential[2 * n], potential[2 * n + 1], scale[n]);
+  __shared__ uint16_t ab_lds[P2_H];
+  for (int h = threadIdx.x; h < P2_H; h += SD_BLOCK) ab_lds[h] = (uint16_t)(p2_combo.a[h] | (p2_combo.b[h] << 8));
   p2_sync_lds();
-  float2* o0 = p2_row2(out, n * 2);
-  float2* o1 = p2_row2(out, n * 2 + 1);
-  const float2* e0 = reinterpret_cast<const float2*>(s.v[0]);
-  const float2* e1 = reinterpret_cast<const float2*>(s.v[1]);
-  for (int i = threadIdx.x; i < P2_HPAIRS; i += SD_BLOCK) {
-    o0[i] = e0[i];
-    o1[i] = e1[i];
+  ShowdownRegs R, Rn;
+  float vk[2][SD_PPT], vkn[2][SD_PPT];
+  int64_t n = blockIdx.x;
+  if (n < m) {
+    showdown_load_regs(tables + (table_row ? table_row[n] : n) * SD_TABLE_BYTES, Rn, ab_lds);
+    showdown_gather(beliefs + n * 2 * P2_H, Rn, vkn);
+  }
+  for (; n < m; n += gridDim.x) {
+    R = Rn;
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int i = 0; i < SD_PPT; ++i) vk[p][i] = vkn[p][i];
+    const int64_t nn = n + gridDim.x;
+    const bool more = nn < m;
+    if (more) showdown_load_regs(tables + (table_row ? table_row[nn] : nn) * SD_TABLE_BYTES, Rn, ab_lds);
+    const float mul0 = potential[2 * n], mul1 = potential[2 * n + 1], div = scale[n];
+    showdown_scans(vk, R, s);
+    if (more) showdown_gather(beliefs + nn * 2 * P2_H, Rn, vkn);
+    // the EVs go over the sorted ranges, which are dead once the card scans are done
+    showdown_finish(vk, R, s, s.v[0], s.v[1], mul0, mul1, div);
+    p2_sync_lds();
+    float2* o0 = p2_row2(out, n * 2);
+    float2* o1 = p2_row2(out, n * 2 + 1);
+    const float2* e0 = reinterpret_cast<const float2*>(s.v[0]);
+    const float2* e1 = reinterpret_cast<const float2*>(s.v[1]);
+    for (int i = threadIdx.x; i < P2_HPAIRS; i += SD_BLOCK) {
+      o0[i] = e0[i];
+      o1[i] = e1[i];
+    }
+    p2_sync_lds();  // the next node overwrites s.v
   }
 }
 
@@ -403,8 +461,9 @@ int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64
   if (m < 0 || (m > 0 && (!beliefs || !tables || !potential || !scale || !out))) return P2_EINVAL;
   if (m == 0) return 0;
   if (!p2_aligned8(tables) || !p2_aligned4(beliefs) || !p2_aligned8(out)) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::showdown_both_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
-                     beliefs, tables, table_row, potential, scale, out);
+  const int64_t cap = 256 * 3;  // three resident workgroups (43 KB of LDS each) on each of the 256 CUs
+  hipLaunchKernelGGL(p2::showdown_both_kernel, dim3((unsigned)(m < cap ? m : cap)), dim3(p2::SD_BLOCK), 0,
+                     (hipStream_t)stream, beliefs, tables, table_row, potential, scale, m, out);
   P2_LAUNCH_CHECK();
   return 0;
 }
