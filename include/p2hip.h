@@ -68,6 +68,25 @@ int p2hip_showdown_setup(const void* boards, int elem_size, int64_t m, int mode,
 int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64_t* table_row,
                         const float* potential, const float* scale, int64_t m, float* out, void* stream);
 
+/* ---- single-card chance node around the leaf network --------------------------------- */
+
+/* For each of n public states (state i reads row root_indices[i] of pre_beliefs [*,2,H] and of
+ * board [*,5] int64, -1 = empty slot; root_indices NULL = identity) and every card c not on its
+ * board, in (i, c) ascending order: post_beliefs[s] = the ranges with the hands that hold c or
+ * a board card removed, renormalised per player (uniform over the allowed hands when the sum
+ * is <= 1e-12); board_samples[s] = the board with c in its first empty slot; root_lookup[s] = i.
+ * sample_offsets [n+1] int64 (device) = prefix sums of 52 - cards on board.  Replaces the
+ * expansion half of ChanceNodeHelper.single_card_chance_values,
+ * search/chance_node_helper.py:394-443. */
+int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
+                        const int64_t* sample_offsets, float* post_beliefs, int64_t* board_samples,
+                        int64_t* root_lookup, void* stream);
+
+/* expected[i] = mean of hand_values [S,2,H] over samples sample_offsets[i] .. sample_offsets[i+1]
+ * (index_add_ + divide of search/chance_node_helper.py:467-477). */
+int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, int64_t n, float* expected,
+                      void* stream);
+
 /* ---- unblocked (card-compatible) mass --------------------------------------------- */
 
 /* target [rows,H] -> out [rows,H] = max(S - cs[a] - cs[b] + t, 0).  Replaces

@@ -1,0 +1,187 @@
+// Single-card chance node around the leaf network: expansion of a public state's ranges over
+// every card that can come next, and the mean of the network's answers.
+//
+// Replaces the tensor program of ChanceNodeHelper.single_card_chance_values
+// (src/p2/search/chance_node_helper.py:360-479):
+//   expand : for every state i and every card c not on its board, in (i, c) ascending order,
+//            post[s][p][h] = pre[i][p][h] if h holds neither c nor a board card, else 0,
+//            renormalised per player (uniform over the allowed hands if the sum is <= 1e-12);
+//            board_samples[s] = board with c in the first empty slot; root_lookup[s] = i
+//            (:394-443)
+//   mean   : expected[i] = sum of hand_values over the samples of state i / their count
+//            (:467-477)
+// The per-sample sum of a player's masked range is T - cs[c] (T = total of the board-masked
+// range, cs[c] = its mass on hands holding c), so one card-sum pass per state serves all of
+// its 46-49 samples.  The expansion is a pure write stream (about 48 x 10.6 KB per state).
+#pragma once
+#include "common.h"
+#include "unblocked.hip"
+
+namespace p2 {
+
+constexpr int CH_BLOCK = 256;
+constexpr int CH_PPT = 3;  // float2 pairs per thread and vector
+static_assert(CH_BLOCK == UB_BLOCK, "card_sums_multi assumes the block size");
+
+__device__ __forceinline__ int chance_board(const int64_t* __restrict__ board5, int (&cards)[5], uint64_t& bits) {
+  int n = 0;
+  bits = 0ull;
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    const int64_t c = board5[j];
+    cards[j] = (int)c;
+    if (c >= 0 && c < P2_CARDS) {
+      bits |= 1ull << c;
+      ++n;
+    }
+  }
+  return n;
+}
+
+__global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __restrict__ pre_beliefs,
+                                                                  const int64_t* __restrict__ root_indices,
+                                                                  const int64_t* __restrict__ board,
+                                                                  const int64_t* __restrict__ sample_offsets,
+                                                                  float* __restrict__ post_beliefs,
+                                                                  int64_t* __restrict__ board_samples,
+                                                                  int64_t* __restrict__ root_lookup) {
+  __shared__ __align__(8) float t[2][P2_H + 2];
+  __shared__ double cs[2 * P2_CARDS];
+  const int64_t i = blockIdx.x;
+  const int64_t root = root_indices ? root_indices[i] : i;
+  int bcards[5];
+  uint64_t bits;
+  const int ncards = chance_board(board + root * 5, bcards, bits);
+
+  // this lane's hands: pairs k -> hands 2*idx, 2*idx+1 with idx = tid + k*256
+  float v[2][CH_PPT][2];
+  uint32_t ab[CH_PPT][2];
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    const bool in = idx < P2_HPAIRS;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int h = in ? 2 * idx + q : 0;
+      ab[k][q] = (uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8);
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      float2 x = make_float2(0.f, 0.f);
+      if (in) x = p2_row2(pre_beliefs, root * 2 + p)[idx];
+      const bool blocked0 = ((bits >> (ab[k][0] & 0xFFu)) | (bits >> (ab[k][0] >> 8))) & 1ull;
+      const bool blocked1 = ((bits >> (ab[k][1] & 0xFFu)) | (bits >> (ab[k][1] >> 8))) & 1ull;
+      v[p][k][0] = blocked0 ? 0.f : x.x;
+      v[p][k][1] = blocked1 ? 0.f : x.y;
+      if (in) reinterpret_cast<float2*>(t[p])[idx] = make_float2(v[p][k][0], v[p][k][1]);
+    }
+  }
+  p2_sync_lds();
+  card_sums_multi(t[0], P2_H + 2, 2, cs);
+  const double total0 = card_total(cs), total1 = card_total(cs + P2_CARDS);
+
+  const int remaining = P2_CARDS - ncards - 1;          // cards left for the hands of a sample
+  const float uniform = 1.0f / fmaxf((float)(remaining * (remaining - 1) / 2), 1.0f);
+  int64_t s = sample_offsets[i];
+  for (int c = 0; c < P2_CARDS; ++c) {
+    if ((bits >> c) & 1ull) continue;
+    const float sum0 = (float)(total0 - cs[c]);
+    const float sum1 = (float)(total1 - cs[P2_CARDS + c]);
+    const bool ok0 = sum0 > 1e-12f, ok1 = sum1 > 1e-12f;
+    const float inv0 = 1.0f / fmaxf(sum0, 1e-12f), inv1 = 1.0f / fmaxf(sum1, 1e-12f);
+    float2* o0 = p2_row2(post_beliefs, s * 2);
+    float2* o1 = p2_row2(post_beliefs, s * 2 + 1);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx >= P2_HPAIRS) continue;
+      float r0[2], r1[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const uint32_t a = ab[k][q] & 0xFFu, b = ab[k][q] >> 8;
+        const bool off = a == (uint32_t)c || b == (uint32_t)c;
+        const bool on_board = ((bits >> a) | (bits >> b)) & 1ull;
+        const float u = (off || on_board) ? 0.f : uniform;
+        r0[q] = ok0 ? (off ? 0.f : v[0][k][q] * inv0) : u;
+        r1[q] = ok1 ? (off ? 0.f : v[1][k][q] * inv1) : u;
+      }
+      o0[idx] = make_float2(r0[0], r0[1]);
+      o1[idx] = make_float2(r1[0], r1[1]);
+    }
+    if (threadIdx.x < 5) {
+      int64_t card = bcards[threadIdx.x];
+      if ((int)threadIdx.x == ncards) card = c;
+      board_samples[s * 5 + threadIdx.x] = card;
+    }
+    if (threadIdx.x == 0) root_lookup[s] = i;
+    ++s;
+  }
+}
+
+__global__ __launch_bounds__(CH_BLOCK) void chance_mean_kernel(const float* __restrict__ hand_values,
+                                                                const int64_t* __restrict__ sample_offsets,
+                                                                float* __restrict__ expected) {
+  const int64_t i = blockIdx.x;
+  const int64_t s0 = sample_offsets[i], s1 = sample_offsets[i + 1];
+  float2 acc[2][CH_PPT];
+#pragma unroll
+  for (int p = 0; p < 2; ++p)
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) acc[p][k] = make_float2(0.f, 0.f);
+  for (int64_t s = s0; s < s1; ++s) {
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const float2* row = p2_row2(hand_values, s * 2 + p);
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) {
+        const int idx = threadIdx.x + k * CH_BLOCK;
+        if (idx < P2_HPAIRS) {
+          const float2 x = row[idx];
+          acc[p][k].x += x.x;
+          acc[p][k].y += x.y;
+        }
+      }
+    }
+  }
+  const float count = fmaxf((float)(s1 - s0), 1.0f);
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    float2* o = p2_row2(expected, i * 2 + p);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx < P2_HPAIRS) o[idx] = make_float2(acc[p][k].x / count, acc[p][k].y / count);
+    }
+  }
+}
+
+}  // namespace p2
+
+extern "C" {
+
+int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
+                        const int64_t* sample_offsets, float* post_beliefs, int64_t* board_samples,
+                        int64_t* root_lookup, void* stream) {
+  if (n < 0) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!pre_beliefs || !board || !sample_offsets || !post_beliefs || !board_samples || !root_lookup) return P2_EINVAL;
+  if (!p2_aligned8(pre_beliefs) || !p2_aligned8(post_beliefs)) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::chance_expand_kernel, dim3((unsigned)n), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     pre_beliefs, root_indices, board, sample_offsets, post_beliefs, board_samples, root_lookup);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, int64_t n, float* expected,
+                      void* stream) {
+  if (n < 0) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!hand_values || !sample_offsets || !expected) return P2_EINVAL;
+  if (!p2_aligned8(hand_values) || !p2_aligned8(expected)) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)n), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     hand_values, sample_offsets, expected);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -6,6 +6,7 @@
 #include "showdown.hip"
 #include "cfr_ops.hip"
 #include "cfr_iter.hip"
+#include "chance.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

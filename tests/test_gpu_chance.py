@@ -1,0 +1,131 @@
+"""GPU parity of the single-card chance node (expansion + mean kernels and the
+ChanceNodeHelper mirror) against the oracle, on the cases of the reference's
+tests/test_chance_node_helper.py:426-590 and on seeded mixed-street inputs."""
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import chance as OCH
+from tests.helpers import random_boards
+
+pytestmark = pytest.mark.gpu
+H = 1326
+
+
+@pytest.fixture(scope="module")
+def K():
+    from poker2_amd import chance_node_helper as M
+    from poker2_amd import _lib
+    assert _lib.hip_is_available(), "libp2hip.so / GPU missing"
+    return M
+
+
+def inputs(rng, b, ks):
+    boards = np.full((b, 5), -1, dtype=np.int64)
+    for i in range(b):
+        k = ks[i % len(ks)]
+        boards[i, :k] = random_boards(rng, 1, k)[0] if k else []
+    pre = rng.gamma(0.5, size=(b, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    return boards, pre
+
+
+def test_expand_matches_oracle_mixed_streets(K):
+    rng = np.random.default_rng(5)
+    boards, pre = inputs(rng, 9, [4, 3, 4, 0])
+    pre[1, 0] = 0.0                      # dead range -> uniform fallback on every sample
+    pre[2, 1] = 0.0
+    pre[2, 1, 7] = 1.0                   # delta range -> dead on the samples that block it
+    roots = np.array([8, 1, 2, 5, 0, 3])
+    post, bs, lookup, offsets = K.chance_expand(torch.from_numpy(pre).cuda(), torch.from_numpy(roots).cuda(),
+                                                torch.from_numpy(boards).cuda())
+    e_post, e_bs, e_lookup = OCH.expand(pre[roots], boards[roots])
+    assert torch.equal(bs.cpu(), torch.from_numpy(e_bs))                 # integer outputs: exact
+    assert torch.equal(lookup.cpu(), torch.from_numpy(e_lookup))
+    assert offsets.cpu().tolist() == np.concatenate([[0], np.cumsum(np.bincount(e_lookup))]).tolist()
+    got = post.cpu().numpy()
+    assert ((got == 0) == (e_post == 0)).all()                           # the mask is exact
+    np.testing.assert_allclose(got, e_post, rtol=1e-5, atol=1e-9)        # float32 tolerance 1e-5 relative
+
+
+def test_mean_matches_oracle_and_ragged_counts(K):
+    rng = np.random.default_rng(6)
+    counts = np.array([48, 49, 0, 52, 1])
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    hv = rng.standard_normal((int(offsets[-1]), 2, H)).astype(np.float32)
+    got = K.chance_mean(torch.from_numpy(hv).cuda(), torch.from_numpy(offsets).cuda()).cpu().numpy()
+    lookup = np.repeat(np.arange(5), counts)
+    exp = OCH.mean_by_root(hv, lookup, 5)
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-6)
+    assert not got[2].any()
+
+
+class EchoModel:
+    def eval(self):
+        pass
+
+    def __call__(self, f):
+        return SimpleNamespace(hand_values=f.beliefs.view(-1, 2, H))
+
+
+class BoardModel:
+    """Values from the board's rank sum only (tests/test_chance_node_helper.py:78-117)."""
+
+    def eval(self):
+        pass
+
+    def __call__(self, f):
+        ranks = torch.where(f.board >= 0, (f.board % 13).float(), torch.zeros_like(f.board, dtype=torch.float32))
+        v = ranks.sum(dim=1, keepdim=True) % H
+        return SimpleNamespace(hand_values=v.unsqueeze(1).expand(-1, 2, H).contiguous())
+
+
+@pytest.mark.parametrize("model_name", ["echo", "board"])
+def test_helper_matches_oracle(K, model_name):
+    rng = np.random.default_rng(8)
+    b = 7
+    boards, pre = inputs(rng, b, [4, 4, 3])
+    roots = np.array([6, 0, 3, 4])
+    dev = torch.device("cuda")
+    model = EchoModel() if model_name == "echo" else BoardModel()
+    helper = K.ChanceNodeHelper(dev, torch.float32, 2, model, autocast_dtype=None)
+    feats = K.MLPFeatures(context=torch.zeros(b, 1, device=dev), street=torch.zeros(b, dtype=torch.long, device=dev),
+                          to_act=torch.zeros(b, dtype=torch.long, device=dev),
+                          board=torch.from_numpy(boards).to(dev), beliefs=torch.zeros(b, 2 * H, device=dev))
+    got = helper.single_card_chance_values(torch.from_numpy(roots).to(dev), feats, torch.from_numpy(pre).to(dev),
+                                           torch.from_numpy(boards).to(dev))
+
+    def np_model(context, street, to_act, board, beliefs):
+        if model_name == "echo":
+            return beliefs.reshape(-1, 2, H)
+        v = (np.where(board >= 0, board % 13, 0).sum(axis=1) % H).astype(np.float32)
+        return np.broadcast_to(v[:, None, None], (board.shape[0], 2, H))
+    exp = OCH.single_card_chance_values(roots, np.zeros((b, 1)), np.zeros(b), np.zeros(b), pre, boards, np_model)
+    assert got.shape == (4, 2, H) and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=1e-7)
+
+
+def test_helper_edge_cases(K):
+    dev = torch.device("cuda")
+    helper = K.ChanceNodeHelper(dev, torch.float32, 2, EchoModel(), autocast_dtype=None)
+    empty = K.MLPFeatures(context=torch.zeros(0, 1, device=dev), street=torch.zeros(0, dtype=torch.long, device=dev),
+                          to_act=torch.zeros(0, dtype=torch.long, device=dev),
+                          board=torch.zeros(0, 5, dtype=torch.long, device=dev), beliefs=torch.zeros(0, 2 * H, device=dev))
+    out = helper.single_card_chance_values(torch.zeros(0, dtype=torch.long, device=dev), empty,
+                                           torch.zeros(0, 2, H, device=dev), torch.zeros(0, 5, dtype=torch.long, device=dev))
+    assert out.shape == (0, 2, H)
+    full = torch.arange(5, device=dev)[None]                 # a river board has no chance card left
+    with pytest.raises(ValueError):
+        K.chance_expand(torch.rand(1, 2, H, device=dev), torch.zeros(1, dtype=torch.long, device=dev), full)
+    with pytest.raises(NotImplementedError):
+        helper.flop_chance_values()
+    # the fixed-count fast path gives the same samples
+    rng = np.random.default_rng(9)
+    boards, pre = inputs(rng, 3, [4])
+    a = K.chance_expand(torch.from_numpy(pre).cuda(), torch.arange(3).cuda(), torch.from_numpy(boards).cuda())
+    b = K.chance_expand(torch.from_numpy(pre).cuda(), torch.arange(3).cuda(), torch.from_numpy(boards).cuda(),
+                        cards_on_board=4)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)

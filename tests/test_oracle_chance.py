@@ -1,0 +1,106 @@
+"""CPU: pins the oracle's restatement of the single-card chance node
+(src/p2/search/chance_node_helper.py:360-479)."""
+import numpy as np
+
+from oracle import cards as OC
+from oracle import chance as OCH
+from tests.helpers import random_boards
+
+H = 1326
+
+
+def setup(rng, b, k):
+    boards = np.full((b, 5), -1, dtype=np.int64)
+    boards[:, :k] = random_boards(rng, b, k)
+    pre = rng.gamma(0.5, size=(b, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    return boards, pre
+
+
+def test_expand_against_per_sample_loop():
+    rng = np.random.default_rng(0)
+    boards, pre = setup(rng, 3, 4)
+    pre[1, 0] = 0.0                         # a dead range: every sample of it falls back to uniform
+    pre[2, 1, :] = 0.0
+    pre[2, 1, OC.combo_index(0, 1)] = 1.0   # a delta range: dead only on samples that deal card 0 or 1
+    post, board_samples, root_lookup = OCH.expand(pre, boards)
+    cm = OC.hand_combos()
+    s = 0
+    for i in range(3):
+        for c in range(52):
+            if c in boards[i]:
+                continue
+            assert root_lookup[s] == i
+            assert list(board_samples[s]) == list(boards[i, :4]) + [c]
+            dead = set(boards[i, :4].tolist()) | {c}
+            ok = np.array([cm[h, 0] not in dead and cm[h, 1] not in dead for h in range(H)])
+            assert ok.sum() == 47 * 46 // 2
+            for p in range(2):
+                x = np.where(ok, pre[i, p].astype(np.float64), 0.0)
+                exp = x / x.sum() if x.sum() > 1e-12 else ok / ok.sum()
+                np.testing.assert_allclose(post[s, p], exp, rtol=2e-6, atol=1e-9)
+            s += 1
+    assert s == post.shape[0] == 3 * 48
+
+
+def test_sample_counts_and_order_for_mixed_streets():
+    rng = np.random.default_rng(1)
+    boards = np.full((4, 5), -1, dtype=np.int64)
+    boards[0, :3] = [5, 17, 40]
+    boards[1, :4] = [0, 1, 2, 3]
+    boards[2, :3] = [51, 50, 49]
+    pre = rng.random((4, 2, H)).astype(np.float32)
+    post, board_samples, root_lookup = OCH.expand(pre, boards)
+    assert np.bincount(root_lookup).tolist() == [49, 48, 49, 52]
+    assert (np.diff(root_lookup) >= 0).all()
+    for i, k in enumerate([3, 4, 3, 0]):
+        dealt = board_samples[root_lookup == i][:, k]
+        assert (np.diff(dealt) > 0).all() and not set(dealt) & set(boards[i])
+    np.testing.assert_allclose(post.sum(-1), 1.0, atol=1e-5)
+
+
+def test_closed_forms_echo_and_board_models():
+    rng = np.random.default_rng(2)
+    boards, pre = setup(rng, 5, 4)
+    roots = np.array([4, 0, 2])
+    ctx = np.zeros((5, 1), np.float32)
+    zeros = np.zeros(5, np.int64)
+
+    def echo(context, street, to_act, board, beliefs):
+        return beliefs.reshape(-1, 2, H)
+    got = OCH.single_card_chance_values(roots, ctx, zeros, zeros, pre, boards, echo)
+    onehot = OC.combo_onehot()
+    for j, r in enumerate(roots):
+        acc = np.zeros((2, H))
+        for c in range(52):
+            if c in boards[r]:
+                continue
+            dead = np.zeros(52, bool)
+            dead[boards[r, :4]] = True
+            dead[c] = True
+            ok = ~(onehot & dead[None, :]).any(axis=1)
+            x = pre[r].astype(np.float64) * ok
+            acc += x / x.sum(-1, keepdims=True)
+        np.testing.assert_allclose(got[j], acc / 48, rtol=1e-5, atol=1e-8)
+    # ranges sum to one, so does their mean; a hand that holds a dealt card contributes 0 there
+    np.testing.assert_allclose(got.sum(-1), 1.0, atol=1e-5)
+
+    def board_rank_sum(context, street, to_act, board, beliefs):
+        v = (np.where(board >= 0, board % 13, 0).sum(axis=1) % H).astype(np.float32)
+        return np.broadcast_to(v[:, None, None], (board.shape[0], 2, H))
+    got = OCH.single_card_chance_values(roots, ctx, zeros, zeros, pre, boards, board_rank_sum)
+    for j, r in enumerate(roots):
+        base = (boards[r, :4] % 13).sum()
+        exp = np.mean([(base + c % 13) % H for c in range(52) if c not in boards[r]])
+        np.testing.assert_allclose(got[j], exp, rtol=1e-6)
+
+
+def test_empty_input_and_shapes():
+    out = OCH.single_card_chance_values(np.zeros(0, np.int64), np.zeros((0, 1)), np.zeros(0), np.zeros(0),
+                                        np.zeros((0, 2, H), np.float32), np.zeros((0, 5), np.int64), None)
+    assert out.shape == (0, 2, H)
+    rng = np.random.default_rng(3)
+    boards, pre = setup(rng, 4, 4)
+    out = OCH.single_card_chance_values(np.arange(4), np.zeros((4, 1)), np.zeros(4), np.zeros(4), pre, boards,
+                                        lambda c, s, t, b, x: np.zeros((b.shape[0], 2, H), np.float32))
+    assert out.shape == (4, 2, H) and out.dtype == np.float32 and not out.any()
