@@ -612,7 +612,7 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max
   if (n_roots == 0) return 0;
   const P2HipIterArgs& h = *host_args;
   const void* required[] = {h.child_offsets, h.child_count, h.to_act, h.node_flags, h.root_parent_offsets, h.root_parents,
-                            h.root_showdown_offsets, h.root_showdown_nodes,
+                            h.root_showdown_offsets,  // root_showdown_nodes is empty (null) without showdown rows
                             h.t_sample, h.allowed, h.allowed_prob, h.potential, h.scale, h.policy, h.policy_avg,
                             h.policy_sample, h.cum, h.wsum, h.beliefs, h.beliefs_avg, h.reach, h.reach_avg, h.latest,
                             h.values_avg, h.scratch, h.fscal, h.iscal};

@@ -1,0 +1,112 @@
+"""Leaf value networks for the evaluator and the chance node in front of them.
+
+The evaluator asks its ``model`` for ``leaf_values(beliefs[K,2,1326], node_rows[K], evaluator)``.
+``ChanceLeafModel`` answers with a PyTorch network: leaves in the middle of a betting round
+are evaluated on their own board; leaves where the round has ended and a card is still to
+come are expanded over every card that can come next (blocker masking, renormalisation,
+network, mean — the semantics of ``ChanceNodeHelper.single_card_chance_values``,
+src/p2/search/chance_node_helper.py:360-479).  The network stays ordinary PyTorch; only the
+expansion and the mean are HIP kernels.
+
+``RangeBoardMLP`` is the network of the turn benchmark configuration: input 2 x 1326 ranges +
+52-dim board one-hot, three hidden ReLU layers, output 2 x 1326; orthogonal initialisation with
+zero biases as in src/p2/models/mlp/rebel_ffn.py:139-148.
+"""
+from __future__ import annotations
+
+from types import SimpleNamespace
+
+import numpy as np
+import torch
+
+from .card_utils import NUM_HANDS
+from .chance_node_helper import ChanceNodeHelper, MLPFeatures
+
+
+class RangeBoardMLP(torch.nn.Module):
+    def __init__(self, hidden: int = 1536, layers: int = 3, seed: int = 42) -> None:
+        super().__init__()
+        dims = [2 * NUM_HANDS + 52] + [hidden] * layers + [2 * NUM_HANDS]
+        self.linears = torch.nn.ModuleList(torch.nn.Linear(a, b) for a, b in zip(dims[:-1], dims[1:]))
+        gen = torch.Generator().manual_seed(seed)
+        for lin in self.linears:
+            torch.nn.init.orthogonal_(lin.weight, generator=gen)
+            torch.nn.init.zeros_(lin.bias)
+
+    def forward(self, features: MLPFeatures) -> SimpleNamespace:
+        board = features.board
+        onehot = torch.zeros(board.shape[0], 53, dtype=features.beliefs.dtype, device=board.device)
+        onehot.scatter_(1, torch.where(board >= 0, board, torch.full_like(board, 52)), 1.0)
+        x = torch.cat([features.beliefs, onehot[:, :52]], dim=1)
+        for lin in self.linears[:-1]:
+            x = torch.relu(lin(x))
+        x = self.linears[-1](x)
+        return SimpleNamespace(hand_values=x.view(-1, 2, NUM_HANDS))
+
+
+class ChanceLeafModel:
+    """Evaluator leaf protocol on top of a value network and the single-card chance node."""
+
+    def __init__(self, net, device, *, enforce_zero_sum: bool = False, autocast_dtype: torch.dtype | None = None,
+                 max_samples_per_call: int = 1 << 19) -> None:
+        self.net = net
+        self.device = torch.device(device)
+        self.enforce_zero_sum = enforce_zero_sum
+        self.autocast_dtype = autocast_dtype
+        self.max_samples_per_call = int(max_samples_per_call)
+        self.helper = ChanceNodeHelper(self.device, torch.float32, 2, net, autocast_dtype=autocast_dtype)
+        self._plan_for = None
+        self._plan = None
+
+    def _make_plan(self, rows: torch.Tensor, ev):
+        """Static split of the evaluator's model rows (the tree does not change between iterations)."""
+        r = rows.cpu().numpy()
+        tree = ev.tree
+        board = tree.board[tree.root_index[r]]
+        on_board = (board >= 0).sum(axis=1)
+        chance = tree.new_street_mask[r] & (on_board < 5)
+        dev = self.device
+        plan = SimpleNamespace(
+            direct=torch.from_numpy(np.nonzero(~chance)[0]).to(dev),
+            chance=torch.from_numpy(np.nonzero(chance)[0]).to(dev),
+            board=torch.from_numpy(board).to(dev),
+            street=ev.env.street[rows].to(torch.long),
+            to_act=ev.env.to_act[rows].to(torch.long),
+            cards=int(on_board[chance][0]) if chance.any() and (on_board[chance] == on_board[chance][0]).all() else None,
+        )
+        return plan
+
+    def _features(self, beliefs: torch.Tensor, plan, sel: torch.Tensor | None = None) -> MLPFeatures:
+        k = beliefs.shape[0]
+        f = MLPFeatures(context=torch.zeros(k, 1, dtype=torch.float32, device=self.device), street=plan.street,
+                        to_act=plan.to_act, board=plan.board, beliefs=beliefs.reshape(k, -1))
+        return f if sel is None else f[sel]
+
+    @torch.no_grad()
+    def leaf_values(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
+        key = (id(ev), id(ev.tree), rows.data_ptr(), rows.numel())
+        if self._plan_for != key:
+            self._plan, self._plan_for = self._make_plan(rows, ev), key
+        plan = self._plan
+        beliefs = beliefs.contiguous().float()
+        out = torch.empty_like(beliefs)
+        if plan.direct.numel():
+            feats = self._features(beliefs, plan, plan.direct)
+            if hasattr(self.net, "eval"):
+                self.net.eval()
+            if self.autocast_dtype is not None:
+                with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                    hv = self.net(feats).hand_values
+            else:
+                hv = self.net(feats).hand_values
+            out.index_copy_(0, plan.direct, hv.to(out.dtype))
+        if plan.chance.numel():
+            feats = self._features(beliefs, plan)
+            per_state = 52 - (plan.cards if plan.cards is not None else 0)
+            step = max(1, self.max_samples_per_call // per_state)
+            for lo in range(0, plan.chance.numel(), step):
+                sel = plan.chance[lo:lo + step]
+                ev_chance = self.helper.single_card_chance_values(sel, feats, beliefs, plan.board,
+                                                                  cards_on_board=plan.cards)
+                out.index_copy_(0, sel, ev_chance.to(out.dtype))
+        return out

@@ -129,3 +129,69 @@ def test_helper_edge_cases(K):
                         cards_on_board=4)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+
+
+# ---- turn subgame: street-end leaves valued through the chance node + a small network --------
+def numpy_mlp(net):
+    ws = [(l.weight.detach().cpu().numpy().astype(np.float32), l.bias.detach().cpu().numpy().astype(np.float32))
+          for l in net.linears]
+
+    def fn(context, street, to_act, board, beliefs):
+        onehot = np.zeros((board.shape[0], 52), np.float32)
+        i, j = np.nonzero(board >= 0)
+        onehot[i, board[i, j]] = 1.0
+        x = np.concatenate([beliefs.astype(np.float32), onehot], axis=1)
+        for k, (w, b) in enumerate(ws):
+            x = x @ w.T + b
+            if k < len(ws) - 1:
+                x = np.maximum(x, 0.0)
+        return x.reshape(-1, 2, H)
+    return fn
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused):
+    from oracle import cfr as OCFR
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import ChanceLeafModel, RangeBoardMLP
+    from poker2_amd.tree import RootStates
+    from tests.helpers import random_ranges
+    from tests.test_gpu_evaluator import compare, tree_as_dict
+    rng = np.random.default_rng(12)
+    n, iters = 2, 5
+    boards = np.full((n, 5), -1, dtype=np.int64)
+    boards[:, :4] = random_boards(rng, n, 4)
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards, button=np.arange(n) % 2)
+    cfg = river_dcfr_config(n, iterations=iters, depth=16, dcfr_delay=0)
+    dev = torch.device("cuda")
+    net = RangeBoardMLP(hidden=64, layers=2, seed=3).to(dev)
+    with torch.no_grad():
+        for lin in net.linears:                       # orthogonal rows of a 2704-wide input give tiny outputs;
+            lin.weight.mul_(4.0)                      # scale them up so leaf values matter to the strategy
+    model = ChanceLeafModel(net, dev)
+    ev = HipSparseCFREvaluator(model, dev, cfg, fused_iteration=fused, max_raises=1)
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+    ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+    tree = ev.tree
+    assert tree.showdown_mask.sum() == 0 and tree.new_street_mask.sum() == 7 * n
+    mlp = numpy_mlp(net)
+    node_board = tree.board[tree.root_index]
+    street, to_act = tree.state["street"], tree.state["to_act"]
+
+    def leaf_fn(bel, rows):
+        k = len(rows)
+        return OCH.single_card_chance_values(np.arange(k), np.zeros((k, 1), np.float32), street[rows], to_act[rows],
+                                             bel[rows], node_board[rows], mlp)
+    orc = OCFR.OracleCFR(tree_as_dict(tree), boards, beliefs, cfr_iterations=iters, leaf_value_fn=leaf_fn,
+                         t_sample_roots=np.full(n, -1, dtype=np.int64), fused_variant=True)
+    orc.prepare()
+    compare(ev, orc, rtol=2e-4, atol=2e-5)
+    assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3     # the network's values are not trivial
+    # the network runs through hipBLASLt here and numpy there: leaf values differ by GEMM summation
+    # order (~1e-6 relative) and regret matching divides by small regret sums, hence the wider bar
+    for t in range(iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+        compare(ev, orc, rtol=1e-3, atol=3e-4)
