@@ -114,6 +114,19 @@ def cases(repeats: int):
     res = torch.empty_like(bel)
     yield ("showdown_value_both states=4096", 4 * m * H * 4,
            lambda: R.showdown_value_both(bel, tables, pot, sc, out=res))
+    del tables, res
+
+    # --- single-card chance node: 3584 turn leaves (512 roots x 7) x 48 river cards
+    from . import chance_node_helper as CH
+    k = 3584
+    tb = torch.full((k, 5), -1, dtype=torch.int64, device=dev)
+    tb[:, :4] = boards[:k, :4]
+    roots = torch.arange(k, device=dev)
+    pre = bel[:k].contiguous()
+    post, _, _, offsets = CH.chance_expand(pre, roots, tb, cards_on_board=4)
+    yield ("chance_expand states=3584 x48", k * (2 + 2 * 48) * H * 4,
+           lambda: CH.chance_expand(pre, roots, tb, cards_on_board=4))
+    yield ("chance_mean states=3584 x48", k * (2 * 48 + 2) * H * 4, lambda: CH.chance_mean(post, offsets))
 
 
 def main() -> None:

@@ -21,6 +21,8 @@ namespace p2 {
 
 constexpr int CH_BLOCK = 256;
 constexpr int CH_PPT = 3;  // float2 pairs per thread and vector
+constexpr int CH_SPLIT = 4;  // workgroups per state in the expansion (13 candidate cards each)
+static_assert(P2_CARDS % CH_SPLIT == 0, "card runs");
 static_assert(CH_BLOCK == UB_BLOCK, "card_sums_multi assumes the block size");
 
 __device__ __forceinline__ int chance_board(const int64_t* __restrict__ board5, int (&cards)[5], uint64_t& bits) {
@@ -55,6 +57,7 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
 
   // this lane's hands: pairs k -> hands 2*idx, 2*idx+1 with idx = tid + k*256
   float v[2][CH_PPT][2];
+  float uni[CH_PPT][2];   // the hand's share of the uniform fallback (0 for hands on the board)
   uint32_t ab[CH_PPT][2];
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) {
@@ -82,8 +85,18 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
 
   const int remaining = P2_CARDS - ncards - 1;          // cards left for the hands of a sample
   const float uniform = 1.0f / fmaxf((float)(remaining * (remaining - 1) / 2), 1.0f);
-  int64_t s = sample_offsets[i];
-  for (int c = 0; c < P2_CARDS; ++c) {
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const bool on_board = ((bits >> (ab[k][q] & 0xFFu)) | (bits >> (ab[k][q] >> 8))) & 1ull;
+      uni[k][q] = on_board ? 0.f : uniform;
+    }
+  // blockIdx.y splits the 52 candidate cards into CH_SPLIT runs so that more workgroups share
+  // the write stream; a sample's position counts the cards below it that are not on the board
+  const int c_begin = blockIdx.y * (P2_CARDS / CH_SPLIT), c_end = c_begin + P2_CARDS / CH_SPLIT;
+  int64_t s = sample_offsets[i] + c_begin - __popcll(bits & ((1ull << c_begin) - 1ull));
+  for (int c = c_begin; c < c_end; ++c) {
     if ((bits >> c) & 1ull) continue;
     const float sum0 = (float)(total0 - cs[c]);
     const float sum1 = (float)(total1 - cs[P2_CARDS + c]);
@@ -100,10 +113,8 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
       for (int q = 0; q < 2; ++q) {
         const uint32_t a = ab[k][q] & 0xFFu, b = ab[k][q] >> 8;
         const bool off = a == (uint32_t)c || b == (uint32_t)c;
-        const bool on_board = ((bits >> a) | (bits >> b)) & 1ull;
-        const float u = (off || on_board) ? 0.f : uniform;
-        r0[q] = ok0 ? (off ? 0.f : v[0][k][q] * inv0) : u;
-        r1[q] = ok1 ? (off ? 0.f : v[1][k][q] * inv1) : u;
+        r0[q] = off ? 0.f : (ok0 ? v[0][k][q] * inv0 : uni[k][q]);
+        r1[q] = off ? 0.f : (ok1 ? v[1][k][q] * inv1 : uni[k][q]);
       }
       o0[idx] = make_float2(r0[0], r0[1]);
       o1[idx] = make_float2(r1[0], r1[1]);
@@ -166,7 +177,8 @@ int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, c
   if (n == 0) return 0;
   if (!pre_beliefs || !board || !sample_offsets || !post_beliefs || !board_samples || !root_lookup) return P2_EINVAL;
   if (!p2_aligned8(pre_beliefs) || !p2_aligned8(post_beliefs)) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::chance_expand_kernel, dim3((unsigned)n), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+  if (n > 0x7FFFFFFF) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::chance_expand_kernel, dim3((unsigned)n, p2::CH_SPLIT), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
                      pre_beliefs, root_indices, board, sample_offsets, post_beliefs, board_samples, root_lookup);
   P2_LAUNCH_CHECK();
   return 0;
