@@ -32,6 +32,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_showdown_table_bytes": [],
     "p2hip_showdown_setup": [_P, _I, _L, _I, _P, _P, _P, _P],
     "p2hip_showdown_both": [_P, _P, _P, _P, _P, _L, _P, _P],
+    "p2hip_best_response_level": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _P],
     "p2hip_chance_expand": [_P, _P, _P, _L, _P, _P, _P, _P, _P],
     "p2hip_chance_mean": [_P, _P, _L, _P, _P],
     "p2hip_unblocked_mass": [_P, _L, _P, _P],

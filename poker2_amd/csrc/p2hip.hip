@@ -7,6 +7,7 @@
 #include "cfr_ops.hip"
 #include "cfr_iter.hip"
 #include "chance.hip"
+#include "best_response.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

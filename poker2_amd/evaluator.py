@@ -27,6 +27,7 @@ exploitability statistics, warm start.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 from types import SimpleNamespace
 
 import numpy as np
@@ -56,6 +57,13 @@ class _IterArgs(ctypes.Structure):
 
 def _cfr_type_name(x) -> str:
     return getattr(x, "name", str(x))
+
+
+@dataclass
+class ExploitabilityStats:
+    """src/p2/search/cfr_evaluator.py:35-38."""
+    local_exploitability: torch.Tensor          # [N]
+    local_best_response_values: torch.Tensor    # [N, 2]
 
 
 class HipSparseCFREvaluator:
@@ -582,6 +590,52 @@ class HipSparseCFREvaluator:
             s = (self.values_avg * self.beliefs_avg).sum(dim=2, keepdim=True).mean(dim=1, keepdim=True)
             s.masked_fill_(self.env.done[:, None, None], 0.0)
             self.values_avg -= s
+
+    # ------------------------------------------------------------------ best response
+    def _fan_out_deep(self, per_root: torch.Tensor) -> torch.Tensor:
+        """Per-root values repeated on every node of the root's subtree (sparse_cfr_evaluator.py:504-523)."""
+        return per_root.index_select(0, self._root_index)
+
+    def _best_response_values(self, policy: torch.Tensor, beliefs: torch.Tensor, base_values: torch.Tensor,
+                              deviating_player: torch.Tensor | None = None) -> torch.Tensor:
+        """Values when ``deviating_player`` (per node; default: the root's player to act) plays a
+        per-hand best response and the other player follows ``policy``
+        (cfr_evaluator.py:603-716).  One kernel launch per tree level, deepest first."""
+        n = self.root_nodes
+        if deviating_player is None:
+            deviating_player = self._fan_out_deep(self.env.to_act[:n])
+        deviating_player = deviating_player.to(device=self.device, dtype=torch.int64).contiguous()
+        assert deviating_player.shape == (self.total_nodes,)
+        policy = policy.contiguous()
+        beliefs = beliefs.contiguous()
+        values_br = torch.where(self.leaf_mask[:, None, None], base_values, torch.zeros_like(base_values)).contiguous()
+        for depth in range(self.tree_depth - 1, -1, -1):
+            base, end = self.depth_offsets[depth], self.depth_offsets[depth + 1]
+            _lib.call("p2hip_best_response_level", _lib.ptr(values_br), _lib.ptr(policy), _lib.ptr(beliefs),
+                      _lib.ptr(self.env.to_act), _lib.ptr(deviating_player), _lib.ptr(self.child_offsets),
+                      _lib.ptr(self.child_count), int(base), int(end - base), _lib.stream_ptr())
+        return values_br
+
+    def _compute_exploitability(self) -> ExploitabilityStats:
+        """Gain of a per-hand best response over the average strategy, per root, summed over the
+        two players and weighted by the root beliefs (cfr_evaluator.py:718-764)."""
+        n = self.root_nodes
+        if n == 0:
+            return ExploitabilityStats(torch.empty(0, device=self.device, dtype=self.float_dtype),
+                                       torch.empty(0, 2, device=self.device, dtype=self.float_dtype))
+        policy, beliefs = self.policy_probs_avg, self.beliefs_avg
+        leaf_values = self.values_avg.clamp(-1.0, 1.0)
+        base_values = torch.zeros_like(leaf_values)
+        self.compute_expected_values(policy=policy, beliefs=beliefs, leaf_values=leaf_values, values=base_values)
+        improvements, br_agg = [], []
+        for player in range(2):
+            deviator = torch.full((n,), player, device=self.device, dtype=torch.int64)
+            br = self._best_response_values(policy, beliefs, leaf_values, self._fan_out_deep(deviator))
+            root_beliefs = beliefs[:n, player]
+            improvements.append(((br[:n, player] - base_values[:n, player]) * root_beliefs).sum(dim=-1))
+            br_agg.append((br[:n, player] * root_beliefs).sum(dim=-1))
+        return ExploitabilityStats(local_exploitability=improvements[0] + improvements[1],
+                                   local_best_response_values=torch.stack(br_agg, dim=-1))
 
     def state_dict(self) -> dict:
         return {n: getattr(self, n) for n in STATE_NAMES}

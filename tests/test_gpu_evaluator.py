@@ -158,3 +158,31 @@ def test_structural_invariants_after_many_iterations():
     # blocked hands never carry reach below the root
     blocked = ~ev.allowed_hands[n:]
     assert (ev.self_reach[n:, 0][blocked] == 0).all() and (ev.self_reach[n:, 1][blocked] == 0).all()
+
+
+@pytest.mark.parametrize("depth,max_raises", [(2, None), (16, 2)])
+def test_best_response_and_exploitability_match_oracle(depth, max_raises):
+    """The best-response kernels against the oracle ON THE SAME STATE (the evaluator's tensors are
+    copied into the oracle first), so that only the operation under test is compared."""
+    from oracle import best_response as OBR
+    iters = 6
+    ev, orc = make_pair(3, depth, max_raises, seed=31, fused=True, iters=iters)
+    for t in range(iters):
+        ev.cfr_iteration(t)
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        getattr(orc, name)[:] = getattr(ev, name).cpu().numpy()
+    rng = np.random.default_rng(0)
+    for dev_np in (np.zeros(ev.total_nodes, np.int64), np.ones(ev.total_nodes, np.int64),
+                   rng.integers(0, 2, ev.total_nodes), None):
+        dev_t = None if dev_np is None else torch.from_numpy(dev_np).cuda()
+        got = ev._best_response_values(ev.policy_probs_avg, ev.beliefs_avg, ev.values_avg, dev_t).cpu().numpy()
+        exp = OBR.best_response_values(orc, orc.policy_probs_avg, orc.beliefs_avg, orc.values_avg, dev_np)
+        err = np.abs(got - exp) - (2e-6 + 1e-5 * np.abs(exp))       # float32: 1e-5 relative
+        # exempt by count: a hand whose two best children tie within rounding may pick the other
+        # child, which moves the OTHER player's value by O(1)
+        assert (err > 0).mean() <= FLIP_FRACTION, f"max abs diff {np.abs(got - exp).max():.3e}"
+    stats = ev._compute_exploitability()
+    expl, br = OBR.compute_exploitability(orc)
+    np.testing.assert_allclose(stats.local_exploitability.cpu().numpy(), expl, rtol=1e-4, atol=2e-6)
+    np.testing.assert_allclose(stats.local_best_response_values.cpu().numpy(), br, rtol=1e-4, atol=2e-6)
+    assert (expl > 0).all()
