@@ -186,3 +186,32 @@ def test_best_response_and_exploitability_match_oracle(depth, max_raises):
     np.testing.assert_allclose(stats.local_exploitability.cpu().numpy(), expl, rtol=1e-4, atol=2e-6)
     np.testing.assert_allclose(stats.local_best_response_values.cpu().numpy(), br, rtol=1e-4, atol=2e-6)
     assert (expl > 0).all()
+
+
+def test_200_iterations_average_strategy_quality_and_root_values():
+    """River subgames on the three-raise tree (105 nodes per root), 200 discounted-CFR iterations.
+    Element-wise agreement cannot survive that long: the algorithm's thresholds make the
+    iteration chaotic (two ORACLE runs whose initial ranges differ by 2e-7 relative on 50 hands
+    differ by 0.36 in single policy entries and by 1.2e-3 in root values after 200 iterations).
+    What must agree is what a search returns: the root values and the quality of the average
+    strategy, measured by the reference's own local exploitability."""
+    from oracle import best_response as OBR
+    iters, n = 200, 2
+    ev, orc = make_pair(n, 16, 3, seed=77, fused=True, iters=iters)
+    assert ev.total_nodes == 105 * n
+    for t in range(iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+        if t == 4:
+            compare(ev, orc, rtol=2e-4, atol=2e-5)          # element-wise early on ...
+        if t == 9:
+            compare(ev, orc, rtol=1e-3, atol=1e-4)          # ... growing about tenfold per 25 iterations
+    got = ev._compute_exploitability()
+    expl, br = OBR.compute_exploitability(orc)
+    np.testing.assert_allclose(got.local_exploitability.cpu().numpy(), expl, rtol=0.05)
+    np.testing.assert_allclose(got.local_best_response_values.cpu().numpy(), br, atol=2e-3)
+    assert (expl < 0.12).all()                              # started at 0.47-0.48 (uniform play)
+    root_gpu, root_orc = ev.values_avg[:n].cpu().numpy(), orc.values_avg[:n]
+    assert np.abs(root_gpu - root_orc).max() < 1e-2
+    w = orc.beliefs_avg[:n]
+    np.testing.assert_allclose((root_gpu * w).sum(-1), (root_orc * w).sum(-1), atol=1e-3)
