@@ -73,6 +73,8 @@ class OracleCFR:
         cfr_avg: bool = False,
         cfr_iterations: int = 200,
         warm_start_iterations: int = 0,
+        warm_start_type: str = "model_br",
+        warm_start_multiplier: float = 1.0,
         use_final_policy_values: bool = False,
         enforce_zero_sum: bool = False,
         dcfr_alpha_final: float | None = None,
@@ -121,6 +123,9 @@ class OracleCFR:
         self.cfr_avg = cfr_avg
         self.cfr_iterations = cfr_iterations
         self.warm_start_iterations = warm_start_iterations
+        assert warm_start_type in ("model", "model_br")
+        self.warm_start_type = warm_start_type
+        self.warm_start_multiplier = warm_start_multiplier
         self.use_final_policy_values = use_final_policy_values
         self.enforce_zero_sum = enforce_zero_sum
         self.leaf_value_fn = leaf_value_fn
@@ -444,11 +449,38 @@ class OracleCFR:
         if not self.use_final_policy_values:
             self.update_average_values(t)
 
+    # ---- warm start (cfr_evaluator.py:888-955) -----------------------------------
+    def warm_start(self) -> None:
+        from .best_response import best_response_values
+        self.set_leaf_values(0)
+        self.compute_expected_values(policy=self.policy_probs, beliefs=self.beliefs,
+                                     leaf_values=self.latest_values, values=self.latest_values)
+        t_ws = self.warm_start_iterations
+        scale = F32(float(t_ws) * float(self.warm_start_multiplier))
+        self.apply_schedules(t_ws)
+        bottom = self.depth_offsets[1]
+        if self.warm_start_type == "model":
+            regrets = self.compute_instantaneous_regrets(self.latest_values)
+            weights = scale * np.maximum(regrets[bottom:], F32(0.0)).mean(axis=-1, dtype=F32)
+            self.cumulative_regrets[bottom:] = self.policy_probs[bottom:] * weights[:, None]
+            self.regret_weight_sums[bottom:] = weights[:, None]
+            self.update_policy(t_ws)
+            return
+        br0 = best_response_values(self, self.policy_probs, self.beliefs, self.latest_values,
+                                   np.zeros_like(self.to_act))
+        br1 = best_response_values(self, self.policy_probs, self.beliefs, self.latest_values,
+                                   np.ones_like(self.to_act))
+        values_br = np.where((self.prev_actor == 0)[:, None, None], br0, br1)
+        regrets = self.compute_instantaneous_regrets(values_br, self.latest_values)
+        self.cumulative_regrets += scale * regrets
+        self.regret_weight_sums += scale
+        self.update_policy(t_ws)
+
     def prepare(self) -> None:
-        """The part of evaluate_cfr that precedes the loop (:1505-1515), without
-        warm start."""
-        assert self.warm_start_iterations == 0, "warm start is not restated"
+        """The part of evaluate_cfr that precedes the loop (:1505-1515)."""
         self.initialize_policy_and_beliefs()
+        if self.warm_start_iterations > 0:
+            self.warm_start()
         self.set_leaf_values(0)
         self.compute_expected_values()
         self.values_avg[:] = self.latest_values

@@ -17,7 +17,7 @@ class SearchConfig:
     depth: int = 2
     iterations: int = 100
     warm_start_iterations: int = 15
-    warm_start_type: str = "best_response"
+    warm_start_type: str = "model_br"     # model | model_br (structured_config.py:53-55)
     warm_start_multiplier: float = 1.0
     dcfr_alpha: float = 1.5
     dcfr_beta: float = 0.0

@@ -87,8 +87,10 @@ class HipSparseCFREvaluator:
         self.max_depth = s.depth
         self.cfr_iterations = s.iterations
         self.warm_start_iterations = max(0, min(s.warm_start_iterations, max(1, self.cfr_iterations - 1)))
-        if self.warm_start_iterations > 0:
-            raise NotImplementedError("warm start is not part of this build; set warm_start_iterations=0")
+        self.warm_start_type = str(getattr(s.warm_start_type, "name", s.warm_start_type))
+        if self.warm_start_type not in ("model", "model_br"):
+            raise ValueError(f"unknown warm_start_type {self.warm_start_type!r} (model | model_br)")
+        self.warm_start_multiplier = float(s.warm_start_multiplier)
         self.cfr_type = CFRType[_cfr_type_name(s.cfr_type)]
         self.cfr_avg = bool(s.cfr_avg)
         self.cfr_plus = bool(s.cfr_plus)
@@ -563,9 +565,53 @@ class HipSparseCFREvaluator:
         self.self_reach_avg[:] = self.self_reach
         self.beliefs_avg[:] = self.beliefs
 
+    def warm_start(self) -> None:
+        """Seed the regrets before the first iteration (cfr_evaluator.py:888-955).
+        ``model``: regrets that make regret matching replay the initial (model) policy, weighted
+        by the mean positive regret of each action.  ``model_br``: one best-response pass — the
+        regret of every action against each player's best-response values, scaled by
+        warm_start_iterations x warm_start_multiplier."""
+        self.set_leaf_values(0)
+        if not torch.isfinite(self.latest_values).all():
+            raise ValueError("Non-finite values in latest_values after set_leaf_values")
+        self.compute_expected_values(policy=self.policy_probs, beliefs=self.beliefs, leaf_values=self.latest_values,
+                                     values=self.latest_values)
+        if not torch.isfinite(self.latest_values).all():
+            raise ValueError("Non-finite values in latest_values after compute_expected_values")
+        self._record_initial_exploitability()
+        t_ws = self.warm_start_iterations
+        scale = float(t_ws) * self.warm_start_multiplier
+        self.prepare_replay(t_ws)
+        if self.warm_start_type == "model":
+            bottom = self.depth_offsets[1]
+            regrets = self.compute_instantaneous_regrets(self.latest_values)
+            weights = scale * regrets[bottom:].clamp(min=0.0).mean(dim=-1)
+            self.cumulative_regrets[bottom:] = self.policy_probs[bottom:] * weights[:, None]
+            self.regret_weight_sums[bottom:] = weights[:, None]
+            self.update_policy(t_ws)
+            return
+        br0 = self._best_response_values(self.policy_probs, self.beliefs, self.latest_values,
+                                         torch.zeros_like(self.env.to_act))
+        br1 = self._best_response_values(self.policy_probs, self.beliefs, self.latest_values,
+                                         torch.ones_like(self.env.to_act))
+        # (not meaningful on root rows, which take no part in the regrets)
+        values_br = torch.where(self.prev_actor[:, None, None] == 0, br0, br1)
+        regrets = self.compute_instantaneous_regrets(values_achieved=values_br, values_expected=self.latest_values)
+        self.cumulative_regrets += scale * regrets
+        self.regret_weight_sums += scale
+        self.update_policy(t_ws)
+
+    def _record_initial_exploitability(self) -> None:
+        """cfr_evaluator.py:1618-1633 (mean over roots; no per-street split)."""
+        if self._skip_record_stats:
+            return
+        self.stats["local_exploitability_init"] = self._compute_exploitability().local_exploitability.mean().item()
+
     def prepare_search(self, t_sample: torch.Tensor | None = None) -> None:
         """Everything ``evaluate_cfr`` does before its loop (cfr_evaluator.py:1505-1515)."""
         self.initialize_policy_and_beliefs()
+        if self.warm_start_iterations > 0:
+            self.warm_start()
         self.prepare_replay(0)
         self.set_leaf_values(0)
         self.compute_expected_values()

@@ -20,7 +20,8 @@ def tree_as_dict(t):
 
 
 def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discounted", delay=0, cfr_plus=False,
-              enforce_zs=False, stacks=(800, 800), pot=200, t_sample=None, bins=(0.5, 1.0)):
+              enforce_zs=False, stacks=(800, 800), pot=200, t_sample=None, bins=(0.5, 1.0), warm_start=0,
+              warm_start_type="model_br", warm_start_multiplier=1.0):
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.fused_cfr_hip import CFRType
@@ -35,6 +36,9 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
     cfg.search.cfr_type = CFRType[cfr_type]
     cfg.search.cfr_plus = cfr_plus
     cfg.env.bet_bins = list(bins)
+    cfg.search.warm_start_iterations = warm_start
+    cfg.search.warm_start_type = warm_start_type
+    cfg.search.warm_start_multiplier = warm_start_multiplier
     model = None
     if enforce_zs:
         class ZeroModel:
@@ -55,7 +59,8 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
     orc = OCFR.OracleCFR(tree_as_dict(ev.tree), boards, beliefs, cfr_type=cfr_type, dcfr_alpha=1.5, dcfr_beta=0.0,
                          dcfr_gamma=2.0, dcfr_delay=delay, cfr_plus=cfr_plus, cfr_iterations=iters,
                          enforce_zero_sum=enforce_zs, t_sample_roots=t_sample, ranker=ranker,
-                         fused_variant=True)
+                         warm_start_iterations=warm_start, warm_start_type=warm_start_type,
+                         warm_start_multiplier=warm_start_multiplier, fused_variant=True)
     ev.prepare_search(t_sample=torch.from_numpy(np.asarray(t_sample))[torch.from_numpy(ev.tree.root_index)])
     orc.prepare()
     return ev, orc
@@ -215,3 +220,16 @@ def test_200_iterations_average_strategy_quality_and_root_values():
     assert np.abs(root_gpu - root_orc).max() < 1e-2
     w = orc.beliefs_avg[:n]
     np.testing.assert_allclose((root_gpu * w).sum(-1), (root_orc * w).sum(-1), atol=1e-3)
+
+
+@pytest.mark.parametrize("ws_type,mult", [("model", 10.0), ("model_br", 1.0)])
+def test_warm_start_matches_oracle(ws_type, mult):
+    iters = 8
+    ev, orc = make_pair(3, 16, 1, seed=41, fused=True, iters=iters, cfr_type="discounted_plus", delay=4,
+                        warm_start=3, warm_start_type=ws_type, warm_start_multiplier=mult)
+    compare(ev, orc, rtol=2e-4, atol=2e-5)                  # state right after the warm start
+    assert ev.regret_weight_sums[ev.root_nodes:].abs().max().item() > 0
+    for t in range(3, iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+    compare(ev, orc, rtol=5e-4, atol=5e-5)

@@ -428,3 +428,51 @@ def test_oracle_matches_independent_solver_on_tiny_ranges(depth):
     v0 = o.values_avg[0, 0, hands0]
     value_oracle = float((p0 * m1 * v0).sum() / (p0 * m1).sum())
     assert abs(value_oracle - nash_value) < 3e-3
+
+
+# ---------------------------------------------------------------------------------------
+# warm start (cfr_evaluator.py:888-955)
+def test_warm_start_model_replays_the_initial_policy_and_model_br_reduces_exploitability():
+    from oracle import best_response as OBR
+    rng = np.random.default_rng(9)
+    n = 2
+    t = river_tree(n, depth=3)
+    boards = random_boards(rng, n)
+    bel = random_ranges(rng, boards)
+    logits = rng.standard_normal((t["depth_offsets"][-1], 1326, t["legal_mask"].shape[1])).astype(np.float32)
+
+    def policy_logits(beliefs, rows):
+        return logits[rows]
+    base = OCFR.OracleCFR(t, boards, bel, cfr_iterations=30, policy_logits_fn=policy_logits)
+    base.prepare()
+    # `model`: cumulative regrets = policy x weight, so regret matching gives the policy back
+    # wherever the action's mean positive regret is > 0, and the weight sums hold the weights
+    o = OCFR.OracleCFR(t, boards, bel, cfr_iterations=30, policy_logits_fn=policy_logits,
+                       warm_start_iterations=5, warm_start_type="model", warm_start_multiplier=10.0)
+    o.initialize_policy_and_beliefs()
+    before = o.policy_probs.copy()
+    o.warm_start()
+    nroot = o.root_nodes
+    w = o.regret_weight_sums[nroot:, 0]
+    assert (w >= 0).all() and (w > 0).any()
+    np.testing.assert_allclose(o.cumulative_regrets[nroot:], before[nroot:] * w[:, None], rtol=1e-6)
+    wsum = np.zeros(o.depth_offsets[-2], np.float32)
+    np.add.at(wsum, o.parent_index[nroot:] , w)
+    full = np.repeat(wsum > 0, o.child_count[: o.depth_offsets[-2]])       # families with some weight
+    expect = before[nroot:] * w[:, None]
+    fam = np.zeros((o.depth_offsets[-2], 1326), np.float32)
+    np.add.at(fam, o.parent_index[nroot:], expect)
+    expect = expect / np.maximum(np.repeat(fam, o.child_count[: o.depth_offsets[-2]], axis=0), 1e-30)
+    live = full[:, None] & (np.repeat(fam, o.child_count[: o.depth_offsets[-2]], axis=0) > 1e-8)
+    np.testing.assert_allclose(o.policy_probs[nroot:][live], expect[live], rtol=1e-5, atol=1e-7)
+    # `model_br`: regrets against best-response values push the policy towards the best response
+    e0, _ = OBR.compute_exploitability(base)
+    b = OCFR.OracleCFR(t, boards, bel, cfr_iterations=30, policy_logits_fn=policy_logits,
+                       warm_start_iterations=5, warm_start_type="model_br")
+    b.prepare()
+    assert (b.regret_weight_sums[nroot:] == np.float32(5.0)).all()
+    assert np.abs(b.policy_probs - base.policy_probs).max() > 0.05
+    for it in range(5, 30):
+        b.cfr_iteration(it)
+    e1, _ = OBR.compute_exploitability(b)
+    assert (e1 < e0).all()
