@@ -214,7 +214,9 @@ int p2hip_sample_snapshot(const float* policy_probs, float* policy_probs_sample,
  *   potential [total,2] float, scale [total] float: showdown pay-off factors per row
  *   scratch [total,H] float workspace
  *   fscal[8]: t^alpha, t^beta, t^alpha+1, t^beta+1, mix_old, mix_new, mix_old+mix_new, 1/(mix_old+mix_new)
- *   iscal[6]: t, apply_dcfr, cfr_plus, average_policy_is_copied, enforce_zero_sum, update_average_values */
+ *   iscal[8]: t, apply_dcfr, cfr_plus, average_policy_is_copied, enforce_zero_sum, update_average_values,
+ *             cfr_avg (regret weights and showdown values from beliefs_avg), linear (regrets of player t mod 2
+ *             dropped, no discount) */
 typedef struct P2HipIterArgs {
   const int64_t* child_offsets;
   const int64_t* child_count;

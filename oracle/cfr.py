@@ -441,7 +441,9 @@ class OracleCFR:
             self.regret_weight_sums /= den
         self.regret_weight_sums += F32(1.0)
         self.cumulative_regrets += regrets
-        if self.cfr_plus:
+        # the fused evaluator accumulates linear-CFR regrets without the CFR+ clamp
+        # (fused_sparse_cfr_evaluator.py:503-507); the base class clamps for every type (:1366-1368)
+        if self.cfr_plus and not (self.fused_variant and self.cfr_type == "linear"):
             np.maximum(self.cumulative_regrets, F32(0.0), out=self.cumulative_regrets)
         self.update_policy(t)
         self.set_leaf_values(t)

@@ -68,7 +68,7 @@ struct IterArgs {
   float* scratch;                    // [total,H] workspace
   // iteration-dependent scalars in device memory
   const float* fscal;    // t_alpha_num, t_beta_num, t_alpha_den, t_beta_den, mix_old, mix_new, mix_total, mix_inv_total
-  const int64_t* iscal;  // t, apply_dcfr, cfr_plus, avg_policy_copy, enforce_zero_sum, update_avg_values
+  const int64_t* iscal;  // t, apply_dcfr, cfr_plus, avg_policy_copy, enforce_zero_sum, update_avg_values, cfr_avg, linear
   int phases;            // bit 0: sweeps 1+2, bit 1: sweep 3
 };
 
@@ -171,6 +171,11 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
   const int64_t t_now = A.iscal[0];
   const bool apply_dcfr = A.iscal[1] != 0, cfr_plus = A.iscal[2] != 0, avg_copy = A.iscal[3] != 0;
   const bool enforce_zs = A.iscal[4] != 0, update_avg = A.iscal[5] != 0;
+  // cfr_avg: regret weights and showdown values come from the average-policy beliefs
+  // (fused_sparse_cfr_evaluator.py:322,455); linear: the regrets of the player whose turn it is
+  // not (t mod 2) are dropped and nothing is discounted (:503-507)
+  const bool cfr_avg = A.iscal[6] != 0, linear = A.iscal[7] != 0;
+  const float* leaf_beliefs = cfr_avg ? A.beliefs_avg : A.beliefs;
 
   if (A.phases & 1) {
     // ---------------- sweep 1: regrets -> DCFR -> regret matching ----------------
@@ -205,7 +210,7 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
           const int64_t p = A.root_parents[i0 + u];
           const int actor = (int)A.to_act[p];
           float2 bo[IT_PPT], tmp[IT_PPT];
-          ld(bo, A.beliefs, p * 2 + (1 - actor), ln);
+          ld(bo, leaf_beliefs, p * 2 + (1 - actor), ln);
           ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
           to_lds(L.u.vecs[u], bo, ln);
           st(A.scratch, p, tmp, ln);
@@ -226,6 +231,9 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
           IT_FOR(j) bo[j] = ln.ok[j] ? v2[ln.idx[j]] : make_float2(0.f, 0.f);
         }
         unblocked_regs(w, bo, L.cs + u * P2_CARDS, card_total(L.cs + u * P2_CARDS), ln);
+        if (linear && actor == (int)(t_now & 1)) {
+          IT_FOR(j) w[j] = make_float2(0.f, 0.f);   // this player's regrets are skipped at this t
+        }
 
         float2 pos[MAXC][IT_PPT];
         float2 sum[IT_PPT];
@@ -412,11 +420,11 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
       // global memory, hence a full barrier
       __syncthreads();
       float vk[2][SD_PPT];
-      showdown_gather(A.beliefs + A.root_showdown_nodes[sd0] * 2 * P2_H, sdr, vk);
+      showdown_gather(leaf_beliefs + A.root_showdown_nodes[sd0] * 2 * P2_H, sdr, vk);
       for (int64_t i = sd0; i < sd1; ++i) {
         const int64_t c = A.root_showdown_nodes[i];
         float vnext[2][SD_PPT];
-        if (i + 1 < sd1) showdown_gather(A.beliefs + A.root_showdown_nodes[i + 1] * 2 * P2_H, sdr, vnext);
+        if (i + 1 < sd1) showdown_gather(leaf_beliefs + A.root_showdown_nodes[i + 1] * 2 * P2_H, sdr, vnext);
         // the EVs land in the sorted-range buffers, which the evaluation no longer needs by then
         showdown_eval(vk, sdr, L.u.sd, L.u.sd.v[0], L.u.sd.v[1], A.potential[2 * c], A.potential[2 * c + 1],
                       A.scale[c]);

@@ -310,7 +310,11 @@ class HipSparseCFREvaluator:
         f[4], f[5], f[6] = float(mix_old), float(mix_new), total
         f[7] = 1.0 / total if total != 0.0 else 1.0
         i = self._iscal_host
-        i[0], i[1], i[2] = int(t), int(apply_dcfr), int(self.cfr_plus)
+        linear = self.cfr_type == CFRType.linear
+        # the reference's fused evaluator accumulates linear-CFR regrets without the CFR+ clamp
+        # (fused_sparse_cfr_evaluator.py:503-507)
+        i[0], i[1], i[2] = int(t), int(apply_dcfr), int(self.cfr_plus and not linear)
+        i[6], i[7] = int(self.cfr_avg), int(linear)
         i[3], i[4], i[5] = int(self._avg_policy_copies(t)), int(self.enforce_zero_sum), int(not self.use_final_policy_values)
         _lib.call("p2hip_write_scalars", _lib.ptr(self._fscal), _lib.ptr(self._iscal),
                   ctypes.cast(f, ctypes.c_void_p), ctypes.cast(i, ctypes.c_void_p), _lib.stream_ptr())
@@ -496,8 +500,6 @@ class HipSparseCFREvaluator:
     def _launch_iteration(self, phases: int) -> None:
         if self._iter_args is None:
             self._iter_args = self._build_iter_args()
-        if self.cfr_avg:
-            raise NotImplementedError("the one-kernel iteration covers cfr_avg=False; use fused_iteration=False")
         code = _lib.load().p2hip_cfr_iteration(ctypes.byref(self._iter_args), self.root_nodes, self._max_children,
                                                phases, _lib.stream_ptr())
         _lib.check(code, "p2hip_cfr_iteration")
@@ -506,8 +508,6 @@ class HipSparseCFREvaluator:
         """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533)."""
         if not self._skip_t_scalars_update:
             self.prepare_replay(t)
-        if self.cfr_type == CFRType.linear and self.fused_iteration:
-            raise NotImplementedError("linear CFR runs through fused_iteration=False")
         if self.fused_iteration:
             if self._has_model_leaves and self.model is not None:
                 self._launch_iteration(1)

@@ -21,7 +21,7 @@ def tree_as_dict(t):
 
 def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discounted", delay=0, cfr_plus=False,
               enforce_zs=False, stacks=(800, 800), pot=200, t_sample=None, bins=(0.5, 1.0), warm_start=0,
-              warm_start_type="model_br", warm_start_multiplier=1.0):
+              warm_start_type="model_br", warm_start_multiplier=1.0, cfr_avg=False):
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.fused_cfr_hip import CFRType
@@ -35,6 +35,7 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
     cfg = river_dcfr_config(n_roots, iterations=iters, depth=depth, dcfr_delay=delay)
     cfg.search.cfr_type = CFRType[cfr_type]
     cfg.search.cfr_plus = cfr_plus
+    cfg.search.cfr_avg = cfr_avg
     cfg.env.bet_bins = list(bins)
     cfg.search.warm_start_iterations = warm_start
     cfg.search.warm_start_type = warm_start_type
@@ -57,7 +58,7 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
         packed, order = rank_hands_cards(board)
         return packed, order
     orc = OCFR.OracleCFR(tree_as_dict(ev.tree), boards, beliefs, cfr_type=cfr_type, dcfr_alpha=1.5, dcfr_beta=0.0,
-                         dcfr_gamma=2.0, dcfr_delay=delay, cfr_plus=cfr_plus, cfr_iterations=iters,
+                         dcfr_gamma=2.0, dcfr_delay=delay, cfr_plus=cfr_plus, cfr_avg=cfr_avg, cfr_iterations=iters,
                          enforce_zero_sum=enforce_zs, t_sample_roots=t_sample, ranker=ranker,
                          warm_start_iterations=warm_start, warm_start_type=warm_start_type,
                          warm_start_multiplier=warm_start_multiplier, fused_variant=True)
@@ -107,13 +108,18 @@ def test_iterations_match_oracle(fused, depth, max_raises):
     assert ev.policy_probs_sample[ev._root_index == 0].abs().max().item() > 0.0
 
 
-@pytest.mark.parametrize("cfr_type,delay,cfr_plus,zs", [("discounted", 3, False, False),
-                                                         ("discounted_plus", 2, True, False),
-                                                         ("standard", 0, False, True)])
-def test_variants_fused_vs_oracle(cfr_type, delay, cfr_plus, zs):
+@pytest.mark.parametrize("cfr_type,delay,cfr_plus,zs,cfr_avg", [("discounted", 3, False, False, False),
+                                                                 ("discounted_plus", 2, True, False, False),
+                                                                 ("standard", 0, False, True, False),
+                                                                 ("linear", 0, False, False, False),
+                                                                 ("discounted", 0, False, False, True),
+                                                                 ("linear", 0, False, True, True),
+                                                                 ("linear", 0, True, False, False)])
+def test_variants_fused_vs_oracle(cfr_type, delay, cfr_plus, zs, cfr_avg):
     iters = 7
     ev, orc = make_pair(2, 2, None, seed=5, fused=True, iters=iters, cfr_type=cfr_type, delay=delay,
-                        cfr_plus=cfr_plus, enforce_zs=zs, stacks=(500, 900), pot=300, bins=(0.33, 0.75, 1.5))
+                        cfr_plus=cfr_plus, enforce_zs=zs, stacks=(500, 900), pot=300, bins=(0.33, 0.75, 1.5),
+                        cfr_avg=cfr_avg)
     for t in range(iters):
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
