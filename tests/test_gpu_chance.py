@@ -149,8 +149,8 @@ def numpy_mlp(net):
     return fn
 
 
-@pytest.mark.parametrize("fused", [True, False])
-def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused):
+@pytest.mark.parametrize("fused,streets", [(True, (2, 2)), (False, (2, 2)), (True, (3, 2, 2, 3))])
+def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused, streets):
     from oracle import cfr as OCFR
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.evaluator import HipSparseCFREvaluator
@@ -159,11 +159,13 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused):
     from tests.helpers import random_ranges
     from tests.test_gpu_evaluator import compare, tree_as_dict
     rng = np.random.default_rng(12)
-    n, iters = 2, 5
-    boards = np.full((n, 5), -1, dtype=np.int64)
-    boards[:, :4] = random_boards(rng, n, 4)
+    n, iters = len(streets), 5
+    streets = np.array(streets)
+    boards = random_boards(rng, n, 5)
+    boards[streets == 2, 4] = -1                      # turn roots: the river card is still to come
     beliefs = random_ranges(rng, boards)
-    roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards, button=np.arange(n) % 2)
+    roots = RootStates.at_round_start(streets, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards,
+                                      button=np.arange(n) % 2)
     cfg = river_dcfr_config(n, iterations=iters, depth=16, dcfr_delay=0)
     dev = torch.device("cuda")
     net = RangeBoardMLP(hidden=64, layers=2, seed=3).to(dev)
@@ -175,7 +177,8 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused):
     ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
     ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
     tree = ev.tree
-    assert tree.showdown_mask.sum() == 0 and tree.new_street_mask.sum() == 7 * n
+    n_turn, n_river = int((streets == 2).sum()), int((streets == 3).sum())
+    assert ev.model_indices.numel() == 7 * n_turn and tree.showdown_mask.sum() == 7 * n_river
     mlp = numpy_mlp(net)
     node_board = tree.board[tree.root_index]
     street, to_act = tree.state["street"], tree.state["to_act"]
