@@ -221,30 +221,39 @@ __global__ __launch_bounds__(RANK_BLOCK) void rank_cards_i64_kernel(const int64_
 }
 
 // planes [n, HANDS, 52] bytes (non-zero = card present), suit-major.
+// The 52-byte rows of a workgroup's 256 hands are fetched with coalesced dword loads into LDS;
+// a lane then reads its own 13 dwords (stride 13: conflict free) and folds each into four card
+// bits with one multiply.
 template <int HANDS>
 __global__ __launch_bounds__(RANK_BLOCK) void rank_planes_kernel(const uint8_t* __restrict__ planes, int64_t n,
                                                                   int32_t* __restrict__ out, int flush_first) {
-  // 52 bytes = 13 dwords per hand; rows are dword aligned because 52 % 4 == 0
-  const int64_t row = (int64_t)blockIdx.x * RANK_BLOCK + threadIdx.x;
-  if (row >= n) return;
+  constexpr int ROW_DW = 13 * HANDS;  // 52 bytes = 13 dwords per hand; rows are dword aligned
+  __shared__ uint32_t buf[RANK_BLOCK * ROW_DW];
+  const int64_t row0 = (int64_t)blockIdx.x * RANK_BLOCK;
+  const int64_t rows_here = (n - row0) < RANK_BLOCK ? (n - row0) : RANK_BLOCK;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(planes) + row0 * ROW_DW;
+  const int total = (int)rows_here * ROW_DW;
+  for (int i = threadIdx.x; i < total; i += RANK_BLOCK) buf[i] = src[i];
+  __syncthreads();
+  if ((int64_t)threadIdx.x >= rows_here) return;
   int32_t sc[HANDS];
-  const uint32_t* p32 = reinterpret_cast<const uint32_t*>(planes);
 #pragma unroll
   for (int hnd = 0; hnd < HANDS; ++hnd) {
-    const uint32_t* src = p32 + (row * HANDS + hnd) * 13;
-    uint32_t s[4] = {0, 0, 0, 0};
+    const uint32_t* mine = buf + threadIdx.x * ROW_DW + hnd * 13;
+    uint64_t cards = 0;
 #pragma unroll
     for (int w = 0; w < 13; ++w) {
-      uint32_t v = src[w];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int card = 4 * w + k;  // compile-time after unrolling
-        const int suit = card / 13, rank = card % 13;
-        if ((v >> (8 * k)) & 0xFFu) s[suit] |= 1u << rank;
-      }
+      const uint32_t v = mine[w];
+      // bit 7 of every non-zero byte, moved to bit 0, then the four flags gathered into a nibble
+      const uint32_t nz = ((((v & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | v) >> 7) & 0x01010101u;
+      const uint32_t nib = (nz * 0x01020408u) >> 24;
+      cards |= (uint64_t)(nib & 0xFu) << (4 * w);
     }
-    sc[hnd] = score_hand(hand_from_suits(s[0], s[1], s[2], s[3]), flush_first != 0);
+    sc[hnd] = score_hand(hand_from_suits((uint32_t)(cards & 0x1FFFu), (uint32_t)((cards >> 13) & 0x1FFFu),
+                                         (uint32_t)((cards >> 26) & 0x1FFFu), (uint32_t)((cards >> 39) & 0x1FFFu)),
+                         flush_first != 0);
   }
+  const int64_t row = row0 + threadIdx.x;
   if (HANDS == 1) out[row] = sc[0];
   else out[row] = (sc[0] > sc[HANDS - 1]) ? 1 : ((sc[0] < sc[HANDS - 1]) ? -1 : 0);
 }

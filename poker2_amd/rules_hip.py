@@ -31,7 +31,10 @@ def _planes_i8(ab_batch: torch.Tensor, tail: tuple[int, ...]) -> torch.Tensor:
         raise ValueError(f"Expected [N, {', '.join(map(str, tail))}] input, got {tuple(ab_batch.shape)}")
     if ab_batch.device.type != "cuda":
         raise ValueError("The HIP hand evaluator requires a GPU tensor.")
-    return ab_batch.contiguous().to(torch.int8)
+    x = ab_batch.contiguous()
+    if x.dtype in (torch.bool, torch.int8, torch.uint8):
+        return x.view(torch.uint8)            # one byte per card already: no copy (non-zero = present)
+    return (x != 0).view(torch.uint8)
 
 
 def _compare_planes(ab_batch: torch.Tensor, flush_first: int) -> torch.Tensor:
