@@ -304,3 +304,22 @@ def test_unblocked_mass_opp_at_parents_and_ratio(F):
     close(out, exp, rtol=1e-4, atol=1e-6)
     out2 = F.unblocked_mass_ratio_triton(dev(numer), dev(actor[pidx]))
     close(out2, exp, rtol=1e-4, atol=1e-6)
+
+
+def test_unblocked_mass_grid_stride_ragged_and_empty(F):
+    """More rows than one pass of the persistent kernels covers (4 rows x 1024 workgroups),
+    a row count that is not a multiple of the group size, an odd ratio count, and no rows."""
+    rng = np.random.default_rng(53)
+    rows = 2 * 4096 + 3
+    t = rng.random((rows, H)).astype(np.float32)
+    t[5] = 0.0
+    out = F.unblocked_mass_triton(dev(t))
+    close(out, OU.calculate_unblocked_mass(t), rtol=1e-6, atol=1e-4)
+    n = 2 * 2048 + 1
+    numer = (t[:n] * rng.random((n, 1)).astype(np.float32)).astype(np.float32)
+    pidx = rng.integers(0, rows, n).astype(np.int64)
+    out = F.unblocked_mass_ratio_indirect_triton(dev(numer), dev(t), dev(pidx))
+    close(out, OU.unblocked_mass_ratio(numer, t, 1e-5, pidx), rtol=1e-4, atol=1e-6)
+    empty = torch.zeros(0, H, device="cuda")
+    assert F.unblocked_mass_triton(empty).shape == (0, H)
+    assert F.unblocked_mass_ratio_triton(empty, empty).shape == (0, H)
