@@ -66,6 +66,16 @@ class ExploitabilityStats:
     local_best_response_values: torch.Tensor    # [N, 2]
 
 
+@dataclass
+class SampledLeaves:
+    """What ``sample_leaves`` hands to the next search: the sampled non-root leaf rows, their
+    public beliefs and their game states as roots (the reference wraps the same three things in a
+    PublicBeliefState, sparse_cfr_evaluator.py:413-426)."""
+    nodes: torch.Tensor      # [K] rows of this evaluator's tree
+    beliefs: torch.Tensor    # [K, 2, 1326]
+    roots: RootStates        # K root states for ``initialize_subgame``
+
+
 class HipSparseCFREvaluator:
     def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
                  compile_model: bool = True, fused_iteration: bool = True,
@@ -102,6 +112,7 @@ class HipSparseCFREvaluator:
         self.dcfr_gamma_final = s.dcfr_gamma_final
         self.dcfr_delay = s.dcfr_plus_delay
         self.use_final_policy_values = bool(s.value_targets_from_final_policy)
+        self.sample_epsilon = float(getattr(s, "sample_epsilon", 0.25))
         self.generator = generator
         self.fused_iteration = bool(fused_iteration)
         self.max_raises = max_raises
@@ -620,13 +631,15 @@ class HipSparseCFREvaluator:
             t_sample = self._get_sampling_schedule()
         self.t_sample.copy_(t_sample.to(self.device))
 
-    def evaluate_cfr(self, training_mode: bool = True) -> None:
-        """cfr_evaluator.py:1497-1528 without the post-search leaf sampling and statistics."""
+    def evaluate_cfr(self, training_mode: bool = True) -> SampledLeaves:
+        """cfr_evaluator.py:1497-1528 (statistics recording left out): the search, then the
+        leaves from which the next searches continue."""
         self.prepare_search()
         for t in range(self.warm_start_iterations, self.cfr_iterations):
             self.cfr_iteration(t)
         if self.use_final_policy_values:
             self.update_average_values_final()
+        return self.sample_leaves(training_mode)
 
     def update_average_values_final(self) -> None:
         """cfr_evaluator.py:1276-1292."""
@@ -636,6 +649,70 @@ class HipSparseCFREvaluator:
             s = (self.values_avg * self.beliefs_avg).sum(dim=2, keepdim=True).mean(dim=1, keepdim=True)
             s.masked_fill_(self.env.done[:, None, None], 0.0)
             self.values_avg -= s
+
+    # ------------------------------------------------------------------ leaf sampling
+    def _pull_back(self, tensor: torch.Tensor) -> torch.Tensor:
+        """Child-aligned [total, ...] -> [top, num_actions, ...] action slices, zero where an
+        action has no child (sparse_cfr_evaluator.py:465-489)."""
+        top, bottom = self.depth_offsets[-2], self.depth_offsets[1]
+        out = torch.zeros((top, self.num_actions, *tensor.shape[1:]), dtype=tensor.dtype, device=self.device)
+        out[self.parent_index[bottom:], self.action_from_parent[bottom:]] = tensor[bottom:]
+        return out
+
+    def sample_leaves(self, training_mode: bool) -> SampledLeaves:
+        """One leaf per root, sampled by walking down with ``policy_probs_sample`` for a hand
+        drawn from the root actor's beliefs; with probability ``sample_epsilon`` the randomly
+        chosen exploring player acts uniformly; terminal children are never entered
+        (sparse_cfr_evaluator.py:325-426).  Host-side control flow on a handful of small tensors."""
+        n, top = self.root_nodes, self.depth_offsets[-2]
+        gen, dev = self.generator, self.device
+        gdev = gen.device if gen is not None else dev      # draws happen where the generator lives
+
+        def multinomial(p):
+            return torch.multinomial(p.to(gdev), 1, generator=gen).squeeze(1).to(dev)
+        players = torch.randint(0, 2, (n,), generator=gen, device=gdev).to(dev)
+        sample_epsilon = self.sample_epsilon if training_mode else 0.0
+        done_src = self._pull_back(self.env.done)
+        sampling_masks = self.child_mask.clone()
+        sampling_masks[:top] &= ~done_src
+        sampling_counts = sampling_masks.float().sum(dim=-1, keepdim=True)
+        uniform = torch.where(sampling_masks, 1 / sampling_counts, torch.zeros_like(sampling_counts))
+        probs_by_src = self._pull_back(self.policy_probs_sample)
+        probs_by_src.masked_fill_(done_src[:, :, None], 0.0)
+        denom = probs_by_src.sum(dim=1, keepdim=True)
+        probs_by_src = torch.where(denom >= 1e-12, probs_by_src / denom, uniform[:top, :, None])
+        child_action_index = self.child_mask.int().cumsum(dim=1) - self.child_mask.int()
+        effective_leaf = self.leaf_mask | (sampling_counts.squeeze(1) == 0)
+        actor_beliefs = self.beliefs[:n].gather(
+            1, self.env.to_act[:n, None, None].expand(-1, -1, NUM_HANDS)).squeeze(1)
+        selected_hands = multinomial(actor_beliefs)
+        sampled = torch.arange(n, device=dev)
+        depth = 0
+        active = ~effective_leaf[sampled]
+        while bool(active.any()):
+            assert depth <= self.tree_depth
+            nodes = sampled[active]
+            to_act = self.env.to_act[nodes]
+            explore = torch.rand(nodes.numel(), generator=gen, device=gdev).to(dev) < sample_epsilon
+            explore &= to_act == players[active]
+            p_active = probs_by_src[nodes, :, selected_hands[active]]
+            actions = multinomial(torch.where(explore[:, None], uniform[nodes], p_active))
+            sampled[active] = self.child_offsets[nodes] + child_action_index[nodes, actions]
+            active = ~effective_leaf[sampled]
+            depth += 1
+        assert bool(effective_leaf[sampled].all()) and not bool(self.env.done[sampled].any())
+        keep = sampled[sampled >= n]            # roots that are leaves themselves are not continued
+        rows = keep.cpu().numpy()
+        tree = self.tree
+        fields = {}
+        for name in RootStates.__dataclass_fields__:
+            if name == "board":
+                fields[name] = tree.board[tree.root_index[rows]]
+            elif name == "bb":
+                fields[name] = int(self.env.bb)
+            else:
+                fields[name] = np.asarray(tree.state[name])[rows]
+        return SampledLeaves(nodes=keep, beliefs=self.beliefs[keep].clone(), roots=RootStates(**fields))
 
     # ------------------------------------------------------------------ best response
     def _fan_out_deep(self, per_root: torch.Tensor) -> torch.Tensor:

@@ -239,3 +239,54 @@ def test_warm_start_matches_oracle(ws_type, mult):
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
     compare(ev, orc, rtol=5e-4, atol=5e-5)
+
+
+def test_sample_leaves_walks_the_sampled_policy():
+    """sparse_cfr_evaluator.py:325-426: every sampled row is a non-terminal leaf below its own
+    root, terminal children are never entered, the walk follows policy_probs_sample of the drawn
+    hand (checked on a tree whose sampled policy is deterministic), and the returned root states
+    start a new search."""
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    n, iters = 64, 4
+    ev, _ = make_pair(n, 2, None, seed=3, fused=True, iters=iters, t_sample=np.full(n, 2))
+    ev.generator = torch.Generator(device="cpu").manual_seed(5)
+    for t in range(iters):
+        ev.cfr_iteration(t)
+    assert ev.policy_probs_sample.abs().sum().item() > 0
+    out = ev.sample_leaves(training_mode=True)
+    rows = out.nodes.cpu().numpy()
+    tree = ev.tree
+    done = tree.state["done"]
+    # a leaf of the tree, or a node whose every child is terminal (nothing left to search below it)
+    dead_end = np.array([tree.leaf_mask[r] or done[tree.child_offsets[r]:tree.child_offsets[r] + tree.child_count[r]].all()
+                         for r in rows])
+    assert (rows >= n).all() and dead_end.all() and not done[rows].any()
+    assert len(np.unique(tree.root_index[rows])) == len(rows) <= n      # at most one leaf per root
+    assert out.beliefs.shape == (len(rows), 2, 1326) and out.roots.n == len(rows)
+    assert torch.equal(out.beliefs, ev.beliefs[out.nodes])
+    np.testing.assert_array_equal(out.roots.pot, tree.state["pot"][rows])
+    # deterministic sampled policy: always the LAST non-terminal action, no exploration
+    top, bottom = ev.depth_offsets[-2], ev.depth_offsets[1]
+    ev.policy_probs_sample.zero_()
+    target = np.zeros(ev.total_nodes, dtype=bool)
+    for p in range(top):
+        ch = np.arange(tree.child_offsets[p], tree.child_offsets[p] + tree.child_count[p])
+        live = ch[~done[ch]]
+        if len(live):
+            target[live[-1]] = True
+    ev.policy_probs_sample[torch.from_numpy(target).cuda()] = 1.0
+    out = ev.sample_leaves(training_mode=False)
+    for node in out.nodes.cpu().numpy():
+        while node >= n:
+            assert target[node]
+            node = tree.parent_index[node]
+    # the leaves continue as a new search
+    cfg2 = ev.cfg
+    ev2 = HipSparseCFREvaluator(None, torch.device("cuda"), cfg2, fused_iteration=True)
+    ev2.root_nodes = out.roots.n
+    ev2.cfg.num_envs = out.roots.n
+    ev2.initialize_subgame(out.roots, np.arange(out.roots.n), out.beliefs)
+    ev2.prepare_search()
+    ev2.cfr_iteration(0)
+    assert torch.isfinite(ev2.values_avg).all()
