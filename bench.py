@@ -30,7 +30,7 @@ if ROOT not in sys.path:
 H = 1326
 BYTES_PER_NODE_ITER = 29 * H * 4          # 17 vectors written + 12 read per node per iteration
 HBM_PEAK_GBS = 8000.0
-TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2)}
+TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2), "raise3": (16, 3), "depth5": (5, None)}
 # HBM bytes per launch of the iteration kernel from two rocprofv3 --pmc passes (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy): an offline
 # measurement per workload, quoted in the JSON line; None where no counter run exists.

@@ -100,6 +100,29 @@ int p2hip_best_response_level(float* values, const float* policy, const float* b
                               const int64_t* deviating_player, const int64_t* child_offsets,
                               const int64_t* child_count, int64_t parent_base, int64_t num_parents, void* stream);
 
+/* ---- betting tree on the device ----------------------------------------------------------- */
+
+/* A node is a row of p2hip_tree_node_columns() int64 (21): street, to_act, button, pot, stack0,
+ * stack1, committed0, committed1, min_raise, actions_this_round, is_allin0, is_allin1,
+ * starting_stack0, starting_stack1, done, raises, scale (float32 bits), root row, parent row (-1),
+ * action from parent (-1), fold reward (float32 bits).  Two launches per level replace the host
+ * depth loop over HUNLTensorEnv (search/sparse_cfr_evaluator.py:142-306; rules of
+ * env/hunl_tensor_env.py:348-423, 684-724, 766-992); the caller prefix-sums count_out in
+ * between.  host_bins: bet fractions of the pot, at most 5, in HOST memory. */
+int64_t p2hip_tree_node_columns(void);
+
+/* legal_out [n, n_bins+3] bytes: legal action bins (fold, call, bets..., all-in) of every node;
+ * count_out [n]: children the node gets (0 unless `expand`; 0 below the root level when the
+ * node's betting round has just closed).  max_raises < 0: no cap on bets and raises per round. */
+int p2hip_tree_legal(const int64_t* nodes, int64_t n, const float* host_bins, int n_bins, int max_raises,
+                     int is_root_level, int expand, uint8_t* legal_out, int64_t* count_out, void* stream);
+
+/* Children of the n parents (global rows parent_row_base ..), action ascending, written from row
+ * child_start[i] of `children` on (exclusive prefix sums of count_out). */
+int p2hip_tree_step(const int64_t* parents, int64_t n, int64_t parent_row_base, const float* host_bins, int n_bins,
+                    int max_raises, int64_t bb, int is_root_level, const int64_t* child_start, int64_t* children,
+                    void* stream);
+
 /* ---- unblocked (card-compatible) mass --------------------------------------------- */
 
 /* target [rows,H] -> out [rows,H] = max(S - cs[a] - cs[b] + t, 0).  Replaces

@@ -33,6 +33,9 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_showdown_setup": [_P, _I, _L, _I, _P, _P, _P, _P],
     "p2hip_showdown_both": [_P, _P, _P, _P, _P, _L, _P, _P],
     "p2hip_best_response_level": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _P],
+    "p2hip_tree_node_columns": [],
+    "p2hip_tree_legal": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _P],
+    "p2hip_tree_step": [_P, _L, _L, _P, _I, _I, _L, _I, _P, _P, _P],
     "p2hip_chance_expand": [_P, _P, _P, _L, _P, _P, _P, _P, _P],
     "p2hip_chance_mean": [_P, _P, _L, _P, _P],
     "p2hip_unblocked_mass": [_P, _L, _P, _P],
@@ -58,7 +61,8 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_cfr_iteration": [_P, _L, _I, _I, _P],
     "p2hip_write_scalars": [_P, _P, _P, _P, _P],
 }
-_RESTYPE = {"p2hip_error_string": ctypes.c_char_p, "p2hip_showdown_table_bytes": _L}
+_RESTYPE = {"p2hip_error_string": ctypes.c_char_p, "p2hip_showdown_table_bytes": _L,
+            "p2hip_tree_node_columns": _L}
 
 
 class P2HipError(RuntimeError):

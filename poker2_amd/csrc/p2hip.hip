@@ -8,6 +8,7 @@
 #include "cfr_iter.hip"
 #include "chance.hip"
 #include "best_response.hip"
+#include "tree.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

@@ -291,3 +291,120 @@ def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
                       legal_mask=legal, leaf_mask=leaf, new_street_mask=new_street,
                       fold_mask=(action == 0) & state["done"], showdown_mask=state["street"] == 4,
                       reward=reward, state=state, board=np.array(roots.board))
+
+
+# ---------------------------------------------------------------------------------------------
+# Device builder: the same tree, expanded by two HIP kernels per level.
+_DEVICE_COLS = ("street", "to_act", "button", "pot", "stack0", "stack1", "comm0", "comm1", "min_raise",
+                "actions_this_round", "allin0", "allin1", "start0", "start1", "done", "raises", "scale", "root",
+                "parent", "action", "reward")
+
+
+def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: int,
+                             max_raises: int | None = None, device="cuda") -> SparseTree:
+    """``build_sparse_tree`` on the GPU (``p2hip_tree_legal`` / ``p2hip_tree_step``): identical
+    arrays, bit for bit.  The returned tree also carries ``device_arrays`` — the index arrays as
+    resident torch tensors — so the evaluator does not upload them again.  One small
+    device-to-host read per level (the number of children) and one copy of the finished node
+    table back to the host."""
+    import ctypes
+
+    import torch
+
+    from . import _lib
+    if not _lib.hip_is_available():
+        raise RuntimeError("build_sparse_tree_device needs libp2hip.so and a GPU; use build_sparse_tree on the host.")
+    assert roots.n > 0, "must supply at least one root state"
+    bins = [float(b) for b in bet_bins]
+    if len(bins) > 5:
+        raise ValueError("at most 5 bet fractions (8 action bins) are supported")
+    nb = len(bins) + 3
+    n = roots.n
+    dev = torch.device(device)
+    cols = int(_lib.load().p2hip_tree_node_columns())
+    assert cols == len(_DEVICE_COLS)
+    host = np.zeros((n, cols), dtype=np.int64)
+    col = {name: i for i, name in enumerate(_DEVICE_COLS)}
+    for name in ("street", "to_act", "button", "pot", "min_raise", "actions_this_round", "done"):
+        host[:, col[name]] = np.asarray(getattr(roots, name)).astype(np.int64)
+    for name, src in (("stack", roots.stacks), ("comm", roots.committed), ("allin", roots.is_allin),
+                      ("start", roots.starting_stacks)):
+        host[:, col[name + "0"]] = np.asarray(src)[:, 0].astype(np.int64)
+        host[:, col[name + "1"]] = np.asarray(src)[:, 1].astype(np.int64)
+    host[:, col["scale"]] = np.asarray(roots.scale, dtype=np.float32).view(np.uint32).astype(np.int64)
+    host[:, col["root"]] = np.arange(n)
+    host[:, col["parent"]] = -1
+    host[:, col["action"]] = -1
+    bins_c = (ctypes.c_float * max(1, len(bins)))(*bins)
+    bins_p = ctypes.cast(bins_c, ctypes.c_void_p)
+    mr = -1 if max_raises is None else int(max_raises)
+    levels = [torch.from_numpy(host).to(dev)]
+    legal_l, count_l = [], []
+    offsets = [0, n]
+    d = 0
+    while True:
+        cur = levels[-1]
+        k = cur.shape[0]
+        expand = d < depth
+        legal = torch.empty(k, nb, dtype=torch.uint8, device=dev)
+        count = torch.empty(k, dtype=torch.int64, device=dev)
+        _lib.call("p2hip_tree_legal", _lib.ptr(cur), k, bins_p, len(bins), mr, int(d == 0), int(expand),
+                  _lib.ptr(legal), _lib.ptr(count), _lib.stream_ptr())
+        legal_l.append(legal)
+        count_l.append(count)
+        if not expand:
+            break
+        ends = torch.cumsum(count, 0)
+        n_next = int(ends[-1].item())
+        if n_next == 0:
+            break
+        start = (ends - count).contiguous()
+        child = torch.empty(n_next, cols, dtype=torch.int64, device=dev)
+        _lib.call("p2hip_tree_step", _lib.ptr(cur), k, int(offsets[-2]), bins_p, len(bins), mr, int(roots.bb),
+                  int(d == 0), _lib.ptr(start), _lib.ptr(child), _lib.stream_ptr())
+        levels.append(child)
+        offsets.append(offsets[-1] + n_next)
+        d += 1
+    nodes = torch.cat(levels) if len(levels) > 1 else levels[0]
+    legal = torch.cat(legal_l).bool()
+    child_count = torch.cat(count_l)
+    total = offsets[-1]
+    child_offsets = (n + torch.cumsum(child_count, 0) - child_count).contiguous()
+    table = nodes.cpu().numpy()                     # the one bulk copy back to the host
+
+    def c(name):
+        return np.ascontiguousarray(table[:, col[name]])
+    state = {
+        "street": c("street"), "to_act": c("to_act"), "button": c("button"), "pot": c("pot"),
+        "stacks": np.stack([c("stack0"), c("stack1")], axis=1),
+        "committed": np.stack([c("comm0"), c("comm1")], axis=1),
+        "min_raise": c("min_raise"), "actions_this_round": c("actions_this_round"),
+        "is_allin": np.stack([c("allin0"), c("allin1")], axis=1).astype(bool),
+        "starting_stacks": np.stack([c("start0"), c("start1")], axis=1),
+        "scale": c("scale").astype(np.uint32).view(np.float32), "done": c("done").astype(bool), "raises": c("raises"),
+    }
+    parent_index, action = c("parent"), c("action")
+    reward = c("reward").astype(np.uint32).view(np.float32)
+    is_root = np.zeros(total, dtype=bool)
+    is_root[:n] = True
+    new_street = (state["actions_this_round"] == 0) & ~is_root
+    leaf = state["done"] | new_street
+    leaf[offsets[-2]:] = True
+    cc = child_count.cpu().numpy()
+    assert total == n + int(cc.sum())
+    prev_actor = np.full(total, -1, dtype=np.int64)
+    prev_actor[n:] = state["to_act"][parent_index[n:]]
+    tree = SparseTree(depth_offsets=list(offsets), n_roots=n, total=total, num_actions=nb, bet_bins=bins,
+                      parent_index=parent_index, action_from_parent=action, child_count=cc,
+                      child_offsets=child_offsets.cpu().numpy(), prev_actor=prev_actor, root_index=c("root"),
+                      legal_mask=legal.cpu().numpy(), leaf_mask=leaf, new_street_mask=new_street,
+                      fold_mask=(action == 0) & state["done"], showdown_mask=state["street"] == 4,
+                      reward=reward, state=state, board=np.array(roots.board))
+    object.__setattr__(tree, "device_arrays", {
+        "parent_index": nodes[:, col["parent"]].contiguous(), "action_from_parent": nodes[:, col["action"]].contiguous(),
+        "child_count": child_count, "child_offsets": child_offsets, "root_index": nodes[:, col["root"]].contiguous(),
+        "legal_mask": legal, "to_act": nodes[:, col["to_act"]].contiguous(), "street": nodes[:, col["street"]].contiguous(),
+        "pot": nodes[:, col["pot"]].contiguous(), "button": nodes[:, col["button"]].contiguous(),
+        "actions_this_round": nodes[:, col["actions_this_round"]].contiguous(),
+    })
+    return tree

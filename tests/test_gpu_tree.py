@@ -1,0 +1,70 @@
+"""GPU: the device tree builder against the host builder (itself pinned by fixtures written from
+the reference's HUNLTensorEnv, tests/test_tree.py): every array identical, bit for bit."""
+import numpy as np
+import pytest
+
+from tests.helpers import random_boards
+
+pytestmark = pytest.mark.gpu
+
+FIELDS = ("parent_index", "action_from_parent", "child_count", "child_offsets", "prev_actor", "root_index",
+          "legal_mask", "leaf_mask", "new_street_mask", "fold_mask", "showdown_mask", "reward", "board")
+
+
+def same_tree(a, b):
+    assert a.depth_offsets == b.depth_offsets and a.total == b.total and a.num_actions == b.num_actions
+    for name in FIELDS:
+        x, y = getattr(a, name), getattr(b, name)
+        assert x.dtype == y.dtype and x.shape == y.shape, name
+        assert np.array_equal(x, y), name
+    assert set(a.state) == set(b.state)
+    for name in a.state:
+        x, y = a.state[name], b.state[name]
+        assert x.dtype == y.dtype and np.array_equal(x, y), name
+
+
+def random_roots(rng, n, street):
+    from poker2_amd.tree import RootStates
+    k = {1: 3, 2: 4, 3: 5, 0: 0}[street]
+    boards = np.full((n, 5), -1, dtype=np.int64)
+    if k:
+        boards[:, :k] = random_boards(rng, n, k)
+    pot = rng.integers(20, 600, n)
+    stacks = rng.integers(0, 3, (n, 2)) * rng.integers(50, 1500, (n, 2)) + rng.integers(1, 900, (n, 2))
+    return RootStates.at_round_start(street, pot, stacks, boards, button=rng.integers(0, 2, n), bb=rng.choice([10, 100]))
+
+
+@pytest.mark.parametrize("street,bins,depth,max_raises", [
+    (3, [0.5, 1.0], 2, None), (3, [0.5, 1.0], 16, 3), (2, [0.33, 0.75, 1.5], 4, None), (1, [1.0], 6, 2),
+    (3, [], 5, None), (2, [0.25, 0.5, 1.0, 2.0, 4.0], 3, None)])
+def test_device_builder_equals_host_builder(street, bins, depth, max_raises):
+    from poker2_amd.tree import build_sparse_tree, build_sparse_tree_device
+    rng = np.random.default_rng(100 * street + depth)
+    roots = random_roots(rng, 300, street)
+    host = build_sparse_tree(roots, bins, depth, max_raises=max_raises)
+    dev = build_sparse_tree_device(roots, bins, depth, max_raises=max_raises)
+    same_tree(host, dev)
+    for name, t in dev.device_arrays.items():
+        ref = getattr(host, name) if name in FIELDS else host.state[name]
+        assert np.array_equal(t.cpu().numpy(), ref), name
+
+
+def test_device_builder_from_mid_round_roots():
+    """Roots in the middle of a betting round (chips committed, a raise made, one player all-in):
+    the non-terminal nodes of another tree."""
+    from poker2_amd.tree import RootStates, build_sparse_tree, build_sparse_tree_device
+    rng = np.random.default_rng(7)
+    first = build_sparse_tree(random_roots(rng, 60, 2), [0.5, 1.0], 3)
+    rows = np.nonzero(~first.state["done"])[0]
+    fields = {}
+    for name in RootStates.__dataclass_fields__:
+        if name == "board":
+            fields[name] = first.board[first.root_index[rows]]
+        elif name == "bb":
+            fields[name] = 100
+        else:
+            fields[name] = np.asarray(first.state[name])[rows]
+    roots = RootStates(**fields)
+    assert roots.is_allin.any() and (roots.committed.sum(1) > 0).any()
+    same_tree(build_sparse_tree(roots, [0.5, 1.0], 4, max_raises=2),
+              build_sparse_tree_device(roots, [0.5, 1.0], 4, max_raises=2))
