@@ -38,7 +38,7 @@ from . import fused_cfr_hip as F
 from . import rules_hip
 from .card_utils import NUM_HANDS, combo_to_onehot_tensor
 from .fused_cfr_hip import CFRType
-from .tree import RootStates, SparseTree, build_sparse_tree
+from .tree import RootStates, SparseTree, build_sparse_tree, build_sparse_tree_device
 
 STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
                "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",
@@ -79,7 +79,7 @@ class SampledLeaves:
 class HipSparseCFREvaluator:
     def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
                  compile_model: bool = True, fused_iteration: bool = True,
-                 max_raises: int | None = None) -> None:
+                 max_raises: int | None = None, tree_builder: str = "device") -> None:
         self.model = model
         self.device = torch.device(device)
         self.cfg = cfg
@@ -116,6 +116,9 @@ class HipSparseCFREvaluator:
         self.generator = generator
         self.fused_iteration = bool(fused_iteration)
         self.max_raises = max_raises
+        if tree_builder not in ("device", "host"):
+            raise ValueError("tree_builder must be 'device' or 'host'")
+        self.tree_builder = tree_builder     # both give identical trees; 'host' is the numpy builder
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -150,8 +153,18 @@ class HipSparseCFREvaluator:
             roots = src_env.select(idx)
         else:
             roots = RootStates.from_env(src_env, src_indices)
-        tree = build_sparse_tree(roots, self.bet_bins, self.max_depth, max_raises=self.max_raises)
+        if self.tree_builder == "device":
+            tree = build_sparse_tree_device(roots, self.bet_bins, self.max_depth, max_raises=self.max_raises,
+                                            device=self.device)
+        else:
+            tree = build_sparse_tree(roots, self.bet_bins, self.max_depth, max_raises=self.max_raises)
         self.tree: SparseTree = tree
+        resident = getattr(tree, "device_arrays", None) or {}
+
+        def tt(name, host_array):
+            """The tree array as a device tensor: the builder's own tensor when it left one."""
+            t = resident.get(name)
+            return t if t is not None else self._t(host_array)
         dev = self.device
         self.depth_offsets = list(tree.depth_offsets)
         self.tree_depth = tree.tree_depth
@@ -160,23 +173,23 @@ class HipSparseCFREvaluator:
         self.top_nodes = tree.top
         T, N = tree.total, tree.n_roots
         self.valid_mask = torch.ones(T, dtype=torch.bool, device=dev)
-        self.parent_index = self._t(tree.parent_index)
-        self.action_from_parent = self._t(tree.action_from_parent)
-        self.child_count = self._t(tree.child_count)
-        self.child_offsets = self._t(tree.child_offsets)
+        self.parent_index = tt("parent_index", tree.parent_index)
+        self.action_from_parent = tt("action_from_parent", tree.action_from_parent)
+        self.child_count = tt("child_count", tree.child_count)
+        self.child_offsets = tt("child_offsets", tree.child_offsets)
         self.prev_actor = self._t(tree.prev_actor)
-        self.legal_mask = self._t(tree.legal_mask)
+        self.legal_mask = tt("legal_mask", tree.legal_mask)
         self.leaf_mask = self._t(tree.leaf_mask)
         self.new_street_mask = self._t(tree.new_street_mask)
         self.child_mask = self.legal_mask & (~self.leaf_mask)[:, None]
         st = tree.state
         self.env = SimpleNamespace(
-            N=T, to_act=self._t(st["to_act"]), done=self._t(st["done"]), street=self._t(st["street"]),
-            pot=self._t(st["pot"]), stacks=self._t(st["stacks"]), committed=self._t(st["committed"]),
+            N=T, to_act=tt("to_act", st["to_act"]), done=self._t(st["done"]), street=tt("street", st["street"]),
+            pot=tt("pot", st["pot"]), stacks=self._t(st["stacks"]), committed=self._t(st["committed"]),
             starting_stacks=self._t(st["starting_stacks"]), scale=self._t(st["scale"]),
-            actions_this_round=self._t(st["actions_this_round"]), button=self._t(st["button"]),
+            actions_this_round=tt("actions_this_round", st["actions_this_round"]), button=tt("button", st["button"]),
             board_indices=self._t(tree.board[tree.root_index]), bb=roots.bb)
-        self._root_index = self._t(tree.root_index)
+        self._root_index = tt("root_index", tree.root_index)
         model_mask = tree.leaf_mask & ~st["done"]
         self.model_indices = self._t(np.nonzero(model_mask)[0].astype(np.int64))
         self.showdown_indices = self._t(np.nonzero(tree.showdown_mask)[0].astype(np.int64))
