@@ -15,7 +15,9 @@ a parent and ``dev`` the deviating player there:
                  the other player).
 Leaf rows keep ``base_values``.
 
-Pinned by (tests/test_oracle_best_response.py): an exact best response on the explicit
+Pinned by the reference's own numbers (local exploitability and best-response values of six
+searches in tests/golden/cfr_golden.npz, and the ``model_br`` warm start, which is built on
+these values) and by (tests/test_oracle_best_response.py) an exact best response on the explicit
 hand-pair game (every compatible pair enumerated) — per-hand root values of the deviating
 player agree for random full-support strategies at depths 2-4 — and by
 best response >= on-policy value, with equality when the strategy already is a best response.

@@ -20,18 +20,23 @@ the sparse tree helpers of ``src/p2/search/sparse_cfr_evaluator.py``:
   apply_schedules                          <- :1294-1328
   cfr_iteration                            <- :1330-1381
   evaluate_cfr (loop part)                 <- :1497-1528
+  warm_start                               <- :888-955
 
 Every state tensor keeps the reference's name, shape and meaning; a child's row
 holds the quantity "for the action that leads to it".  Arithmetic is float32
 with Python-scalar operands rounded to float32 first, as torch does.
 
-PARITY UNPINNED by reference-held numbers: the reference ships no multi-
-iteration values for this path.  The restatement is pinned instead by (a) the
-golden tree / ranker fixtures underneath it, (b) structural identities
-(sibling policies sum to 1, beliefs sum to 1, reach non-increasing down the
-tree, zero-sum after the zero-sum step), (c) a textbook scalar CFR and a
-brute-force best response on tiny ranges agreeing on the game value
-(tests/test_oracle_cfr.py).
+PINNED by vectors written from the reference itself: tests/golden/cfr_golden.npz holds the
+11 state tensors of the reference's own SparseCFREvaluator (run on the CPU of the build
+container by tests/golden/gen_cfr_golden.py) after the preparation step and after iterations
+of six searches — discounted, discounted_plus with delay, linear + CFR+ + cfr_avg, standard,
+warm start ``model_br`` and ``model``; depths 2 and 3 — and its local exploitability;
+tests/test_oracle_cfr_golden.py holds this restatement to them (1e-5 relative on the first
+iterations).  Further pinned by (tests/test_oracle_cfr.py) an explicit hand-pair game that
+reproduces reach, conditional values and regrets at depths 2-4, the closed form of the average
+policy, a textbook CFR / best response, and structural identities.  The ``fused_variant``
+switches (what FusedSparseCFREvaluator does differently on rows / hands without probability
+mass) are read off the source and agree with the base variant wherever mass lives.
 """
 from __future__ import annotations
 

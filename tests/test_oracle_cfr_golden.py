@@ -1,0 +1,72 @@
+"""CPU: the oracle's whole CFR iteration against vectors written by RUNNING the reference's own
+SparseCFREvaluator in the build container (tests/golden/gen_cfr_golden.py).  Six searches
+(discounted, discounted_plus with delay, linear + CFR+ + cfr_avg, standard, and two that start
+from the reference's warm start; depths 2 and 3): the preparation step, the first iterations,
+the sampling iteration and the last one, all 11 state tensors."""
+import numpy as np
+import pytest
+
+from oracle import cfr as OCFR
+from oracle import tree as OT
+
+STATE = OCFR.OracleCFR.STATE_NAMES
+
+
+@pytest.fixture(scope="module")
+def golden(golden_dir):
+    return np.load(str(golden_dir) + "/cfr_golden.npz")
+
+
+def build(golden, name):
+    cfr_type, cfr_plus, cfr_avg, delay, depth, iters, warm, warm_type, warm_mult = golden[f"{name}/settings"]
+    rows = golden[f"{name}/rows"]
+    roots = [OT.make_root(3, int(p), int(s0), int(s1), button=int(b)) for p, s0, s1, b in rows]
+    t = OT.build_tree(roots, [0.5, 1.0], int(depth))
+    # same tree as the reference built
+    assert list(t["depth_offsets"]) == list(golden[f"{name}/depth_offsets"])
+    for k in ("parent_index", "action_from_parent", "child_count", "child_offsets", "prev_actor", "to_act"):
+        assert np.array_equal(np.asarray(t[k]), golden[f"{name}/{k}"]), k
+    n = len(rows)
+    t_sample = np.full(n, -1, dtype=np.int64)
+    t_sample[0] = 2
+    o = OCFR.OracleCFR(t, golden[f"{name}/board"], golden[f"{name}/beliefs"], cfr_type=str(cfr_type),
+                       cfr_plus=cfr_plus == "True", cfr_avg=cfr_avg == "True", dcfr_delay=int(delay),
+                       dcfr_alpha=1.5, dcfr_beta=0.0, dcfr_gamma=2.0, cfr_iterations=50, enforce_zero_sum=True,
+                       t_sample_roots=t_sample, warm_start_iterations=int(warm), warm_start_type=str(warm_type),
+                       warm_start_multiplier=float(warm_mult))
+    return o, int(warm), int(iters)
+
+
+def check(o, golden, name, tag, rtol, atol):
+    cols = golden["columns"]
+    for s in STATE:
+        got = getattr(o, s)
+        exp = golden[f"{name}/{tag}/{s}"]
+        err = np.abs(got[..., cols] - exp) - (atol + rtol * np.abs(exp))
+        # elements on the algorithm's hard thresholds may differ by more: exempt by count
+        assert (err > 0).sum() <= max(2, 1e-4 * err.size), \
+            f"{name} {tag} {s}: max abs diff {np.abs(got[..., cols] - exp).max():.3e}"
+        assert np.abs(got[..., cols] - exp).max() < 1e-3, f"{name} {tag} {s}"
+        np.testing.assert_allclose(got.astype(np.float64).sum(-1), golden[f"{name}/{tag}/{s}_rowsum"],
+                                   rtol=max(rtol, 1e-4), atol=1e-3, err_msg=f"{name} {tag} {s} row sums")
+
+
+@pytest.mark.parametrize("name", ["discounted_d2", "dplus_d3", "linear_avg_d2", "standard_d2", "warm_br_d2",
+                                  "warm_model_d2"])
+def test_oracle_iterations_match_reference_vectors(golden, name):
+    o, warm, iters = build(golden, name)
+    o.prepare()                                   # includes the warm start of the last two cases
+    check(o, golden, name, "prep", rtol=1e-5, atol=1e-6)
+    stored = set(golden[f"{name}/stored"].tolist())
+    for t in range(warm, iters):
+        o.cfr_iteration(t)
+        if t in stored:
+            # float32, 1e-5 relative on the first iterations; rounding differences between numpy
+            # and torch reductions grow slowly afterwards
+            tol = 1e-5 if t < warm + 2 else 1e-4
+            check(o, golden, name, f"t{t}", rtol=tol, atol=tol / 10)
+    # the reference's own local exploitability of the final average strategy (:718-764)
+    from oracle import best_response as OBR
+    expl, br = OBR.compute_exploitability(o)
+    np.testing.assert_allclose(expl, golden[f"{name}/local_exploitability"], rtol=1e-3, atol=2e-5)
+    np.testing.assert_allclose(br, golden[f"{name}/local_best_response_values"], rtol=1e-3, atol=2e-5)
