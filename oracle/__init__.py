@@ -9,13 +9,15 @@ never as a compute path that ships.
 Every function restates, in numpy (plus a small C file for the integer
 ranker), what the reference computes, and cites the reference file:line it
 follows.  How each function is pinned (reference-held vectors, golden fixtures
-written by running the reference's own ``rules.py`` / ``hunl_tensor_env.py`` in
-the build container, closed forms, brute force) is listed per module.
+written by running the reference's own ``rules.py`` / ``hunl_tensor_env.py`` /
+``sparse_cfr_evaluator.py`` in the build container, closed forms, brute force) is
+listed per module.
 
 Parity status
 -------------
 * cards, ranker, unblocked mass, showdown, betting tree: pinned (see modules).
-* cfr (multi-iteration numeric values): **parity unpinned** by any
-  reference-held vector; pinned only by per-step identities, game-theoretic
-  invariants and brute force on tiny ranges (see ``oracle/cfr.py``).
+* cfr, warm start, best response / exploitability: pinned by vectors written from the
+  reference's own evaluator (``tests/golden/cfr_golden.npz``) and by an explicit hand-pair
+  game (see ``oracle/cfr.py``, ``oracle/best_response.py``).
+* chance node: pinned by per-sample loops and closed forms (``oracle/chance.py``).
 """
