@@ -38,6 +38,7 @@ CASES = [
     ("discounted_d2", "discounted", False, False, 0, 2, 6, [(200, 800, 800, 0), (200, 800, 800, 1)], (0, "model_br", 1.0)),
     ("dplus_d3", "discounted_plus", False, False, 2, 3, 6, [(300, 500, 900, 1), (120, 2000, 700, 0)], (0, "model_br", 1.0)),
     ("linear_avg_d2", "linear", True, True, 0, 2, 5, [(200, 800, 800, 0)], (0, "model_br", 1.0)),
+    ("linear_noplus_d2", "linear", False, True, 0, 2, 5, [(200, 800, 800, 1)], (0, "model_br", 1.0)),
     ("standard_d2", "standard", False, False, 0, 2, 4, [(450, 300, 300, 1)], (0, "model_br", 1.0)),
     ("warm_br_d2", "discounted_plus", False, False, 4, 2, 7, [(200, 800, 800, 1)], (3, "model_br", 1.0)),
     ("warm_model_d2", "discounted", False, False, 0, 2, 6, [(260, 700, 900, 0)], (3, "model", 10.0)),

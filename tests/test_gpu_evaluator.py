@@ -290,3 +290,69 @@ def test_sample_leaves_walks_the_sampled_policy():
     ev2.prepare_search()
     ev2.cfr_iteration(0)
     assert torch.isfinite(ev2.values_avg).all()
+
+
+# ---- the product against vectors written by running the reference's own evaluator -----------
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("name", ["discounted_d2", "dplus_d3", "linear_noplus_d2", "standard_d2", "warm_br_d2",
+                                  "warm_model_d2"])
+def test_product_matches_reference_vectors(golden_dir, name, fused):
+    """tests/golden/cfr_golden.npz holds state tensors of the reference's SparseCFREvaluator (its
+    base torch path).  The product follows the fused evaluator, which differs from the base class
+    only on hands that carry no probability mass (board-blocked hands); on every other entry the
+    two must agree, so the comparison runs over the hands the board allows.  (The fixture's
+    linear + CFR+ search is left out: the fused evaluator accumulates linear-CFR regrets without
+    the CFR+ clamp of the base class, fused_sparse_cfr_evaluator.py:503-507.)"""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType
+    from poker2_amd.tree import RootStates
+    from oracle import cards as OC
+    g = np.load(str(golden_dir) + "/cfr_golden.npz")
+    cfr_type, cfr_plus, cfr_avg, delay, depth, iters, warm, warm_type, warm_mult = g[f"{name}/settings"]
+    rows, board, bel = g[f"{name}/rows"], g[f"{name}/board"], g[f"{name}/beliefs"]
+    n = len(rows)
+    roots = RootStates.at_round_start(3, rows[:, 0], rows[:, 1:3], board, button=rows[:, 3])
+    cfg = river_dcfr_config(n, iterations=50, depth=int(depth), dcfr_delay=int(delay))
+    cfg.search.cfr_type = CFRType[str(cfr_type)]
+    cfg.search.cfr_plus = cfr_plus == "True"
+    cfg.search.cfr_avg = cfr_avg == "True"
+    cfg.search.warm_start_iterations = int(warm)
+    cfg.search.warm_start_type = str(warm_type)
+    cfg.search.warm_start_multiplier = float(warm_mult)
+
+    class ZeroModel:                                   # the reference run used a zero-value network
+        enforce_zero_sum = True
+
+        def leaf_values(self, beliefs, rows_, ev_):
+            return torch.zeros_like(beliefs)
+    ev = HipSparseCFREvaluator(ZeroModel(), torch.device("cuda"), cfg, fused_iteration=fused)
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(bel))
+    assert list(ev.depth_offsets) == list(g[f"{name}/depth_offsets"])
+    t_sample = torch.full((ev.total_nodes,), -1, dtype=torch.long)
+    t_sample[ev._root_index.cpu() == 0] = 2
+    ev.prepare_search(t_sample=t_sample)
+    cols = g["columns"]
+    allowed = OC.allowed_hands_for_boards(board)[0][ev.tree.root_index][:, cols]       # [total, 128]
+
+    def check(tag, rtol, atol):
+        for s in OCFR.OracleCFR.STATE_NAMES:
+            got = getattr(ev, s).cpu().numpy()[..., cols]
+            exp = g[f"{name}/{tag}/{s}"]
+            m = allowed if got.ndim == 2 else np.broadcast_to(allowed[:, None, :], got.shape)
+            err = (np.abs(got - exp) - (atol + rtol * np.abs(exp)))[m]
+            assert (err > 0).sum() <= max(2, 1e-4 * err.size), \
+                f"{name} {tag} {s}: max abs diff {np.abs(got - exp)[m].max():.3e}"
+            assert np.abs(got - exp)[m].max() < 2e-3, f"{name} {tag} {s}"
+    check("prep", 1e-5, 2e-6)
+    stored = set(g[f"{name}/stored"].tolist())
+    for t in range(int(warm), int(iters)):
+        ev.cfr_iteration(t)
+        if t in stored:
+            # float32 throughout; regret matching divides by small sums, so a relative 1e-5 in the
+            # regrets shows as ~5e-5 in a policy and in the reach products built from it
+            tol = 5e-5 if t < int(warm) + 2 else 3e-4
+            check(f"t{t}", tol, tol / 5)
+    stats = ev._compute_exploitability()
+    np.testing.assert_allclose(stats.local_exploitability.cpu().numpy(), g[f"{name}/local_exploitability"],
+                               rtol=2e-3, atol=5e-5)
