@@ -11,7 +11,9 @@ Follows ``ChanceNodeHelper.single_card_chance_values``
   mean     :467-477  sum of the network's hand values per state / number of its samples; the
                      hands that hold the dealt card are NOT excluded from the mean
 
-Pinned by (tests/test_oracle_chance.py): a per-sample Python loop written from the docstring
+Pinned by vectors written from the reference's own helper (tests/golden/chance_golden.npz,
+made by tests/golden/gen_chance_golden.py: echo and board-and-range networks, mixed turn / flop
+boards, dead and delta ranges) and by (tests/test_oracle_chance.py) a per-sample Python loop written from the docstring
 above, closed forms for an echo network (mean of the renormalised ranges), a board-only
 network (mean over cards of a function of the board), sample counts 52 - k, and the
 reference's own empty / shape cases (tests/test_chance_node_helper.py:426-478).

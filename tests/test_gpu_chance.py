@@ -198,3 +198,30 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused, streets):
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
         compare(ev, orc, rtol=1e-3, atol=3e-4)
+
+
+def test_helper_matches_vectors_from_the_reference_helper(K, golden_dir):
+    """The HIP path against tests/golden/chance_golden.npz (written by running the reference's own
+    ChanceNodeHelper.single_card_chance_values): bit-for-bit sample order is implied by the mean
+    of a board-dependent network; values within float32 1e-5 relative."""
+    g = np.load(str(golden_dir) + "/chance_golden.npz")
+    board, pre, roots = g["board"], g["pre_beliefs"], g["root_indices"]
+    n = board.shape[0]
+    dev = torch.device("cuda")
+
+    class BoardAndRange:
+        def eval(self):
+            pass
+
+        def __call__(self, f):
+            b = f.beliefs.view(-1, 2, H).float()
+            ranks = torch.where(f.board >= 0, (f.board % 13).float(), torch.zeros_like(f.board, dtype=torch.float32))
+            return SimpleNamespace(hand_values=b * (1.0 + ranks.sum(dim=1) / 100.0)[:, None, None])
+    feats = K.MLPFeatures(context=torch.zeros(n, 1, device=dev), street=torch.full((n,), 3, dtype=torch.long, device=dev),
+                          to_act=torch.zeros(n, dtype=torch.long, device=dev), board=torch.from_numpy(board).to(dev),
+                          beliefs=torch.zeros(n, 2 * H, device=dev))
+    for name, model in (("echo", EchoModel()), ("board_and_range", BoardAndRange())):
+        helper = K.ChanceNodeHelper(dev, torch.float32, 2, model, autocast_dtype=None)
+        got = helper.single_card_chance_values(torch.from_numpy(roots).to(dev), feats, torch.from_numpy(pre).to(dev),
+                                               torch.from_numpy(board).to(dev))
+        np.testing.assert_allclose(got.cpu().numpy(), g[name], rtol=1e-5, atol=1e-8)

@@ -104,3 +104,23 @@ def test_empty_input_and_shapes():
     out = OCH.single_card_chance_values(np.arange(4), np.zeros((4, 1)), np.zeros(4), np.zeros(4), pre, boards,
                                         lambda c, s, t, b, x: np.zeros((b.shape[0], 2, H), np.float32))
     assert out.shape == (4, 2, H) and out.dtype == np.float32 and not out.any()
+
+
+def test_oracle_matches_vectors_from_the_reference_helper(golden_dir):
+    """tests/golden/chance_golden.npz: outputs of the reference's own single_card_chance_values
+    (run by tests/golden/gen_chance_golden.py) for an echo network and a board-and-range network,
+    mixed turn / flop boards, a dead range and a delta range."""
+    g = np.load(str(golden_dir) + "/chance_golden.npz")
+    board, pre, roots = g["board"], g["pre_beliefs"], g["root_indices"]
+    n = board.shape[0]
+
+    def echo(context, street, to_act, b, beliefs):
+        return beliefs.reshape(-1, 2, H)
+
+    def board_and_range(context, street, to_act, b, beliefs):
+        w = 1.0 + np.where(b >= 0, b % 13, 0).sum(axis=1).astype(np.float32) / np.float32(100.0)
+        return beliefs.reshape(-1, 2, H) * w[:, None, None]
+    for name, fn in (("echo", echo), ("board_and_range", board_and_range)):
+        got = OCH.single_card_chance_values(roots, np.zeros((n, 1), np.float32), np.full(n, 3), np.zeros(n, np.int64),
+                                            pre, board, fn)
+        np.testing.assert_allclose(got, g[name], rtol=1e-5, atol=1e-8)
