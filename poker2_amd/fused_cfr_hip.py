@@ -472,3 +472,30 @@ class TScalars:
             self.mix_onon.fill_(total / float(mix_new))
             self.mix_oon.fill_(float(mix_old) / float(mix_new))
         self.t_tensor.fill_(int(t))
+
+
+class ParentBeliefUnblockedStats:
+    """Total and per-card sums of both players' beliefs at the parent rows
+    (fused_cfr_triton.py:1029-1064).  The HIP kernels take their card sums inside the kernel, so
+    passing this object as ``cached_stats`` changes nothing; it exists for callers that build it."""
+
+    def __init__(self, beliefs_parents: torch.Tensor) -> None:
+        assert beliefs_parents.dim() == 3 and beliefs_parents.shape[1] == 2
+        self.top = beliefs_parents.shape[0]
+        self.beliefs_parents = beliefs_parents
+
+    def slice_for_player(self, player_per_node: torch.Tensor):
+        from .card_utils import combo_to_onehot_tensor
+        rows = torch.arange(self.top, device=self.beliefs_parents.device)
+        target = self.beliefs_parents[rows, player_per_node, :].contiguous()
+        onehot = combo_to_onehot_tensor(device=target.device).to(target.dtype)
+        return target, target.sum(dim=-1), target @ onehot
+
+
+def __getattr__(name):
+    # GraphedCFRIteration lives with the evaluator (which imports this module); the reference
+    # exports it from fused_cfr_triton.py:2359-2451
+    if name == "GraphedCFRIteration":
+        from .evaluator import GraphedCFRIteration
+        return GraphedCFRIteration
+    raise AttributeError(name)

@@ -8,12 +8,38 @@ the current stream; there is no CPU path.
 """
 from __future__ import annotations
 
+from enum import Enum
+
 import torch
 
 from . import _lib
 from ._lib import hip_is_available
 
 NUM_HANDS = 1326
+
+
+class HandType(Enum):
+    """Hand categories = field 0 of the comparison vector (src/p2/env/rules.py:17-28)."""
+    NUM_HAND_TYPES = 10
+    STRAIGHT_FLUSH = 9
+    FOUR_OF_A_KIND = 8
+    FULL_HOUSE = 7
+    FLUSH = 6
+    STRAIGHT = 5
+    THREE_OF_A_KIND = 4
+    TWO_PAIR = 3
+    ONE_PAIR = 2
+    HIGH_CARD = 1
+    EMPTY = 0
+
+
+def rank(card: int) -> int:
+    """src/p2/env/rules.py: rank 0..12 = 2..A of card = suit * 13 + rank."""
+    return card % 13
+
+
+def suit(card: int) -> int:
+    return card // 13
 
 
 def triton_is_available() -> bool:
@@ -58,6 +84,29 @@ def compare_7_batches_triton(a_batch: torch.Tensor, b_batch: torch.Tensor) -> to
     if a_batch.dim() != 3 or tuple(a_batch.shape[1:]) != (4, 13):
         raise ValueError(f"Expected [N, 4, 13] inputs, got {tuple(a_batch.shape)}")
     return compare_7_single_batch_triton(torch.stack([a_batch, b_batch], dim=1).bool())
+
+
+def create_comparison_vector(ab_batch: torch.Tensor) -> torch.Tensor:
+    """[N, P, 4, 13] planes -> [N, P, 6] int32 (hand type, five rank fields; 0 where unused), the
+    vector whose nibble packing is the score (src/p2/env/rules.py:136-299, :406-407)."""
+    _require_backend()
+    if ab_batch.dim() != 4 or tuple(ab_batch.shape[2:]) != (4, 13):
+        raise ValueError(f"Expected [N, P, 4, 13] input, got {tuple(ab_batch.shape)}")
+    n, p = ab_batch.shape[:2]
+    packed = rank_7_planes(ab_batch.reshape(n * p, 4, 13)).view(n, p)
+    shifts = torch.tensor([20, 16, 12, 8, 4, 0], device=packed.device, dtype=torch.int32)
+    return (packed[..., None] >> shifts) & 0xF
+
+
+def compare_7(a_cards, b_cards) -> int:
+    """Two lists of 7 card ids -> 1 / -1 / 0 (src/p2/env/rules.py:358-387)."""
+    assert len(a_cards) == 7, f"Expected 7 cards for hand A, got {len(a_cards)}"
+    assert len(b_cards) == 7, f"Expected 7 cards for hand B, got {len(b_cards)}"
+    planes = torch.zeros(1, 2, 4, 13, dtype=torch.bool)
+    for p, cards in enumerate((a_cards, b_cards)):
+        for card in cards:
+            planes[0, p, card // 13, card % 13] = True
+    return int(compare_7_single_batch(planes.cuda())[0].item())
 
 
 def compare_7_single_batch(ab_batch: torch.Tensor) -> torch.Tensor:

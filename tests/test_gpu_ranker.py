@@ -116,3 +116,27 @@ def test_rank_hands_golden_and_oracle(K, golden_dir):
     for dt in (torch.int8, torch.int16, torch.int32, torch.int64):
         p, o = K.rank_hands_triton(torch.from_numpy(b).to(dt).cuda())
         assert np.array_equal(p.cpu().numpy(), ep) and np.array_equal(o.cpu().numpy(), eo2)
+
+
+def test_comparison_vector_and_scalar_compare(K, golden_dir):
+    """create_comparison_vector / compare_7 / HandType of src/p2/env/rules.py against the fields
+    the reference itself produced for the golden hands."""
+    g = np.load(str(golden_dir) + "/ranker_golden.npz")
+    cards, fields = g["cards"].astype(np.int64), g["fields"].astype(np.int32)
+    n = 1024
+    planes = np.zeros((n, 1, 4, 13), dtype=bool)
+    for i in range(n):
+        planes[i, 0, cards[i] // 13, cards[i] % 13] = True
+    got = K.create_comparison_vector(torch.from_numpy(planes).cuda()).cpu().numpy()
+    assert got.shape == (n, 1, 6) and np.array_equal(got[:, 0], fields[:n])
+    assert {int(x) for x in np.unique(got[:, 0, 0])} <= {t.value for t in K.HandType}
+    for i in range(0, 40, 2):
+        exp = int(np.sign(int(g["packed"][i]) - int(g["packed"][i + 1])))
+        assert K.compare_7(cards[i].tolist(), cards[i + 1].tolist()) == exp
+    from poker2_amd import fused_cfr_hip as F
+    from poker2_amd.evaluator import GraphedCFRIteration
+    assert F.GraphedCFRIteration is GraphedCFRIteration
+    stats = F.ParentBeliefUnblockedStats(torch.rand(5, 2, 1326, device="cuda"))
+    t, s, cs = stats.slice_for_player(torch.tensor([0, 1, 1, 0, 1], device="cuda"))
+    assert t.shape == (5, 1326) and s.shape == (5,) and cs.shape == (5, 52)
+    torch.testing.assert_close(cs.sum(-1), 2 * s, rtol=1e-5, atol=1e-5)
