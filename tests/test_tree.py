@@ -77,3 +77,28 @@ def test_full_river_tree_is_terminal_and_max_raises_extension():
     assert capped.total < full.total
     with pytest.raises(AssertionError):
         build_sparse_tree(RootStates.at_round_start(3, np.zeros(0), np.zeros((0, 2)), np.zeros((0, 5))), [0.5], 2)
+
+
+def test_roots_from_an_env_like_object_with_torch_tensors():
+    """RootStates.from_env reads the attribute names of the reference's HUNLTensorEnv
+    (hunl_tensor_env.py:130-135,296) from torch tensors and selects rows."""
+    import types
+
+    import torch
+    from poker2_amd.tree import RootStates, build_sparse_tree
+    n = 5
+    base = RootStates.at_round_start(3, np.arange(n) * 50 + 100, np.tile([[900, 700]], (n, 1)),
+                                     np.tile(np.arange(5), (n, 1)), button=np.arange(n) % 2, bb=10)
+    env = types.SimpleNamespace(bb=10)
+    for name in ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",
+                 "is_allin", "starting_stacks", "scale", "done"):
+        setattr(env, name, torch.from_numpy(np.asarray(getattr(base, name))))
+    env.board_indices = torch.from_numpy(base.board)
+    idx = torch.tensor([4, 1, 2])
+    roots = RootStates.from_env(env, idx)
+    ref = base.select(np.array([4, 1, 2]))
+    for name in RootStates.__dataclass_fields__:
+        a, b = getattr(roots, name), getattr(ref, name)
+        assert np.array_equal(a, b) if isinstance(a, np.ndarray) else a == b, name
+    t1, t2 = build_sparse_tree(roots, [0.5, 1.0], 2), build_sparse_tree(ref, [0.5, 1.0], 2)
+    assert t1.total == t2.total and np.array_equal(t1.child_count, t2.child_count)
