@@ -16,7 +16,7 @@ zero-value / uniform-policy mock network like the reference's own ``MockModel``
 (tests/test_sparse_cfr_evaluator.py:43-86), seeded Dirichlet ranges.  The fixture stores the
 inputs (boards, ranges, chips, settings), the tree arrays, and after the preparation step and
 the first two iterations, the sampling iteration and the last one, the 11 state tensors
-restricted to 128 seeded hand columns plus their full row sums (float64).  Two cases start from
+restricted to 64 seeded hand columns plus their full row sums (float64).  Two cases start from
 the reference's warm start (``model_br`` and ``model``).
 """
 from __future__ import annotations
@@ -105,7 +105,7 @@ def main() -> None:
             pass
 
     rng = np.random.default_rng(2024)
-    cols = np.sort(rng.choice(NUM_HANDS, 128, replace=False))
+    cols = np.sort(rng.choice(NUM_HANDS, 64, replace=False))
     out = {"columns": cols, "case_names": np.array([c[0] for c in CASES])}
     dev = torch.device("cpu")
     for name, cfr_type, cfr_plus, cfr_avg, delay, depth, iters, rows, (warm, warm_type, warm_mult) in CASES:
