@@ -285,6 +285,12 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max
  * soon as the call returns.  Plays the role of TScalars.update, search/fused_cfr_triton.py:2131-2158. */
 int p2hip_write_scalars(float* fscal, int64_t* iscal, const float* host_f, const int64_t* host_i, void* stream);
 
+/* dst[0..n) (device, n <= 8) = host_values[0..n): the values travel as kernel arguments, in
+ * stream order, so the scalar-taking wrappers (fused_dcfr_update_ etc., fused_cfr_triton.py:123-197)
+ * need no host-to-device copies.  No counterpart in the reference, which passes Python floats to
+ * Triton. */
+int p2hip_upload_floats(float* dst, const float* host_values, int n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -583,6 +583,13 @@ __global__ void write_scalars_kernel(float* __restrict__ fscal, int64_t* __restr
   }
 }
 
+struct FloatPack { float f[8]; };
+
+__global__ void upload_floats_kernel(float* __restrict__ dst, FloatPack v, int n) {
+  const int k = threadIdx.x;
+  if (k < n) dst[k] = v.f[k];
+}
+
 }  // namespace p2
 
 extern "C" {
@@ -607,6 +614,16 @@ int p2hip_write_scalars(float* fscal, int64_t* iscal, const float* host_f, const
     v.i[k] = host_i[k];
   }
   hipLaunchKernelGGL(p2::write_scalars_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, fscal, iscal, v);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_upload_floats(float* dst, const float* host_values, int n, void* stream) {
+  if (!dst || !host_values || n < 0 || n > 8) return P2_EINVAL;
+  if (n == 0) return 0;
+  p2::FloatPack v;
+  for (int k = 0; k < 8; ++k) v.f[k] = k < n ? host_values[k] : 0.f;
+  hipLaunchKernelGGL(p2::upload_floats_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, dst, v, n);
   P2_LAUNCH_CHECK();
   return 0;
 }

@@ -39,8 +39,19 @@ def _need() -> None:
         raise RuntimeError("libp2hip.so or a GPU is not available; there is no other backend.")
 
 
+def _scalars(values, like: torch.Tensor):
+    """Python floats -> 0-dim float32 device tensors, written by ONE tiny kernel whose arguments
+    carry the values (stream ordered; no host-to-device copies)."""
+    import ctypes
+    n = len(values)
+    buf = torch.empty(n, dtype=torch.float32, device=like.device)
+    host = (ctypes.c_float * n)(*[float(v) for v in values])
+    _lib.call("p2hip_upload_floats", _lib.ptr(buf), ctypes.cast(host, ctypes.c_void_p), n, _lib.stream_ptr())
+    return [buf[k] for k in range(n)]
+
+
 def _scalar(value: float, like: torch.Tensor) -> torch.Tensor:
-    return torch.tensor(float(value), dtype=like.dtype, device=like.device)
+    return _scalars([value], like)[0]
 
 
 _S = _lib.stream_ptr
@@ -67,7 +78,7 @@ def fused_dcfr_update_(cumulative_regrets, regret_weight_sums, regrets, t: int, 
         vals = (a, b, a + 1.0, b + 1.0)
     else:
         vals = (1.0, 1.0, 1.0, 1.0)
-    an, bn, ad, bd = (_scalar(v, cumulative_regrets) for v in vals)
+    an, bn, ad, bd = _scalars(vals, cumulative_regrets)
     fused_dcfr_update_with_tensors_(cumulative_regrets, regret_weight_sums, regrets, an, bn, ad, bd, apply_dcfr,
                                     cfr_plus, positive_regrets_out=positive_regrets_out, block_size=block_size)
 
@@ -146,9 +157,8 @@ def fused_update_average_values_(values_avg, latest_values, old: float, new: flo
     assert values_avg.shape == latest_values.shape
     total = float(old) + float(new)
     assert total != 0.0
-    fused_update_average_values_with_tensors_(values_avg, latest_values, _scalar(old, values_avg),
-                                              _scalar(new, values_avg), _scalar(1.0 / total, values_avg),
-                                              block_size=block_size)
+    o_t, n_t, inv_t = _scalars([old, new, 1.0 / total], values_avg)
+    fused_update_average_values_with_tensors_(values_avg, latest_values, o_t, n_t, inv_t, block_size=block_size)
 
 
 def fused_update_average_values_with_tensors_(values_avg, latest_values, old, new, inv_total,
@@ -216,10 +226,9 @@ def fused_average_policy_mix_(policy_probs_avg, policy_probs, self_reach, self_r
     assert parent_index.shape == (total,)
     total_weight = float(old) + float(new)
     assert total_weight != 0.0
+    o_t, n_t, tot_t = _scalars([old, new, total_weight], policy_probs_avg)
     fused_average_policy_mix_with_tensors_(policy_probs_avg, policy_probs, self_reach, self_reach_avg, to_act,
-                                           parent_index, _scalar(old, policy_probs_avg),
-                                           _scalar(new, policy_probs_avg), _scalar(total_weight, policy_probs_avg),
-                                           bottom=bottom, eps=eps, block_h=block_h)
+                                           parent_index, o_t, n_t, tot_t, bottom=bottom, eps=eps, block_h=block_h)
 
 
 def fused_average_policy_mix_with_tensors_(policy_probs_avg, policy_probs, self_reach, self_reach_avg, to_act,
@@ -343,8 +352,8 @@ def fused_model_values_mix(hand_values, last_model_values, old: float, new: floa
     assert hand_values.shape == last_model_values.shape
     assert new != 0.0
     out = torch.empty_like(hand_values)
-    fused_model_values_mix_with_tensors(hand_values, last_model_values, _scalar((old + new) / new, hand_values),
-                                        _scalar(old / new, hand_values), out, block_size=block_size)
+    onon_t, oon_t = _scalars([(old + new) / new, old / new], hand_values)
+    fused_model_values_mix_with_tensors(hand_values, last_model_values, onon_t, oon_t, out, block_size=block_size)
     return out
 
 
