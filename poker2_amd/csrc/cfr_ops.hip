@@ -19,7 +19,10 @@ constexpr int FLAT_BLOCK = 256;
 
 static inline unsigned flat_grid(int64_t npairs) {
   int64_t g = (npairs + FLAT_BLOCK - 1) / FLAT_BLOCK;
-  const int64_t cap = 256 * 64;  // grid-stride beyond this
+  // One pair per lane up to 2^30 workgroups: workgroups start in address order, which keeps the
+  // DRAM accesses of the whole chip sequential in time; a capped grid with a long stride between a
+  // lane's iterations measured 20 % slower (4.97 vs 5.92 TB/s on the DCFR update).
+  const int64_t cap = (int64_t)1 << 30;
   return (unsigned)(g < cap ? g : cap);
 }
 
