@@ -61,9 +61,9 @@ __device__ __forceinline__ float unblocked_at(const float* t, const double* cs, 
 }
 
 // ---- standalone kernels -------------------------------------------------------------
-// A workgroup takes UB_ROWS vectors at a time and walks the groups with a grid stride.  The
-// next group's rows are fetched into registers while the current one is reduced out of LDS,
-// so enough bytes stay in flight per CU to cover HBM latency.
+// A workgroup takes a group of UB_ROWS vectors: rows through registers into LDS, one card-sum pass
+// for the group, outputs.  The launch gives every group its own workgroup (see ub_grid); the
+// group loop with its register prefetch of the next group only repeats on grids that were capped.
 constexpr int UB_ROWS = 4;
 constexpr int UB_PPT = 3;                  // float2 pairs per thread and row: 3 * 256 >= 663
 constexpr int UB_STRIDE = P2_H + 2;
