@@ -356,3 +356,51 @@ def test_product_matches_reference_vectors(golden_dir, name, fused):
     stats = ev._compute_exploitability()
     np.testing.assert_allclose(stats.local_exploitability.cpu().numpy(), g[f"{name}/local_exploitability"],
                                rtol=2e-3, atol=5e-5)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_one_kernel_and_per_op_paths_agree_on_random_subgames(seed):
+    """Seeded sweep over tree shapes the other tests do not reach: random chips (including short
+    stacks that remove bets and leave one- and two-child families), one to five bet fractions (up
+    to 8 children), depths 1-5, raise caps, CFR variants.  The two product paths share no kernel
+    for the iteration itself, so their agreement checks each against the other."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(1, 6))
+    all_bins = [0.25, 0.5, 0.75, 1.0, 2.0]
+    bins = sorted(rng.choice(all_bins, size=int(rng.integers(1, 6)), replace=False).tolist())
+    depth = int(rng.integers(1, 6))
+    max_raises = [None, 1, 2, 3][int(rng.integers(0, 4))]
+    cfr_type = ["discounted", "discounted_plus", "standard", "linear"][int(rng.integers(0, 4))]
+    boards = random_boards(rng, n)
+    beliefs = random_ranges(rng, boards)
+    pot = rng.integers(40, 900, n)
+    stacks = rng.integers(30, 2500, (n, 2))
+    roots = RootStates.at_round_start(3, pot, stacks, boards, button=rng.integers(0, 2, n), bb=int(rng.choice([10, 100])))
+    evs = []
+    for fused in (True, False):
+        cfg = river_dcfr_config(n, iterations=20, depth=depth, dcfr_delay=int(rng.integers(0, 3)) if fused else 0)
+        if not fused:
+            cfg.search.dcfr_plus_delay = evs[0].dcfr_delay
+        cfg.search.cfr_type = CFRType[cfr_type]
+        cfg.search.cfr_plus = bool(seed % 2)
+        cfg.search.cfr_avg = bool((seed // 2) % 2)
+        cfg.env.bet_bins = bins
+        ev = HipSparseCFREvaluator(None, torch.device("cuda"), cfg, fused_iteration=fused, max_raises=max_raises,
+                                   tree_builder="device" if fused else "host")
+        ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), 1, dtype=torch.long))
+        evs.append(ev)
+    a, b = evs
+    assert a.total_nodes == b.total_nodes
+    for t in range(4):
+        a.cfr_iteration(t)
+        b.cfr_iteration(t)
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        x, y = getattr(a, name), getattr(b, name)
+        bad = ((x - y).abs() > 2e-5 + 2e-4 * y.abs()).float().mean().item()
+        assert bad <= 1e-3, f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type}: {name} {bad:.2e} " \
+                            f"max {float((x - y).abs().max()):.3e}"
