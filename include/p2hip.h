@@ -87,6 +87,19 @@ int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, c
 int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, int64_t n, float* expected,
                       void* stream);
 
+/* Three-card (flop) chance node, flop_chance_values of search/chance_node_helper.py:219-357.
+ * out [n, n_flops, 2, H]: the ranges of state i (row root_indices[i] of pre_beliefs [*,2,H], NULL =
+ * identity) with the hands holding a card of flops[f] (int64 [n_flops,3]) removed, renormalised per
+ * player (uniform over the 1176 surviving hands when the sum is <= 1e-12). */
+int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int64_t n, const int64_t* flops,
+                      int64_t n_flops, float* out, void* stream);
+
+/* out [n,2,H] (+= if accumulate) sum_f weight[f] * mean_q hand_values[i][f][p][perms[q][h]]:
+ * hand_values [n, n_flops, 2, H], perms int16 [n_perms <= 24, H] hand permutations (the suit-orbit
+ * mean of _avg_over_perms, :18-28, and the weighted flop sum, :352-357). */
+int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
+                    const float* weight, int accumulate, float* out, void* stream);
+
 /* ---- local best response -------------------------------------------------------------- */
 
 /* One tree level of _best_response_values (search/cfr_evaluator.py:636-714), in place on

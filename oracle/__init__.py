@@ -19,6 +19,7 @@ Parity status
 * cfr, warm start, best response / exploitability: pinned by vectors written from the
   reference's own evaluator (``tests/golden/cfr_golden.npz``) and by an explicit hand-pair
   game (see ``oracle/cfr.py``, ``oracle/best_response.py``).
-* chance node: pinned by vectors written from the reference's own helper
-  (``tests/golden/chance_golden.npz``), per-sample loops and closed forms (``oracle/chance.py``).
+* chance nodes (one card, flop): pinned by vectors written from the reference's own helper
+  (``tests/golden/chance_golden.npz``, ``flop_chance_golden.npz``), per-sample loops and closed
+  forms (``oracle/chance.py``).
 """

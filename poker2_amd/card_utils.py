@@ -79,6 +79,32 @@ def combo_compatible_tensor(device: torch.device | None = None) -> torch.Tensor:
     return out if device is None else out.to(device)
 
 
+def suit_permutations_tensor(device: torch.device | None = None) -> torch.Tensor:
+    """[24, 4] int64: every permutation of the four suits, lexicographic (card_utils.py:153-158)."""
+    from itertools import permutations
+    perms = torch.tensor(tuple(permutations(range(4))), dtype=torch.long)
+    return perms if device is None else perms.to(device)
+
+
+@lru_cache(maxsize=8)
+def combo_suit_permutation_tensor(device: torch.device | None = None) -> torch.Tensor:
+    """[24, 1326] int64: index of the combo each combo becomes when the suits are permuted
+    (card_utils.py:161-181)."""
+    combos = hand_combos_tensor()
+    ranks, suits = combos % 13, combos // 13
+    cards = suit_permutations_tensor()[:, suits] * 13 + ranks[None]          # [24, 1326, 2]
+    lo, hi = cards.min(dim=2).values, cards.max(dim=2).values
+    out = combo_lookup_tensor()[lo, hi]
+    return out if device is None else out.to(device)
+
+
+@lru_cache(maxsize=8)
+def combo_suit_permutation_inverse_tensor(device: torch.device | None = None) -> torch.Tensor:
+    """[24, 1326] int64: argsort of ``combo_suit_permutation_tensor`` per row (card_utils.py:184-193)."""
+    inv = torch.argsort(combo_suit_permutation_tensor(), dim=1)
+    return inv if device is None else inv.to(device)
+
+
 def calculate_unblocked_mass(target: torch.Tensor) -> torch.Tensor:
     """[..., 1326] -> same shape: mass of the combos sharing no card with each combo,
     clamped at 0 (card_utils.py:196-222).  Runs ``p2hip_unblocked_mass``."""

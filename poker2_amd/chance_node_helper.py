@@ -6,8 +6,9 @@ to the network (src/p2/models/mlp/mlp_features.py:13-62): same names, arguments,
 order (state-major, next card ascending) and return value.  The masking / renormalising
 expansion and the per-state mean run as HIP kernels (``p2hip_chance_expand``,
 ``p2hip_chance_mean``); the network itself stays an ordinary PyTorch module.
-``flop_chance_values`` (three-card chance nodes through the canonical-flop cache) is not
-part of this package.
+``flop_chance_values`` (three-card chance nodes, :219-357) enumerates or samples the 1755
+suit-canonical flops (:76-216), expands through ``p2hip_flop_expand`` and averages each flop's
+answers over its suit orbit with ``p2hip_perm_mean``.
 """
 from __future__ import annotations
 
@@ -16,8 +17,10 @@ from typing import Any
 
 import torch
 
+import numpy as np
+
 from . import _lib
-from .card_utils import NUM_HANDS
+from .card_utils import NUM_HANDS, combo_suit_permutation_tensor, suit_permutations_tensor
 
 
 @dataclass
@@ -106,9 +109,95 @@ def chance_mean(hand_values: torch.Tensor, sample_offsets: torch.Tensor) -> torc
     return out
 
 
+def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, flops: torch.Tensor) -> torch.Tensor:
+    """pre_chance_beliefs [R,2,1326] fp32, root_indices [B], flops [K,3] card ids ->
+    [B,K,2,1326]: the ranges of each selected state without the hands that touch each flop,
+    renormalised per player (uniform over the 1176 hands left where the sum is <= 1e-12)."""
+    if not _lib.hip_is_available():
+        raise RuntimeError("flop_expand needs libp2hip.so and a GPU (no CPU fallback exists).")
+    _lib.require_gpu(pre_chance_beliefs, "flop_expand")
+    dev = pre_chance_beliefs.device
+    assert pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS)
+    assert flops.dim() == 2 and flops.shape[1] == 3
+    pre = pre_chance_beliefs.contiguous().float()
+    roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
+    if roots.numel() and (int(roots.min()) < 0 or int(roots.max()) >= pre.shape[0]):
+        raise IndexError("root_indices out of range")
+    fl = flops.to(device=dev, dtype=torch.int64).contiguous()
+    b, k = roots.numel(), fl.shape[0]
+    post = torch.empty(b, k, 2, NUM_HANDS, dtype=torch.float32, device=dev)
+    _lib.call("p2hip_flop_expand", _lib.ptr(pre), _lib.ptr(roots), b, _lib.ptr(fl), k, _lib.ptr(post),
+              _lib.stream_ptr())
+    return post
+
+
+def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tensor,
+              out: torch.Tensor | None = None) -> torch.Tensor:
+    """hand_values [B,K,2,1326] fp32, perms [P,1326] hand-index maps (P <= 24), weight [K] ->
+    [B,2,1326]: sum_k weight[k] * mean_q hand_values[b,k,p,perms[q,h]]; added to ``out`` if given."""
+    if not _lib.hip_is_available():
+        raise RuntimeError("perm_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
+    _lib.require_gpu(hand_values, "perm_mean")
+    dev = hand_values.device
+    assert hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)
+    assert perms.dim() == 2 and perms.shape[1] == NUM_HANDS and 1 <= perms.shape[0] <= 24
+    b, k = hand_values.shape[0], hand_values.shape[1]
+    assert weight.shape == (k,)
+    hv = hand_values.contiguous().float()
+    pt = perms.to(device=dev, dtype=torch.int16).contiguous()
+    w = weight.to(device=dev, dtype=torch.float32).contiguous()
+    accumulate = out is not None
+    if out is None:
+        out = torch.empty(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
+    else:
+        assert out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()
+    _lib.call("p2hip_perm_mean", _lib.ptr(hv), b, k, _lib.ptr(pt), int(pt.shape[0]), _lib.ptr(w), int(accumulate),
+              _lib.ptr(out), _lib.stream_ptr())
+    return out
+
+
+def canonical_flops():
+    """The suit-canonical flops (src/p2/search/chance_node_helper.py:76-216), on the host.
+
+    Every flop's cards are ordered by rank, high first; under each of the 24 suit permutations
+    the suits of equal ranks are put in ascending order and the three cards are read as a base-52
+    number; the smallest number over the permutations is the flop's canonical form.  Returns
+    (canonical [1755,3] int64 cards in that order, count [1755] int64 flops per class,
+    flop_to_class [22100] int64 in itertools.combinations order, board_to_flop_id [52,52,52] int64
+    with -1 off the c0 < c1 < c2 entries)."""
+    from itertools import combinations
+    flops = np.array(list(combinations(range(52), 3)), dtype=np.int64)            # [22100, 3], ascending ids
+    ranks, suits = flops % 13, flops // 13
+    order = np.argsort(-ranks, axis=1, kind="stable")
+    ranks_s = np.take_along_axis(ranks, order, axis=1)
+    perms = suit_permutations_tensor().numpy()                                     # [24, 4]
+    suits_p = np.take_along_axis(perms[:, suits], np.broadcast_to(order, (24,) + order.shape), axis=2)  # [24,N,3]
+    eq01, eq12 = ranks_s[:, 0] == ranks_s[:, 1], ranks_s[:, 1] == ranks_s[:, 2]
+    all_eq, first2, last2 = eq01 & eq12, eq01 & ~eq12, eq12 & ~eq01
+    suits_p[:, all_eq, :] = np.sort(suits_p[:, all_eq, :], axis=2)
+    suits_p[:, first2, :2] = np.sort(suits_p[:, first2, :2], axis=2)
+    suits_p[:, last2, 1:] = np.sort(suits_p[:, last2, 1:], axis=2)
+    cards = suits_p * 13 + ranks_s[None]
+    code = cards[..., 0] * 2704 + cards[..., 1] * 52 + cards[..., 2]               # [24, N]
+    best = code.min(axis=0)
+    unique, flop_to_class = np.unique(best, return_inverse=True)
+    canonical = np.stack([unique // 2704, (unique // 52) % 52, unique % 52], axis=1).astype(np.int64)
+    count = np.bincount(flop_to_class, minlength=unique.shape[0]).astype(np.int64)
+    board_to_flop_id = np.full((52, 52, 52), -1, dtype=np.int64)
+    board_to_flop_id[flops[:, 0], flops[:, 1], flops[:, 2]] = flop_to_class
+    return canonical, count, flop_to_class.astype(np.int64), board_to_flop_id
+
+
 class ChanceNodeHelper:
     """Utilities for enumerating chance nodes when generating value targets
-    (src/p2/search/chance_node_helper.py:31-75; the canonical-flop cache is not built)."""
+    (src/p2/search/chance_node_helper.py:31-75)."""
+
+    FLOP_CHUNK_SIZE = 128
+    # Canonical flops drawn per call with probability proportional to their class size; 0 = all
+    # 1755 classes, weighted by class size, in chunks of FLOP_CHUNK_SIZE (:36-38)
+    FLOP_SAMPLE_SIZE = 256
+    # Suit permutations averaged per flop; 0 or >= 24 = the whole orbit (:39-42)
+    NUM_PERM_SAMPLES = 6
 
     def __init__(self, device: torch.device, float_dtype: torch.dtype, num_players: int, model: Any,
                  generator: torch.Generator | None = None, autocast_dtype: torch.dtype | None = torch.float16) -> None:
@@ -120,9 +209,79 @@ class ChanceNodeHelper:
         self.model = model
         self.generator = generator
         self.autocast_dtype = autocast_dtype   # the reference runs the network under fp16 autocast (:460)
+        self.suit_permutations = suit_permutations_tensor(device=self.device)
+        self.num_permutations = self.suit_permutations.shape[0]
+        self.combo_perm = combo_suit_permutation_tensor(device=self.device)
+        self._combo_perm_i16 = self.combo_perm.to(torch.int16).contiguous()
+        canonical, count, flop_to_class, board_to_flop_id = canonical_flops()
+        self.flop_id_to_canonical = torch.from_numpy(canonical).to(self.device)
+        self.flop_id_to_count = torch.from_numpy(count).to(self.device)
+        self.board_to_flop_id = torch.from_numpy(board_to_flop_id).to(self.device)
+        self.flop_to_canon = torch.from_numpy(flop_to_class).to(self.device)
+        self.total_flop_count = int(count.sum())
 
-    def flop_chance_values(self, *args, **kwargs):
-        raise NotImplementedError("three-card chance nodes (canonical-flop cache) are not part of this package")
+    def _run_model(self, features: MLPFeatures) -> torch.Tensor:
+        model = self.model
+        if hasattr(model, "eval"):
+            model.eval()
+        if self.autocast_dtype is not None:
+            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                hand_values = model(features).hand_values
+        else:
+            hand_values = model(features).hand_values
+        return hand_values.to(torch.float32)
+
+    @torch.no_grad()
+    def flop_chance_values(self, root_indices: torch.Tensor, root_features: MLPFeatures,
+                           pre_chance_beliefs: torch.Tensor) -> torch.Tensor:
+        """Expected network values over the three-card flop chance node (:219-357): the canonical
+        flops (all of them weighted by class size, or FLOP_SAMPLE_SIZE drawn in proportion to it),
+        each answer averaged over NUM_PERM_SAMPLES suit permutations of the hands (all 24 if 0)."""
+        if not _lib.hip_is_available():
+            raise RuntimeError("flop_chance_values needs libp2hip.so and a GPU (no CPU fallback exists).")
+        if root_indices.numel() == 0:
+            return torch.zeros(0, self.num_players, NUM_HANDS, device=self.device, dtype=self.float_dtype)
+        dev = self.device
+        roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
+        b = roots.numel()
+        pre = pre_chance_beliefs.to(device=dev).contiguous().float()
+        _lib.require_gpu(pre, "flop_chance_values")
+        context_root = root_features.context[roots]
+        street_root = root_features.street[roots]
+        to_act_root = root_features.to_act[roots]
+        num_flops = self.flop_id_to_canonical.shape[0]
+        gdev = self.generator.device if self.generator is not None else dev
+        out = torch.zeros(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
+
+        def eval_chunk(canonical_chunk: torch.Tensor, weight: torch.Tensor) -> None:
+            k = canonical_chunk.shape[0]
+            flops = canonical_chunk.contiguous()
+            post = flop_expand(pre, roots, flops)
+            board5 = torch.cat([flops, torch.full((k, 2), -1, device=dev, dtype=torch.int64)], dim=1)
+            feats = MLPFeatures(
+                context=context_root.unsqueeze(1).expand(-1, k, -1).reshape(-1, context_root.shape[1]),
+                street=street_root.unsqueeze(1).expand(-1, k).reshape(-1),
+                to_act=to_act_root.unsqueeze(1).expand(-1, k).reshape(-1),
+                board=board5.unsqueeze(0).expand(b, -1, -1).reshape(-1, 5),
+                beliefs=post.reshape(b * k, -1).to(self.float_dtype))
+            hv = self._run_model(feats).reshape(b, k, 2, NUM_HANDS).contiguous()
+            p = self.NUM_PERM_SAMPLES
+            if 0 < p < self.num_permutations:
+                perm_idx = torch.randperm(self.num_permutations, device=gdev, generator=self.generator)[:p].to(dev)
+            else:
+                perm_idx = torch.arange(self.num_permutations, device=dev)
+            perm_mean(hv, self._combo_perm_i16[perm_idx], weight, out=out)
+
+        s = self.FLOP_SAMPLE_SIZE
+        if 0 < s < num_flops:
+            probs = self.flop_id_to_count.to(torch.float32)
+            idx = torch.multinomial(probs.to(gdev), s, replacement=True, generator=self.generator).to(dev)
+            eval_chunk(self.flop_id_to_canonical[idx], torch.full((s,), 1.0 / s))
+            return out.to(self.float_dtype)
+        for start in range(0, num_flops, self.FLOP_CHUNK_SIZE):
+            end = min(start + self.FLOP_CHUNK_SIZE, num_flops)
+            eval_chunk(self.flop_id_to_canonical[start:end], self.flop_id_to_count[start:end].to(torch.float32))
+        return (out / float(self.total_flop_count)).to(self.float_dtype)
 
     @torch.no_grad()
     def single_card_chance_values(self, root_indices: torch.Tensor, root_features: MLPFeatures,
@@ -145,13 +304,5 @@ class ChanceNodeHelper:
             board=board_samples,
             beliefs=post.reshape(post.shape[0], -1).to(self.float_dtype),
         )
-        model = self.model
-        if hasattr(model, "eval"):
-            model.eval()
-        if self.autocast_dtype is not None:
-            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
-                hand_values = model(synthetic_features).hand_values
-        else:
-            hand_values = model(synthetic_features).hand_values
-        expected = chance_mean(hand_values.to(torch.float32), offsets)
+        expected = chance_mean(self._run_model(synthetic_features), offsets)
         return expected.to(self.float_dtype)

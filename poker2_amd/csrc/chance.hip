@@ -166,6 +166,142 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_mean_kernel(const float* __re
   }
 }
 
+// ---- three-card (flop) chance node ------------------------------------------------------
+// flop_chance_values (src/p2/search/chance_node_helper.py:219-357): every state is expanded over
+// a list of candidate flops (the canonical ones, or a sample of them); a hand survives a flop
+// if it holds none of its three cards, the survivors are renormalised (uniform over them if the
+// sum is <= 1e-12).  By inclusion-exclusion the surviving mass of a range is
+//   T - cs[a] - cs[b] - cs[c] + t[ab] + t[ac] + t[bc]
+// so again one card-sum pass per state serves all of its flops.  out is [n, flops, 2, H].
+__global__ __launch_bounds__(CH_BLOCK) void flop_expand_kernel(const float* __restrict__ pre_beliefs,
+                                                                const int64_t* __restrict__ root_indices,
+                                                                const int64_t* __restrict__ flops, int64_t n_flops,
+                                                                float* __restrict__ out) {
+  __shared__ __align__(8) float t[2][P2_H + 2];
+  __shared__ double cs[2 * P2_CARDS];
+  const int64_t i = blockIdx.x;
+  const int64_t root = root_indices ? root_indices[i] : i;
+  float v[2][CH_PPT][2];
+  uint32_t ab[CH_PPT][2];
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    const bool in = idx < P2_HPAIRS;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int h = in ? 2 * idx + q : 0;
+      ab[k][q] = (uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8);
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      float2 x = make_float2(0.f, 0.f);
+      if (in) {
+        x = p2_row2(pre_beliefs, root * 2 + p)[idx];
+        reinterpret_cast<float2*>(t[p])[idx] = x;
+      }
+      v[p][k][0] = x.x;
+      v[p][k][1] = x.y;
+    }
+  }
+  p2_sync_lds();
+  card_sums_multi(t[0], P2_H + 2, 2, cs);
+  const double total[2] = {card_total(cs), card_total(cs + P2_CARDS)};
+  const float uniform = 1.0f / (float)(49 * 48 / 2);   // hands left once three cards are out
+  // blockIdx.y takes every gridDim.y-th flop
+  for (int64_t f = blockIdx.y; f < n_flops; f += gridDim.y) {
+    int c[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) c[j] = (int)flops[f * 3 + j];
+    bool valid = true;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) valid = valid && c[j] >= 0 && c[j] < P2_CARDS;
+    valid = valid && c[0] != c[1] && c[0] != c[2] && c[1] != c[2];
+    float inv[2];
+    bool ok[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      double sum = 0.0;
+      if (valid) {
+        sum = total[p];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) sum -= cs[p * P2_CARDS + c[j]];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          const int x = c[j], y = c[(j + 1) % 3];
+          sum += (double)t[p][p2_combo_index(x < y ? x : y, x < y ? y : x)];
+        }
+      }
+      const float sf = (float)sum;
+      ok[p] = sf > 1e-12f;
+      inv[p] = 1.0f / fmaxf(sf, 1e-12f);
+    }
+    float2* o0 = p2_row2(out, ((int64_t)i * n_flops + f) * 2);
+    float2* o1 = p2_row2(out, ((int64_t)i * n_flops + f) * 2 + 1);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx >= P2_HPAIRS) continue;
+      float r0[2], r1[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int a = (int)(ab[k][q] & 0xFFu), b = (int)(ab[k][q] >> 8);
+        const bool off = !valid || a == c[0] || a == c[1] || a == c[2] || b == c[0] || b == c[1] || b == c[2];
+        r0[q] = off ? 0.f : (ok[0] ? v[0][k][q] * inv[0] : uniform);
+        r1[q] = off ? 0.f : (ok[1] ? v[1][k][q] * inv[1] : uniform);
+      }
+      o0[idx] = make_float2(r0[0], r0[1]);
+      o1[idx] = make_float2(r1[0], r1[1]);
+    }
+  }
+}
+
+// out[i][p][h] (+)= sum_f weight[f] * mean_q hand_values[i][f][p][perms[q][h]]
+// (the suit-orbit mean of _avg_over_perms, chance_node_helper.py:18-28, and the weighted sum over
+// flops, :352-357).  One workgroup per (state, player); the permutation table lives in LDS.
+constexpr int CH_MAX_PERMS = 24;
+__global__ __launch_bounds__(CH_BLOCK) void perm_mean_kernel(const float* __restrict__ hand_values,
+                                                              const int16_t* __restrict__ perms, int n_perms,
+                                                              const float* __restrict__ weight, int64_t n_flops,
+                                                              int accumulate, float* __restrict__ out) {
+  extern __shared__ __align__(8) unsigned char lds_raw[];
+  float* row = reinterpret_cast<float*>(lds_raw);                          // [H + 2]
+  int16_t* ptab = reinterpret_cast<int16_t*>(lds_raw + (P2_H + 2) * 4);    // [n_perms][H]
+  const int64_t i = blockIdx.x;
+  const int p = blockIdx.y;
+  for (int e = threadIdx.x; e < n_perms * P2_H; e += CH_BLOCK) ptab[e] = perms[e];
+  double acc[CH_PPT][2];
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) acc[k][0] = acc[k][1] = 0.0;
+  const float inv_perms = 1.0f / (float)n_perms;
+  for (int64_t f = 0; f < n_flops; ++f) {
+    p2_sync_lds();   // the previous row has been consumed (and, first time, ptab is complete)
+    const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
+    for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += CH_BLOCK) reinterpret_cast<float2*>(row)[idx] = src[idx];
+    p2_sync_lds();
+    const float w = weight[f];
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx >= P2_HPAIRS) continue;
+#pragma unroll
+      for (int q2 = 0; q2 < 2; ++q2) {
+        const int h = 2 * idx + q2;
+        float s = 0.f;
+        for (int q = 0; q < n_perms; ++q) s += row[ptab[q * P2_H + h]];
+        acc[k][q2] += (double)(w * (s * inv_perms));
+      }
+    }
+  }
+  float2* o = p2_row2(out, i * 2 + p);
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    if (idx >= P2_HPAIRS) continue;
+    float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
+    o[idx] = make_float2(prev.x + (float)acc[k][0], prev.y + (float)acc[k][1]);
+  }
+}
+
 }  // namespace p2
 
 extern "C" {
@@ -192,6 +328,37 @@ int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, i
   if (!p2_aligned8(hand_values) || !p2_aligned8(expected)) return P2_EINVAL;
   hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)n), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
                      hand_values, sample_offsets, expected);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int64_t n, const int64_t* flops,
+                      int64_t n_flops, float* out, void* stream) {
+  if (n < 0 || n_flops < 0) return P2_EINVAL;
+  if (n == 0 || n_flops == 0) return 0;
+  if (!pre_beliefs || !flops || !out || !p2_aligned8(pre_beliefs) || !p2_aligned8(out)) return P2_EINVAL;
+  if (n > 0x7FFFFFFF) return P2_EINVAL;
+  const unsigned split = (unsigned)(n_flops < 16 ? n_flops : 16);
+  hipLaunchKernelGGL(p2::flop_expand_kernel, dim3((unsigned)n, split), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     pre_beliefs, root_indices, flops, n_flops, out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
+                    const float* weight, int accumulate, float* out, void* stream) {
+  if (n < 0 || n_flops < 0 || n_perms < 1 || n_perms > p2::CH_MAX_PERMS) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!hand_values || !perms || !weight || !out || !p2_aligned8(hand_values) || !p2_aligned8(out)) return P2_EINVAL;
+  if (n > 0x7FFFFFFF) return P2_EINVAL;
+  const size_t lds = (size_t)(P2_H + 2) * 4 + (size_t)n_perms * P2_H * 2;   // 69 KB with all 24 permutations
+  if (lds > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(p2::perm_mean_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  hipLaunchKernelGGL(p2::perm_mean_kernel, dim3((unsigned)n, 2), dim3(p2::CH_BLOCK), lds, (hipStream_t)stream,
+                     hand_values, perms, n_perms, weight, n_flops, accumulate, out);
   P2_LAUNCH_CHECK();
   return 0;
 }

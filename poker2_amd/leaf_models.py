@@ -5,7 +5,8 @@ The evaluator asks its ``model`` for ``leaf_values(beliefs[K,2,1326], node_rows[
 are evaluated on their own board; leaves where the round has ended and a card is still to
 come are expanded over every card that can come next (blocker masking, renormalisation,
 network, mean — the semantics of ``ChanceNodeHelper.single_card_chance_values``,
-src/p2/search/chance_node_helper.py:360-479).  The network stays ordinary PyTorch; only the
+src/p2/search/chance_node_helper.py:360-479), and leaves where the preflop round has ended
+over the canonical flops (``flop_chance_values``, :219-357).  The network stays ordinary PyTorch; only the
 expansion and the mean are HIP kernels.
 
 ``RangeBoardMLP`` is the network of the turn benchmark configuration: input 2 x 1326 ranges +
@@ -45,7 +46,7 @@ class RangeBoardMLP(torch.nn.Module):
 
 
 class ChanceLeafModel:
-    """Evaluator leaf protocol on top of a value network and the single-card chance node."""
+    """Evaluator leaf protocol on top of a value network and the chance nodes (one card, flop)."""
 
     def __init__(self, net, device, *, enforce_zero_sum: bool = False, autocast_dtype: torch.dtype | None = None,
                  max_samples_per_call: int = 1 << 19) -> None:
@@ -64,11 +65,13 @@ class ChanceLeafModel:
         tree = ev.tree
         board = tree.board[tree.root_index[r]]
         on_board = (board >= 0).sum(axis=1)
-        chance = tree.new_street_mask[r] & (on_board < 5)
+        flop = tree.new_street_mask[r] & (on_board == 0)      # preflop betting closed: three cards come
+        chance = tree.new_street_mask[r] & (on_board < 5) & ~flop
         dev = self.device
         plan = SimpleNamespace(
             direct=torch.from_numpy(np.nonzero(~chance)[0]).to(dev),
             chance=torch.from_numpy(np.nonzero(chance)[0]).to(dev),
+            flop=torch.from_numpy(np.nonzero(flop)[0]).to(dev),
             board=torch.from_numpy(board).to(dev),
             street=ev.env.street[rows].to(torch.long),
             to_act=ev.env.to_act[rows].to(torch.long),
@@ -109,4 +112,11 @@ class ChanceLeafModel:
                 ev_chance = self.helper.single_card_chance_values(sel, feats, beliefs, plan.board,
                                                                   cards_on_board=plan.cards)
                 out.index_copy_(0, sel, ev_chance.to(out.dtype))
+        if plan.flop.numel():
+            feats = self._features(beliefs, plan)
+            flops_per_call = self.helper.FLOP_SAMPLE_SIZE or self.helper.FLOP_CHUNK_SIZE
+            step = max(1, self.max_samples_per_call // flops_per_call)
+            for lo in range(0, plan.flop.numel(), step):
+                sel = plan.flop[lo:lo + step]
+                out.index_copy_(0, sel, self.helper.flop_chance_values(sel, feats, beliefs).to(out.dtype))
         return out

@@ -1,5 +1,6 @@
-"""GPU parity of the single-card chance node (expansion + mean kernels and the
-ChanceNodeHelper mirror) against the oracle, on the cases of the reference's
+"""GPU parity of the chance nodes (single card: expansion + mean kernels; flop: expansion +
+suit-orbit mean kernels; the ChanceNodeHelper mirror) against the oracle and the vectors written
+by the reference's own helper, on the cases of the reference's
 tests/test_chance_node_helper.py:426-590 and on seeded mixed-street inputs."""
 from types import SimpleNamespace
 
@@ -119,8 +120,10 @@ def test_helper_edge_cases(K):
     full = torch.arange(5, device=dev)[None]                 # a river board has no chance card left
     with pytest.raises(ValueError):
         K.chance_expand(torch.rand(1, 2, H, device=dev), torch.zeros(1, dtype=torch.long, device=dev), full)
-    with pytest.raises(NotImplementedError):
-        helper.flop_chance_values()
+    out = helper.flop_chance_values(torch.zeros(0, dtype=torch.long, device=dev), empty, torch.zeros(0, 2, H, device=dev))
+    assert out.shape == (0, 2, H)
+    with pytest.raises(IndexError):                          # a state index beyond the ranges is refused on the host
+        K.flop_expand(torch.rand(2, 2, H, device=dev), torch.tensor([2], device=dev), torch.tensor([[0, 1, 2]], device=dev))
     # the fixed-count fast path gives the same samples
     rng = np.random.default_rng(9)
     boards, pre = inputs(rng, 3, [4])
@@ -225,3 +228,114 @@ def test_helper_matches_vectors_from_the_reference_helper(K, golden_dir):
         got = helper.single_card_chance_values(torch.from_numpy(roots).to(dev), feats, torch.from_numpy(pre).to(dev),
                                                torch.from_numpy(board).to(dev))
         np.testing.assert_allclose(got.cpu().numpy(), g[name], rtol=1e-5, atol=1e-8)
+
+
+# ---- three-card (flop) chance node -------------------------------------------------------------
+def test_flop_expand_matches_oracle(K):
+    rng = np.random.default_rng(21)
+    pre = rng.gamma(0.5, size=(5, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    pre[1, 0] = 0.0                      # dead range -> uniform over the 1176 hands left
+    pre[3, 1] = 0.0
+    pre[3, 1, 0] = 1.0                   # delta on hand (0,1): dead on flops holding card 0 or 1
+    flops = np.stack([rng.permutation(52)[:3] for _ in range(37)]).astype(np.int64)   # any card order, > 16 flops
+    flops[0] = [0, 13, 26]
+    flops[1] = [5, 1, 40]
+    roots = np.array([4, 1, 3, 3, 0])
+    got = K.flop_expand(torch.from_numpy(pre).cuda(), torch.from_numpy(roots).cuda(),
+                        torch.from_numpy(flops).cuda()).cpu().numpy()
+    exp = OCH.flop_expand(pre[roots], flops)
+    assert got.shape == (5, 37, 2, H)
+    assert ((got == 0) == (exp == 0)).all()                              # the mask is exact
+    np.testing.assert_allclose(got, exp, rtol=1e-5, atol=1e-9)           # float32 tolerance 1e-5 relative
+    np.testing.assert_allclose(got.sum(-1), 1.0, rtol=1e-5)
+    # no flops: an empty result, no launch
+    assert K.flop_expand(torch.from_numpy(pre).cuda(), torch.from_numpy(roots).cuda(),
+                         torch.zeros(0, 3, dtype=torch.long).cuda()).shape == (5, 0, 2, H)
+
+
+@pytest.mark.parametrize("n_perms", [1, 6, 24])
+def test_perm_mean_matches_numpy(K, n_perms):
+    rng = np.random.default_rng(22 + n_perms)
+    perms = OCH.combo_suit_perms()[rng.permutation(24)[:n_perms]]
+    hv = rng.standard_normal((3, 11, 2, H)).astype(np.float32)
+    w = rng.random(11).astype(np.float32)
+    exp = np.zeros((3, 2, H))
+    for k in range(11):
+        exp += w[k] * np.mean([hv[:, k][..., q] for q in perms], axis=0, dtype=np.float64)
+    got = K.perm_mean(torch.from_numpy(hv).cuda(), torch.from_numpy(perms).cuda(), torch.from_numpy(w).cuda())
+    np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=2e-6)
+    # accumulation onto an earlier result
+    again = K.perm_mean(torch.from_numpy(hv).cuda(), torch.from_numpy(perms).cuda(), torch.from_numpy(w).cuda(),
+                        out=got.clone())
+    np.testing.assert_allclose(again.cpu().numpy(), 2 * exp, rtol=1e-5, atol=4e-6)
+
+
+def test_helper_flop_cache_matches_the_reference_cache(K, golden_dir):
+    g = np.load(str(golden_dir) + "/flop_chance_golden.npz")
+    helper = K.ChanceNodeHelper(torch.device("cuda"), torch.float32, 2, EchoModel(), autocast_dtype=None)
+    assert np.array_equal(helper.flop_id_to_canonical.cpu().numpy(), g["flop_id_to_canonical"].astype(np.int64))
+    assert np.array_equal(helper.flop_id_to_count.cpu().numpy(), g["flop_id_to_count"].astype(np.int64))
+    assert np.array_equal(helper.flop_to_canon.cpu().numpy(), g["flop_to_canon"].astype(np.int64))
+    assert np.array_equal(helper.combo_perm.cpu().numpy(), g["combo_perm"].astype(np.int64))
+    assert np.array_equal(helper.board_to_flop_id[3, 17, 40:52].cpu().numpy(), g["board_to_flop_id_sample"].astype(np.int64))
+    assert helper.total_flop_count == 22100
+
+
+class SuitAwareModel:
+    """torch twin of the network in tests/golden/gen_flop_chance_golden.py."""
+
+    def eval(self):
+        pass
+
+    def __call__(self, f):
+        b = f.beliefs.view(-1, 2, H).float()
+        w = 1.0 + (f.board[:, 0] // 13).float() / 10.0 + (f.board[:, 2] % 13).float() / 100.0
+        h = (torch.arange(H, device=b.device) % 7).float() * 0.001
+        return SimpleNamespace(hand_values=b * w[:, None, None]
+                               + h[None, None, :] * torch.tensor([1.0, 2.0], device=b.device)[None, :, None])
+
+
+@pytest.mark.parametrize("mode,sample,nperm", [("all", 0, 0), ("all_perm6", 0, 6), ("sample256_perm6", 256, 6)])
+def test_helper_flop_values_match_vectors_from_the_reference_helper(K, golden_dir, mode, sample, nperm):
+    """flop_chance_values against tests/golden/flop_chance_golden.npz (written by running the
+    reference's helper).  The draws come from a CPU generator with the fixture's seed, as in the
+    run that wrote it, so the sampled modes see the same flops and permutations."""
+    g = np.load(str(golden_dir) + "/flop_chance_golden.npz")
+    pre, roots = g["pre_beliefs"], g["root_indices"]
+    n = pre.shape[0]
+    dev = torch.device("cuda")
+    feats = K.MLPFeatures(context=torch.zeros(n, 1, device=dev), street=torch.zeros(n, dtype=torch.long, device=dev),
+                          to_act=torch.zeros(n, dtype=torch.long, device=dev),
+                          board=torch.full((n, 5), -1, dtype=torch.long, device=dev), beliefs=torch.zeros(n, 2 * H, device=dev))
+    for name, model in (("echo", EchoModel()), ("suit_aware", SuitAwareModel())):
+        gen = torch.Generator(device="cpu")
+        gen.manual_seed(int(g["seed"]))
+        helper = K.ChanceNodeHelper(dev, torch.float32, 2, model, generator=gen, autocast_dtype=None)
+        helper.FLOP_SAMPLE_SIZE, helper.NUM_PERM_SAMPLES = sample, nperm
+        got = helper.flop_chance_values(torch.from_numpy(roots).to(dev), feats, torch.from_numpy(pre).to(dev))
+        assert got.shape == (2, 2, H) and got.dtype == torch.float32
+        np.testing.assert_allclose(got.cpu().numpy(), g[f"{name}_{mode}"], rtol=1e-5, atol=1e-7, err_msg=f"{name} {mode}")
+
+
+def test_helper_flop_values_device_generator_is_unbiased_sample(K):
+    """Default settings (256 drawn classes, 6 drawn permutations, device generator): the estimate
+    stays close to the full enumeration for a smooth network and repeats under the same seed."""
+    rng = np.random.default_rng(31)
+    pre = rng.gamma(0.5, size=(2, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    dev = torch.device("cuda")
+    feats = K.MLPFeatures(context=torch.zeros(2, 1, device=dev), street=torch.zeros(2, dtype=torch.long, device=dev),
+                          to_act=torch.zeros(2, dtype=torch.long, device=dev),
+                          board=torch.full((2, 5), -1, dtype=torch.long, device=dev), beliefs=torch.zeros(2, 2 * H, device=dev))
+    outs = []
+    for _ in range(2):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(7)
+        helper = K.ChanceNodeHelper(dev, torch.float32, 2, SuitAwareModel(), generator=gen, autocast_dtype=None)
+        outs.append(helper.flop_chance_values(torch.arange(2, device=dev), feats, torch.from_numpy(pre).to(dev)))
+    assert torch.equal(outs[0], outs[1])
+    helper.FLOP_SAMPLE_SIZE, helper.NUM_PERM_SAMPLES = 0, 0
+    full = helper.flop_chance_values(torch.arange(2, device=dev), feats, torch.from_numpy(pre).to(dev))
+    # total mass per player is preserved by both; the sampled estimate of it is within a few percent
+    np.testing.assert_allclose(outs[0].sum(-1).cpu().numpy(), full.sum(-1).cpu().numpy(), rtol=0.05)

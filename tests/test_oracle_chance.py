@@ -124,3 +124,91 @@ def test_oracle_matches_vectors_from_the_reference_helper(golden_dir):
         got = OCH.single_card_chance_values(roots, np.zeros((n, 1), np.float32), np.full(n, 3), np.zeros(n, np.int64),
                                             pre, board, fn)
         np.testing.assert_allclose(got, g[name], rtol=1e-5, atol=1e-8)
+
+
+# ---- three-card (flop) chance node (src/p2/search/chance_node_helper.py:76-357) ------------
+
+def flop_models():
+    """numpy twins of the networks in tests/golden/gen_flop_chance_golden.py."""
+    def echo(context, street, to_act, board, beliefs):
+        return beliefs.reshape(-1, 2, H).astype(np.float32)
+
+    def suit_aware(context, street, to_act, board, beliefs):
+        b = beliefs.reshape(-1, 2, H).astype(np.float32)
+        w = (1.0 + (board[:, 0] // 13).astype(np.float32) / np.float32(10.0)
+             + (board[:, 2] % 13).astype(np.float32) / np.float32(100.0)).astype(np.float32)
+        h = (np.arange(H) % 7).astype(np.float32) * np.float32(0.001)
+        return b * w[:, None, None] + h[None, None, :] * np.array([1.0, 2.0], dtype=np.float32)[None, :, None]
+
+    return {"echo": echo, "suit_aware": suit_aware}
+
+
+def test_canonical_flops_and_suit_maps_match_the_reference_cache(golden_dir):
+    g = np.load(str(golden_dir) + "/flop_chance_golden.npz")
+    canonical, count, flop_to_class = OCH.canonical_flops()
+    assert np.array_equal(canonical, g["flop_id_to_canonical"].astype(np.int64))
+    assert np.array_equal(count, g["flop_id_to_count"].astype(np.int64))
+    assert np.array_equal(flop_to_class, g["flop_to_canon"].astype(np.int64))
+    assert np.array_equal(OCH.suit_permutations(), g["suit_permutations"].astype(np.int64))
+    perms = OCH.combo_suit_perms()
+    assert np.array_equal(perms, g["combo_perm"].astype(np.int64))
+    assert np.array_equal(np.argsort(perms, axis=1), g["combo_perm_inverse"].astype(np.int64))
+    # what the mathematics fixes: 1755 classes; sizes by rank pattern are 4 (trips), 12 or 24 ... and sum to C(52,3)
+    assert canonical.shape == (1755, 3) and count.sum() == 22100
+    ranks = canonical % 13
+    trips = (ranks[:, 0] == ranks[:, 1]) & (ranks[:, 1] == ranks[:, 2])
+    assert trips.sum() == 13 and (count[trips] == 4).all()
+    distinct = (ranks[:, 0] != ranks[:, 1]) & (ranks[:, 1] != ranks[:, 2])
+    # three distinct ranks: monotone (4), two-tone (3 x 12), rainbow (24) per rank triple
+    assert distinct.sum() == 286 * 5 and sorted(set(count[distinct].tolist())) == [4, 12, 24]
+    assert (~trips & ~distinct).sum() == 13 * 12 * 2 and set(count[~trips & ~distinct].tolist()) == {12}
+    # every row of the hand map is a permutation, the identity comes first
+    assert (np.sort(perms, axis=1) == np.arange(H)).all() and (perms[0] == np.arange(H)).all()
+
+
+def test_flop_oracle_matches_vectors_from_the_reference_helper(golden_dir):
+    g = np.load(str(golden_dir) + "/flop_chance_golden.npz")
+    canonical, count, _ = OCH.canonical_flops()
+    perms = OCH.combo_suit_perms()
+    pre, roots = g["pre_beliefs"], g["root_indices"]
+    n = pre.shape[0]
+    ctx, st, ta = np.zeros((n, 1), np.float32), np.zeros(n, np.int64), np.zeros(n, np.int64)
+    for name, fn in flop_models().items():
+        cases = {"all": dict(), "all_perm6": dict(perm_rows=list(g["all_perm6_rows"])),
+                 "sample256_perm6": dict(sample_idx=g["sample256_idx"].astype(np.int64),
+                                         perm_rows=list(g["sample256_rows"]))}
+        for mode, kw in cases.items():
+            got = OCH.flop_chance_values(roots, ctx, st, ta, pre, fn, canonical, count, perms, **kw)
+            ref = g[f"{name}_{mode}"]
+            np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-7, err_msg=f"{name} {mode}")
+
+
+def test_flop_closed_form_suit_equivariant_network():
+    """A network whose answer moves with the suits (here: echo of ranges that are themselves
+    suit-symmetric, i.e. uniform) gives, through classes x orbit mean, exactly the plain mean over
+    all 22100 flops of the expanded range: every hand is blocked by C(52,3) - C(50,3) flops."""
+    canonical, count, _ = OCH.canonical_flops()
+    perms = OCH.combo_suit_perms()
+    pre = np.full((1, 2, H), 1.0 / H, dtype=np.float32)
+    got = OCH.flop_chance_values(np.array([0]), np.zeros((1, 1)), np.zeros(1, np.int64), np.zeros(1, np.int64), pre,
+                                 flop_models()["echo"], canonical, count, perms)
+    expected = (19600.0 / 22100.0) / 1176.0
+    np.testing.assert_allclose(got, expected, rtol=1e-5)
+
+
+def test_flop_expand_against_per_flop_loop():
+    rng = np.random.default_rng(3)
+    pre = rng.gamma(0.5, size=(2, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    pre[1, 0] = 0.0
+    flops = np.array([[0, 13, 26], [51, 3, 20], [12, 11, 10]], dtype=np.int64)
+    post = OCH.flop_expand(pre, flops)
+    cm = OC.hand_combos()
+    for k, f in enumerate(flops):
+        ok = np.array([cm[h, 0] not in f and cm[h, 1] not in f for h in range(H)])
+        assert ok.sum() == 1176
+        for i in range(2):
+            for p in range(2):
+                x = np.where(ok, pre[i, p].astype(np.float64), 0.0)
+                exp = x / x.sum() if x.sum() > 1e-12 else ok / ok.sum()
+                np.testing.assert_allclose(post[i, k, p], exp, rtol=1e-5, atol=1e-9)
