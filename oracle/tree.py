@@ -202,6 +202,16 @@ def build_tree(roots: list[Node], bins: list[float], depth: int, bb: int = 100) 
     return out
 
 
+def make_preflop_root(starting0: int, starting1: int, button: int = 0, sb: int = 50, bb: int = 100) -> Node:
+    """The state the env's reset leaves (``hunl_tensor_env.py:293-317``): the button has posted
+    the small blind and acts first, the other player the big blind."""
+    committed = [sb if p == button else bb for p in range(2)]
+    return Node(to_act=button, button=button, street=0, pot=sb + bb,
+                stacks=[starting0 - committed[0], starting1 - committed[1]], committed=committed, min_raise=bb,
+                actions_this_round=0, is_allin=[False, False], starting_stacks=[starting0, starting1],
+                scale=float(starting0))
+
+
 def make_root(street: int, pot: int, stack0: int, stack1: int, button: int = 0,
               bb: int = 100, starting: tuple[int, int] | None = None,
               scale: float | None = None) -> Node:

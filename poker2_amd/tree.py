@@ -87,6 +87,22 @@ class RootStates:
                    starting_stacks=starting_stacks, scale=scale, board=full, bb=bb)
 
     @classmethod
+    def preflop(cls, n: int, starting_stacks=20000, button=0, sb: int = 50, bb: int = 100, scale=None) -> "RootStates":
+        """Roots as the environment's reset leaves them (src/p2/env/hunl_tensor_env.py:293-317):
+        the button posts the small blind and acts first, the other player the big blind."""
+        button = np.broadcast_to(np.asarray(button, dtype=np.int64), (n,)).copy()
+        starting_stacks = np.broadcast_to(np.asarray(starting_stacks, dtype=np.int64), (n, 2)).copy()
+        committed = np.where(np.arange(2)[None, :] == button[:, None], sb, bb).astype(np.int64)
+        if scale is None:
+            scale = starting_stacks[:, 0].astype(np.float32)
+        scale = np.broadcast_to(np.asarray(scale, dtype=np.float32), (n,)).copy()
+        return cls(street=np.zeros(n, np.int64), to_act=button.copy(), button=button,
+                   pot=np.full(n, sb + bb, np.int64), stacks=starting_stacks - committed, committed=committed,
+                   min_raise=np.full(n, bb, np.int64), actions_this_round=np.zeros(n, np.int64),
+                   is_allin=np.zeros((n, 2), bool), starting_stacks=starting_stacks, scale=scale,
+                   board=np.full((n, 5), -1, np.int64), bb=bb)
+
+    @classmethod
     def from_env(cls, env, indices) -> "RootStates":
         """Copy rows of an object exposing the reference env's attribute names
         (``HUNLTensorEnv``: button, street, to_act, pot, stacks, committed, min_raise,

@@ -28,6 +28,8 @@ CASES = [
     ("river_b3_d3", 3, [0.33, 0.75, 1.5], 3, [(200, 800, 800, 0), (777, 1333, 901, 1), (90, 45, 300, 0)]),
     ("turn_b2_d3", 2, [0.5, 1.0], 3, [(200, 800, 800, 0), (400, 300, 900, 1)]),
     ("flop_b1_d2", 1, [1.0], 2, [(200, 900, 900, 1)]),
+    # street 0: the roots are the env's reset state (blinds posted); the row holds (pot, starting stacks, button)
+    ("preflop_b2_d4", 0, [0.5, 1.0], 4, [(150, 1000, 1000, 0), (150, 1000, 1000, 1)]),
 ]
 
 
@@ -46,12 +48,13 @@ def main() -> None:
         for _ in range(2 * street):
             env.step_bins(torch.ones(n, dtype=torch.long))
         assert (env.street == street).all() and (env.actions_this_round == 0).all()
-        pot = torch.tensor([r[0] for r in rows])
-        stacks = torch.tensor([[r[1], r[2]] for r in rows])
-        env.pot[:] = pot
-        env.stacks[:] = stacks
-        env.starting_stacks[:] = stacks + (pot // 2)[:, None]
-        env.scale[:] = env.starting_stacks[:, 0].float()
+        if street > 0:
+            pot = torch.tensor([r[0] for r in rows])
+            stacks = torch.tensor([[r[1], r[2]] for r in rows])
+            env.pot[:] = pot
+            env.stacks[:] = stacks
+            env.starting_stacks[:] = stacks + (pot // 2)[:, None]
+            env.scale[:] = env.starting_stacks[:, 0].float()
 
         levels = [env]
         parent_levels = [torch.full((n,), -1, dtype=torch.long)]

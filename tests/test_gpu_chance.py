@@ -339,3 +339,61 @@ def test_helper_flop_values_device_generator_is_unbiased_sample(K):
     full = helper.flop_chance_values(torch.arange(2, device=dev), feats, torch.from_numpy(pre).to(dev))
     # total mass per player is preserved by both; the sampled estimate of it is within a few percent
     np.testing.assert_allclose(outs[0].sum(-1).cpu().numpy(), full.sum(-1).cpu().numpy(), rtol=0.05)
+
+
+def test_preflop_subgame_with_flop_leaves_matches_oracle(K):
+    """Preflop roots: the leaves that close the betting round are valued by the flop chance node
+    (all 1755 classes, all 24 permutations, so nothing is drawn) in front of a small network."""
+    from oracle import cfr as OCFR
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import ChanceLeafModel, RangeBoardMLP
+    from poker2_amd.tree import RootStates
+    from tests.test_gpu_evaluator import compare, tree_as_dict
+    rng = np.random.default_rng(14)
+    n, iters = 2, 3
+    boards = np.full((n, 5), -1, dtype=np.int64)
+    beliefs = rng.gamma(0.5, size=(n, 2, H)).astype(np.float32)
+    beliefs /= beliefs.sum(-1, keepdims=True)
+    roots = RootStates.preflop(n, starting_stacks=1000, button=np.arange(n) % 2)
+    cfg = river_dcfr_config(n, iterations=iters, depth=2, dcfr_delay=0)
+    dev = torch.device("cuda")
+    net = RangeBoardMLP(hidden=64, layers=2, seed=5).to(dev)
+    with torch.no_grad():
+        for lin in net.linears:
+            lin.weight.mul_(4.0)
+    model = ChanceLeafModel(net, dev)
+    model.helper.FLOP_SAMPLE_SIZE, model.helper.NUM_PERM_SAMPLES = 0, 0
+    ev = HipSparseCFREvaluator(model, dev, cfg, fused_iteration=True, max_raises=1)
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+    ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+    tree = ev.tree
+    rows_model = ev.model_indices.cpu().numpy()
+    closes = tree.new_street_mask[rows_model]
+    assert closes.any() and (~closes).any()           # both kinds of leaf: round closed (flop to come) and mid-round
+    mlp = numpy_mlp(net)
+    street, to_act = tree.state["street"], tree.state["to_act"]
+    canonical, count, _ = OCH.canonical_flops()
+    perms = OCH.combo_suit_perms()
+
+    def leaf_fn(bel, rows):
+        rows = np.asarray(rows)
+        out = np.zeros((len(rows), 2, H), np.float32)
+        flop = tree.new_street_mask[rows]
+        if flop.any():
+            r = rows[flop]
+            out[flop] = OCH.flop_chance_values(np.arange(len(r)), np.zeros((len(r), 1), np.float32), street[r],
+                                               to_act[r], bel[r], mlp, canonical, count, perms)
+        if (~flop).any():
+            r = rows[~flop]
+            out[~flop] = mlp(None, street[r], to_act[r], np.full((len(r), 5), -1), bel[r].reshape(len(r), -1))
+        return out
+    orc = OCFR.OracleCFR(tree_as_dict(tree), boards, beliefs, cfr_iterations=iters, leaf_value_fn=leaf_fn,
+                         t_sample_roots=np.full(n, -1, dtype=np.int64), fused_variant=True)
+    orc.prepare()
+    compare(ev, orc, rtol=2e-4, atol=2e-5)
+    assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3
+    for t in range(iters):
+        ev.cfr_iteration(t)
+        orc.cfr_iteration(t)
+        compare(ev, orc, rtol=1e-3, atol=3e-4)      # network through hipBLASLt vs numpy: GEMM summation order

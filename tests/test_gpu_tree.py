@@ -68,3 +68,13 @@ def test_device_builder_from_mid_round_roots():
     assert roots.is_allin.any() and (roots.committed.sum(1) > 0).any()
     same_tree(build_sparse_tree(roots, [0.5, 1.0], 4, max_raises=2),
               build_sparse_tree_device(roots, [0.5, 1.0], 4, max_raises=2))
+
+
+def test_device_builder_from_preflop_roots():
+    """Roots as the environment's reset leaves them: blinds committed, the button to act."""
+    from poker2_amd.tree import RootStates, build_sparse_tree, build_sparse_tree_device
+    rng = np.random.default_rng(11)
+    n = 200
+    roots = RootStates.preflop(n, starting_stacks=rng.integers(150, 20000, (n, 2)), button=rng.integers(0, 2, n))
+    same_tree(build_sparse_tree(roots, [0.5, 1.0], 5, max_raises=3),
+              build_sparse_tree_device(roots, [0.5, 1.0], 5, max_raises=3))

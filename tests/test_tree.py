@@ -22,6 +22,9 @@ def roots_of(case):
     r = case["roots"]
     pot, stacks, button = r[:, 0], r[:, 1:3], r[:, 3]
     street = int(case["root_street"])
+    if street == 0:      # reset state: the row holds the starting stacks
+        return (RootStates.preflop(len(r), starting_stacks=stacks, button=button),
+                [OT.make_preflop_root(int(s[0]), int(s[1]), button=int(b)) for s, b in zip(stacks, button)])
     prod = RootStates.at_round_start(street, pot, stacks, np.full((len(r), 5), -1), button=button)
     orac = [OT.make_root(street, int(p), int(s[0]), int(s[1]), button=int(b)) for p, s, b in zip(pot, stacks, button)]
     return prod, orac
@@ -50,7 +53,7 @@ def test_builders_match_reference_env_fixture(golden_dir):
             assert np.array_equal(getattr(t, k), o[k]), (name, k)
         assert np.array_equal(t.showdown_potential, o["showdown_potential"])
         n += 1
-    assert n >= 6
+    assert n >= 7
 
 
 def test_hand_derived_river_tree():
