@@ -100,6 +100,34 @@ int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int
 int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
                     const float* weight, int accumulate, float* out, void* stream);
 
+/* ---- either side of the search in data generation ------------------------------------------ */
+
+/* Context features and board of RebelFeatureEncoder.encode (models/mlp/rebel_feature_encoder.py:55-127)
+ * for m public states: context [m,4] float32 (16-byte aligned) = (to_act, (to_act - button) mod 2,
+ * clamp(pot / max(starting_stack0 + starting_stack1, 1), 0, 10), committed chips differ and
+ * actions_this_round > 0); board_out [m,5] = last_board where the state is encoded before its
+ * chance event (pre_chance [m] bytes; NULL = pre_chance_all for every state), else board.
+ * All inputs int64: [m] or [m,2] / [m,5]. */
+int p2hip_encode_context(const int64_t* to_act, const int64_t* button, const int64_t* starting_stacks,
+                         const int64_t* pot, const int64_t* committed, const int64_t* actions_this_round,
+                         const uint8_t* pre_chance, int pre_chance_all, const int64_t* last_board,
+                         const int64_t* board, int64_t m, float* context, int64_t* board_out, void* stream);
+
+/* Chip amounts of the action bins, the first result of HUNLTensorEnv.legal_bins_amounts_and_mask
+ * (env/hunl_tensor_env.py:348-405): amounts [m, n_bins + 3] = -1 for fold and call,
+ * to_call + trunc(bin * pot) for each bet bin (legal or not), the actor's stack for all-in.
+ * host_bins: at most 5 pot fractions in HOST memory. */
+int p2hip_bet_amounts(const int64_t* to_act, const int64_t* stacks, const int64_t* committed, const int64_t* pot,
+                      int64_t m, const float* host_bins, int n_bins, int64_t* amounts, void* stream);
+
+/* Policy targets of CFREvaluator.training_data (search/cfr_evaluator.py:1392-1393; _pull_back,
+ * search/sparse_cfr_evaluator.py:465-489): out [n_rows, H, num_actions] with
+ * out[k,h,a] = policy_avg[c,h] for the child c of node rows[k] that action a leads to, 0 for
+ * actions without a child.  policy_avg [total,H]; the three index arrays are [total] int64. */
+int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n_rows, const int64_t* child_offsets,
+                         const int64_t* child_count, const int64_t* action_from_parent, int num_actions, float* out,
+                         void* stream);
+
 /* ---- local best response -------------------------------------------------------------- */
 
 /* One tree level of _best_response_values (search/cfr_evaluator.py:636-714), in place on

@@ -56,6 +56,16 @@ class MLPFeatures:
         return MLPFeatures(context=self.context.clone(), street=self.street.clone(), to_act=self.to_act.clone(),
                            board=self.board.clone(), beliefs=self.beliefs.clone())
 
+    @classmethod
+    def cat(cls, features_list: list["MLPFeatures"]) -> "MLPFeatures":
+        if not features_list:
+            raise ValueError("Cannot concatenate an empty list of features.")
+        return cls(context=torch.cat([f.context for f in features_list], dim=0),
+                   street=torch.cat([f.street for f in features_list], dim=0),
+                   to_act=torch.cat([f.to_act for f in features_list], dim=0),
+                   board=torch.cat([f.board for f in features_list], dim=0),
+                   beliefs=torch.cat([f.beliefs for f in features_list], dim=0))
+
 
 def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, board_pre: torch.Tensor,
                   cards_on_board: int | None = None):

@@ -1,0 +1,151 @@
+// Kernels either side of the search in data generation: feature encoding of public states,
+// bet amounts of the action bins, and policy targets gathered from the children.
+//
+// RebelFeatureEncoder.encode (src/p2/models/mlp/rebel_feature_encoder.py:55-127),
+// HUNLTensorEnv.legal_bins_amounts_and_mask (src/p2/env/hunl_tensor_env.py:348-423, amounts only)
+// and the policy targets of CFREvaluator.training_data (src/p2/search/cfr_evaluator.py:1392-1393:
+// _pull_back of the average policy, then [node, hand, action]).
+#pragma once
+#include "common.h"
+
+namespace p2 {
+
+constexpr int DG_BLOCK = 256;
+constexpr int DG_MAX_ACTIONS = 8;
+
+// context [m,4] = (to_act, (to_act - button) mod 2, clamp(pot / max(start0 + start1, 1), 0, 10),
+//                  committed differ and at least one action this round);
+// board_out [m,5] = last_board where pre_chance (a byte per state, or the same flag for all), else board.
+__global__ __launch_bounds__(DG_BLOCK) void encode_context_kernel(
+    const int64_t* __restrict__ to_act, const int64_t* __restrict__ button, const int64_t* __restrict__ starting_stacks,
+    const int64_t* __restrict__ pot, const int64_t* __restrict__ committed, const int64_t* __restrict__ actions,
+    const uint8_t* __restrict__ pre_chance, int pre_chance_all, const int64_t* __restrict__ last_board,
+    const int64_t* __restrict__ board, int64_t m, float* __restrict__ context, int64_t* __restrict__ board_out) {
+  const int64_t i = (int64_t)blockIdx.x * DG_BLOCK + threadIdx.x;
+  if (i >= m) return;
+  const int64_t ta = to_act[i];
+  const float total = fmaxf((float)starting_stacks[2 * i] + (float)starting_stacks[2 * i + 1], 1.0f);
+  const float frac = fminf(fmaxf((float)pot[i] / total, 0.0f), 10.0f);
+  const bool bet = committed[2 * i] != committed[2 * i + 1] && actions[i] > 0;
+  float4 c;
+  c.x = (float)ta;
+  c.y = (float)(((ta - button[i]) % 2 + 2) % 2);
+  c.z = frac;
+  c.w = bet ? 1.0f : 0.0f;
+  reinterpret_cast<float4*>(context)[i] = c;
+  const bool pre = pre_chance ? pre_chance[i] != 0 : pre_chance_all != 0;
+  const int64_t* src = (pre ? last_board : board) + 5 * i;
+#pragma unroll
+  for (int j = 0; j < 5; ++j) board_out[5 * i + j] = src[j];
+}
+
+struct DgBins {
+  float bins[DG_MAX_ACTIONS - 3];
+  int n_bins;
+};
+
+// amounts [m, n_bins + 3]: -1 for fold and call, to_call + trunc(bin * pot) for the bet bins
+// (whether legal or not), the actor's stack for all-in.
+__global__ __launch_bounds__(DG_BLOCK) void bet_amounts_kernel(const int64_t* __restrict__ to_act,
+                                                                const int64_t* __restrict__ stacks,
+                                                                const int64_t* __restrict__ committed,
+                                                                const int64_t* __restrict__ pot, int64_t m, DgBins B,
+                                                                int64_t* __restrict__ amounts) {
+  const int64_t i = (int64_t)blockIdx.x * DG_BLOCK + threadIdx.x;
+  if (i >= m) return;
+  const int nb = B.n_bins + 3;
+  const int me = (int)to_act[i], opp = 1 - me;
+  const int64_t to_call = committed[2 * i + opp] - committed[2 * i + me];
+  const float pot_f = (float)pot[i];
+  int64_t* out = amounts + i * nb;
+  out[0] = -1;
+  out[1] = -1;
+  for (int b = 0; b < B.n_bins; ++b) out[2 + b] = to_call + (int64_t)(B.bins[b] * pot_f);
+  out[nb - 1] = stacks[2 * i + me];
+}
+
+// out[k, h, a] = policy_avg[c, h] for the child c of node rows[k] reached by action a, 0 where the
+// action has no child.  One workgroup per node: the children's rows are read whole (coalesced),
+// transposed through LDS and written as one contiguous [H * A] run.
+__global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* __restrict__ policy_avg,
+                                                                   const int64_t* __restrict__ rows,
+                                                                   const int64_t* __restrict__ child_offsets,
+                                                                   const int64_t* __restrict__ child_count,
+                                                                   const int64_t* __restrict__ action_from_parent,
+                                                                   int num_actions, float* __restrict__ out) {
+  extern __shared__ __align__(8) float tile[];   // [num_actions][H + 1]
+  const int64_t k = blockIdx.x;
+  const int64_t r = rows[k];
+  const int stride = P2_H + 1;
+  for (int e = threadIdx.x; e < num_actions * stride; e += DG_BLOCK) tile[e] = 0.f;
+  p2_sync_lds();
+  const int64_t first = child_offsets[r];
+  const int n_children = (int)child_count[r];
+  for (int j = 0; j < n_children; ++j) {
+    const int a = (int)action_from_parent[first + j];
+    if (a < 0 || a >= num_actions) continue;
+    const float* src = policy_avg + (first + j) * P2_H;
+    for (int h = threadIdx.x; h < P2_H; h += DG_BLOCK) tile[a * stride + h] = src[h];
+  }
+  p2_sync_lds();
+  float* dst = out + k * (int64_t)P2_H * num_actions;
+  for (int e = threadIdx.x; e < P2_H * num_actions; e += DG_BLOCK) {
+    const int h = e / num_actions, a = e - h * num_actions;
+    dst[e] = tile[a * stride + h];
+  }
+}
+
+}  // namespace p2
+
+extern "C" {
+
+int p2hip_encode_context(const int64_t* to_act, const int64_t* button, const int64_t* starting_stacks,
+                         const int64_t* pot, const int64_t* committed, const int64_t* actions_this_round,
+                         const uint8_t* pre_chance, int pre_chance_all, const int64_t* last_board,
+                         const int64_t* board, int64_t m, float* context, int64_t* board_out, void* stream) {
+  if (m < 0) return P2_EINVAL;
+  if (m == 0) return 0;
+  if (!to_act || !button || !starting_stacks || !pot || !committed || !actions_this_round || !last_board || !board ||
+      !context || !board_out)
+    return P2_EINVAL;
+  if (((uintptr_t)context & 15) != 0) return P2_EINVAL;
+  const int64_t grid = (m + p2::DG_BLOCK - 1) / p2::DG_BLOCK;
+  if (grid > 0x7FFFFFFF) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::encode_context_kernel, dim3((unsigned)grid), dim3(p2::DG_BLOCK), 0, (hipStream_t)stream,
+                     to_act, button, starting_stacks, pot, committed, actions_this_round, pre_chance, pre_chance_all,
+                     last_board, board, m, context, board_out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_bet_amounts(const int64_t* to_act, const int64_t* stacks, const int64_t* committed, const int64_t* pot,
+                      int64_t m, const float* host_bins, int n_bins, int64_t* amounts, void* stream) {
+  if (m < 0 || n_bins < 0 || n_bins > p2::DG_MAX_ACTIONS - 3 || (n_bins > 0 && !host_bins)) return P2_EINVAL;
+  if (m == 0) return 0;
+  if (!to_act || !stacks || !committed || !pot || !amounts) return P2_EINVAL;
+  p2::DgBins B;
+  for (int b = 0; b < p2::DG_MAX_ACTIONS - 3; ++b) B.bins[b] = b < n_bins ? host_bins[b] : 0.f;
+  B.n_bins = n_bins;
+  const int64_t grid = (m + p2::DG_BLOCK - 1) / p2::DG_BLOCK;
+  if (grid > 0x7FFFFFFF) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::bet_amounts_kernel, dim3((unsigned)grid), dim3(p2::DG_BLOCK), 0, (hipStream_t)stream, to_act,
+                     stacks, committed, pot, m, B, amounts);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n_rows, const int64_t* child_offsets,
+                         const int64_t* child_count, const int64_t* action_from_parent, int num_actions, float* out,
+                         void* stream) {
+  if (n_rows < 0 || num_actions < 1 || num_actions > p2::DG_MAX_ACTIONS) return P2_EINVAL;
+  if (n_rows == 0) return 0;
+  if (!policy_avg || !rows || !child_offsets || !child_count || !action_from_parent || !out) return P2_EINVAL;
+  if (n_rows > 0x7FFFFFFF) return P2_EINVAL;
+  const size_t lds = (size_t)num_actions * (P2_H + 1) * sizeof(float);   // at most 42.5 KB
+  hipLaunchKernelGGL(p2::policy_targets_kernel, dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), lds, (hipStream_t)stream,
+                     policy_avg, rows, child_offsets, child_count, action_from_parent, num_actions, out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -9,6 +9,7 @@
 #include "chance.hip"
 #include "best_response.hip"
 #include "tree.hip"
+#include "datagen.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

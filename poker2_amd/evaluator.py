@@ -38,7 +38,10 @@ from . import fused_cfr_hip as F
 from . import rules_hip
 from .card_utils import NUM_HANDS, combo_to_onehot_tensor
 from .fused_cfr_hip import CFRType
-from .tree import RootStates, SparseTree, build_sparse_tree, build_sparse_tree_device
+from .chance_node_helper import ChanceNodeHelper
+from .rebel_batch import RebelBatch
+from .rebel_feature_encoder import RebelFeatureEncoder
+from .tree import CARDS_ON_STREET, RootStates, SparseTree, build_sparse_tree, build_sparse_tree_device
 
 STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
                "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",
@@ -74,6 +77,21 @@ class SampledLeaves:
     nodes: torch.Tensor      # [K] rows of this evaluator's tree
     beliefs: torch.Tensor    # [K, 2, 1326]
     roots: RootStates        # K root states for ``initialize_subgame``
+
+
+class _TreeEnv(SimpleNamespace):
+    """Per-node public states of the tree under the reference env's attribute names."""
+
+    def legal_bins_amounts_and_mask(self, bet_bins: list[float] | None = None):
+        """(amounts [N,B] int64, mask [N,B] bool) of src/p2/env/hunl_tensor_env.py:348-423."""
+        bins = list(self.default_bet_bins if bet_bins is None else bet_bins)
+        if bins != list(self.default_bet_bins):
+            raise ValueError("the tree was built for bet bins %r" % (self.default_bet_bins,))
+        amounts = torch.empty(self.N, len(bins) + 3, dtype=torch.int64, device=self.to_act.device)
+        bins_c = (ctypes.c_float * max(1, len(bins)))(*bins)
+        _lib.call("p2hip_bet_amounts", _lib.ptr(self.to_act), _lib.ptr(self.stacks), _lib.ptr(self.committed),
+                  _lib.ptr(self.pot), self.N, bins_c, len(bins), _lib.ptr(amounts), _lib.stream_ptr())
+        return amounts, self.legal_mask
 
 
 class HipSparseCFREvaluator:
@@ -134,6 +152,7 @@ class HipSparseCFREvaluator:
         self._fscal_host = (ctypes.c_float * 8)()
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
+        self._chance_helper = None
 
     @property
     def enforce_zero_sum(self) -> bool:
@@ -183,12 +202,28 @@ class HipSparseCFREvaluator:
         self.new_street_mask = self._t(tree.new_street_mask)
         self.child_mask = self.legal_mask & (~self.leaf_mask)[:, None]
         st = tree.state
-        self.env = SimpleNamespace(
+        # Boards per node.  Every action saves the board before cards are dealt
+        # (hunl_tensor_env.py:862): below the roots the previous board is the root's board.  The
+        # current board of a node that closed a betting round shows the next cards only when the
+        # roots carry their runout.
+        node_board = tree.board[tree.root_index]
+        last_board = node_board.copy()
+        last_board[:N] = roots.previous_board()
+        if roots.runout is not None:
+            shown = np.arange(5)[None, :] < CARDS_ON_STREET[np.clip(st["street"], 0, 4)][:, None]
+            node_board = np.where(shown, roots.runout[tree.root_index], -1)
+        self._roots = roots
+        self.env = _TreeEnv(
             N=T, to_act=tt("to_act", st["to_act"]), done=self._t(st["done"]), street=tt("street", st["street"]),
             pot=tt("pot", st["pot"]), stacks=self._t(st["stacks"]), committed=self._t(st["committed"]),
             starting_stacks=self._t(st["starting_stacks"]), scale=self._t(st["scale"]),
             actions_this_round=tt("actions_this_round", st["actions_this_round"]), button=tt("button", st["button"]),
-            board_indices=self._t(tree.board[tree.root_index]), bb=roots.bb)
+            min_raise=tt("min_raise", st["min_raise"]), is_allin=self._t(st["is_allin"]),
+            board_indices=self._t(node_board), last_board_indices=self._t(last_board), bb=roots.bb,
+            default_bet_bins=list(self.bet_bins), legal_mask=self.legal_mask)
+        self.feature_encoder = (self.model.create_feature_encoder(self.env, device=dev, dtype=self.float_dtype)
+                                if hasattr(self.model, "create_feature_encoder")
+                                else RebelFeatureEncoder(self.env, device=dev, dtype=self.float_dtype))
         self._root_index = tt("root_index", tree.root_index)
         model_mask = tree.leaf_mask & ~st["done"]
         self.model_indices = self._t(np.nonzero(model_mask)[0].astype(np.int64))
@@ -726,6 +761,96 @@ class HipSparseCFREvaluator:
             else:
                 fields[name] = np.asarray(tree.state[name])[rows]
         return SampledLeaves(nodes=keep, beliefs=self.beliefs[keep].clone(), roots=RootStates(**fields))
+
+    # ------------------------------------------------------------------ training data
+    @property
+    def chance_helper(self) -> ChanceNodeHelper:
+        """Chance-node enumeration around the value network (sparse_cfr_evaluator.py:65-71).  The
+        network is the leaf model's ``net`` (or the model itself when it maps features to an
+        object with ``hand_values``)."""
+        if self._chance_helper is None:
+            helper = getattr(self.model, "helper", None)
+            if not isinstance(helper, ChanceNodeHelper):
+                net = getattr(self.model, "net", None)
+                if net is None and callable(self.model):
+                    net = self.model
+                if net is None:
+                    raise RuntimeError("pre-chance value targets need a value network (model.net)")
+                helper = ChanceNodeHelper(self.device, self.float_dtype, self.num_players, net,
+                                          generator=self.generator,
+                                          autocast_dtype=getattr(self.model, "autocast_dtype", None))
+            self._chance_helper = helper
+        return self._chance_helper
+
+    def _policy_targets(self, rows: torch.Tensor) -> torch.Tensor:
+        """[K, 1326, num_actions]: the average policy of the children of ``rows`` by action, zero
+        for actions without a child (cfr_evaluator.py:1392-1393 on the selected rows)."""
+        rows = rows.to(device=self.device, dtype=torch.int64).contiguous()
+        if rows.numel() and (int(rows.min()) < 0 or int(rows.max()) >= self.total_nodes):
+            raise IndexError("policy target rows out of range")
+        out = torch.empty(rows.numel(), NUM_HANDS, self.num_actions, dtype=self.float_dtype, device=self.device)
+        _lib.call("p2hip_policy_targets", _lib.ptr(self.policy_probs_avg), _lib.ptr(rows), rows.numel(),
+                  _lib.ptr(self.child_offsets), _lib.ptr(self.child_count), _lib.ptr(self.action_from_parent),
+                  self.num_actions, _lib.ptr(out), _lib.stream_ptr())
+        return out
+
+    @torch.no_grad()
+    def training_data(self, exclude_start: bool = True) -> tuple[RebelBatch, RebelBatch, RebelBatch]:
+        """(value batch, pre-chance value batch, policy batch) of a finished search
+        (cfr_evaluator.py:1383-1495).  Value targets: the roots' average values clamped to
+        [-1, 1].  Policy targets: the average policy of every expanded node, [node, hand, action].
+        Roots standing at the start of a betting round after a deal also give a sample for the
+        state BEFORE that deal: its value is the network's answer averaged over the cards that
+        could have come (single card on turn and river, canonical flops on the flop)."""
+        N = self.root_nodes
+        top = self.depth_offsets[-2] if len(self.depth_offsets) > 1 else N
+        dev = self.device
+        value_targets = self.values_avg[:N].clamp(-1.0, 1.0)
+        features = self.feature_encoder.encode(self.beliefs_avg, pre_chance_node=False,
+                                               indices=torch.arange(top, device=dev))
+        bin_amounts, legal_masks = self.env.legal_bins_amounts_and_mask()
+        statistics = {"to_act": self.env.to_act, "street": self.env.street, "stage": 2 * self.env.street,
+                      "board": self.env.board_indices, "pot": self.env.pot, "bet_amounts": bin_amounts}
+        exploit_stats = self._compute_exploitability()
+        value_statistics = {k: v[:N] for k, v in statistics.items()}
+        value_statistics["local_exploitability"] = exploit_stats.local_exploitability
+        value_statistics["local_best_response_values"] = exploit_stats.local_best_response_values
+        valid_top = self.valid_mask[:top] & ~self.leaf_mask[:top]
+        policy_rows = torch.nonzero(valid_top).squeeze(1)
+        policy_statistics = {k: v[:top][valid_top] for k, v in statistics.items()}
+        value_batch = RebelBatch(features=features[:N], value_targets=value_targets, legal_masks=legal_masks[:N],
+                                 statistics=value_statistics)
+        street_root = self.env.street[:N]
+        actions_root = self.env.actions_this_round[:N]
+        if exclude_start:
+            value_batch = value_batch[~((street_root == 0) & (actions_root == 0))]
+        policy_batch = RebelBatch(features=features[valid_top], policy_targets=self._policy_targets(policy_rows),
+                                  legal_masks=legal_masks[:top][valid_top], statistics=policy_statistics)
+
+        pre_features_root = self.feature_encoder.encode(self.beliefs, pre_chance_node=True,
+                                                        indices=torch.arange(N, device=dev)).clone()
+        pre_features_root.beliefs = self.root_pre_chance_beliefs[:N].reshape(N, -1).clone()
+        value_targets_pre = value_targets.clone()
+        value_statistics_pre = {k: v.clone() for k, v in value_statistics.items()}
+        value_statistics_pre["board"] = self.env.last_board_indices[:N].clone()
+        prev_street = torch.where((street_root > 0) & (street_root < 4) & (actions_root == 0), street_root - 1,
+                                  street_root)
+        value_statistics_pre["street"] = prev_street
+        value_statistics_pre["stage"] = 2 * prev_street + 1
+        start_mask = actions_root == 0
+        turn_river_mask = start_mask & ((street_root == 2) | (street_root == 3))
+        if bool(turn_river_mask.any()):
+            value_targets_pre[turn_river_mask] = self.chance_helper.single_card_chance_values(
+                torch.where(turn_river_mask)[0], features[:N], self.root_pre_chance_beliefs,
+                self.env.last_board_indices[:N])
+        flop_mask = start_mask & (street_root == 1)
+        if bool(flop_mask.any()):
+            value_targets_pre[flop_mask] = self.chance_helper.flop_chance_values(
+                torch.where(flop_mask)[0], features[:N], self.root_pre_chance_beliefs)
+        transition_mask = turn_river_mask | flop_mask
+        pre_value_batch = RebelBatch(features=pre_features_root, value_targets=value_targets_pre,
+                                     legal_masks=legal_masks[:N], statistics=value_statistics_pre)[transition_mask]
+        return value_batch, pre_value_batch, policy_batch
 
     # ------------------------------------------------------------------ best response
     def _fan_out_deep(self, per_root: torch.Tensor) -> torch.Tensor:

@@ -45,6 +45,32 @@ class RangeBoardMLP(torch.nn.Module):
         return SimpleNamespace(hand_values=x.view(-1, 2, NUM_HANDS))
 
 
+class NetworkLeafModel:
+    """The reference's own leaf rule (src/p2/search/cfr_evaluator.py:1024-1040): the network sees
+    the encoded features of every leaf that is not terminal; a leaf that closed a betting round
+    is encoded with the board before the next deal, so the network itself stands for the chance
+    node."""
+
+    def __init__(self, net, device, *, enforce_zero_sum: bool = False,
+                 autocast_dtype: torch.dtype | None = None) -> None:
+        self.net = net
+        self.device = torch.device(device)
+        self.enforce_zero_sum = enforce_zero_sum
+        self.autocast_dtype = autocast_dtype
+
+    @torch.no_grad()
+    def leaf_values(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
+        feats = ev.feature_encoder.encode_rows(beliefs.contiguous(), rows, ev.new_street_mask[rows])
+        if hasattr(self.net, "eval"):
+            self.net.eval()
+        if self.autocast_dtype is not None:
+            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                hv = self.net(feats).hand_values
+        else:
+            hv = self.net(feats).hand_values
+        return hv.to(beliefs.dtype)
+
+
 class ChanceLeafModel:
     """Evaluator leaf protocol on top of a value network and the chance nodes (one card, flop)."""
 

@@ -25,6 +25,9 @@ import numpy as np
 H = 1326
 
 
+CARDS_ON_STREET = np.array([0, 3, 4, 5, 5])   # board cards visible on streets 0..3 and at showdown
+
+
 @dataclass
 class RootStates:
     """Public state of N subgame roots (numpy arrays of length N)."""
@@ -42,10 +45,26 @@ class RootStates:
     board: np.ndarray             # [N,5] int64, -1 = not dealt
     done: np.ndarray = None       # [N] bool
     bb: int = 100
+    last_board: np.ndarray = None  # [N,5] board before the latest action (None: derived, see previous_board)
+    runout: np.ndarray = None      # [N,5] the complete board these roots will see (None: cards are drawn when needed)
 
     def __post_init__(self):
         if self.done is None:
             self.done = np.zeros(self.street.shape[0], dtype=bool)
+        if self.runout is not None:
+            shown = np.arange(5)[None, :] < CARDS_ON_STREET[np.clip(self.street, 0, 4)][:, None]
+            assert np.array_equal(np.where(shown, self.runout, -1), self.board), "runout does not continue the board"
+
+    def previous_board(self) -> np.ndarray:
+        """The env's ``last_board_indices`` (src/p2/env/hunl_tensor_env.py:862): every action saves the
+        board before cards are dealt, so a root at the start of a betting round still holds the
+        previous street's board and any other root its own."""
+        if self.last_board is not None:
+            return self.last_board
+        street = np.clip(self.street, 0, 4)
+        at_start = (self.actions_this_round == 0) & (street >= 1)
+        keep = np.where(at_start, CARDS_ON_STREET[np.maximum(street - 1, 0)], 5)
+        return np.where(np.arange(5)[None, :] < keep[:, None], self.board, -1)
 
     @property
     def n(self) -> int:
@@ -120,7 +139,8 @@ class RootStates:
                    actions_this_round=g("actions_this_round").astype(np.int64),
                    is_allin=g("is_allin").astype(bool), starting_stacks=g("starting_stacks").astype(np.int64),
                    scale=g("scale").astype(np.float32), board=g("board_indices").astype(np.int64),
-                   done=g("done").astype(bool), bb=int(getattr(env, "bb", 100)))
+                   done=g("done").astype(bool), bb=int(getattr(env, "bb", 100)),
+                   last_board=g("last_board_indices").astype(np.int64) if hasattr(env, "last_board_indices") else None)
 
 
 _STATE_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",

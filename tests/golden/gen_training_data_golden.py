@@ -1,0 +1,174 @@
+"""Writes tests/golden/training_data_golden.npz by RUNNING the reference's own
+``SparseCFREvaluator`` (search, ``training_data``: src/p2/search/cfr_evaluator.py:1383-1495) with
+its ``RebelFeatureEncoder`` (src/p2/models/mlp/rebel_feature_encoder.py:55-127) and
+``ChanceNodeHelper`` on the CPU of the build container.  Run once, here only:
+    python tests/golden/gen_training_data_golden.py
+
+Roots come from playing the reference env forward from its reset state with scripted bins, so
+every field (committed chips, previous board, min raise) is what the env itself produces: turn
+and river and flop roots at the start of a betting round (these get pre-chance value targets
+through the single-card / flop chance node), roots in the middle of a round, preflop roots (the
+reset state is dropped from the value batch).  The leaf network is a closed-form function of the
+encoded features (written out in ``ValueNet`` below; tests restate it), so the search, the
+encoder and the chance nodes all feed the stored targets.  The flop chance node runs in its
+exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
+"""
+from __future__ import annotations
+
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+from gen_cfr_golden import REF_SRC, install_stand_ins  # noqa: E402
+
+ENV_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",
+              "is_allin", "starting_stacks", "scale", "board_indices", "last_board_indices", "done")
+STATE = ("policy_probs_avg", "beliefs", "beliefs_avg", "values_avg")
+
+# name, depth, iterations, per root: (button, bins played from the reset state)
+CASES = [
+    ("streets_mixed", 3, 4, [(0, [1, 1, 1, 1]), (1, [3, 1, 1, 1]), (0, [1, 1, 1, 1, 1, 1]),
+                             (1, [1, 1, 1, 1, 1, 1, 2]), (0, [2, 1]), (1, [1, 1, 1, 1, 1])]),
+    ("preflop", 2, 3, [(0, []), (1, [1]), (1, [])]),
+]
+
+
+def main() -> None:
+    os.environ.setdefault("TORCHDYNAMO_DISABLE", "1")
+    install_stand_ins()
+    sys.path.insert(0, REF_SRC)
+    import warnings
+    import torch
+    from p2.core.structured_config import CFRType, Config, EnvConfig, ModelConfig, SearchConfig, TrainingConfig
+    from p2.env.card_utils import NUM_HANDS
+    from p2.env.hunl_tensor_env import HUNLTensorEnv
+    from p2.models.model_output import ModelOutput
+    from p2.models.mlp.rebel_feature_encoder import RebelFeatureEncoder
+    from p2.search.sparse_cfr_evaluator import SparseCFREvaluator
+    warnings.filterwarnings("ignore")
+
+    class ValueNet:
+        """hand value of player p, hand h =
+             s_p * 0.05 * w * (1326 * opponent_range[h] - 1) + 0.002 * ((h mod 7) - 3)
+        with s_0 = 1, s_1 = -1 and
+             w = 0.2 + 0.1 * context[2] + 0.05 * context[1] - 0.03 * context[3]
+                 + 0.01 / 13 * sum over dealt board cards of (rank + 1)."""
+
+        def __init__(self, num_actions):
+            self.num_actions = num_actions
+            self.enforce_zero_sum = False
+            self.hidden_dim = 1
+
+        def create_feature_encoder(self, env, device=None, dtype=None):
+            return RebelFeatureEncoder(env=env, device=device, dtype=dtype)
+
+        def eval(self):
+            pass
+
+        def __call__(self, f, include_policy=True):
+            b = f.beliefs.view(-1, 2, NUM_HANDS).float()
+            ranks = torch.where(f.board >= 0, (f.board % 13 + 1).float(), torch.zeros_like(f.board, dtype=torch.float32))
+            w = (0.2 + 0.1 * f.context[:, 2] + 0.05 * f.context[:, 1] - 0.03 * f.context[:, 3]
+                 + 0.01 / 13.0 * ranks.sum(dim=1))
+            opp = torch.flip(b, dims=[1])
+            sign = torch.tensor([1.0, -1.0])[None, :, None]
+            h = ((torch.arange(NUM_HANDS) % 7).float() - 3.0) * 0.002
+            hv = sign * 0.05 * w[:, None, None] * (NUM_HANDS * opp - 1.0) + h[None, None, :]
+            return ModelOutput(policy_logits=torch.zeros(b.shape[0], NUM_HANDS, self.num_actions),
+                               value=torch.zeros(b.shape[0]), hand_values=hv)
+
+    rng = np.random.default_rng(515)
+    cols = np.sort(rng.choice(NUM_HANDS, 64, replace=False))
+    out = {"columns": cols, "case_names": np.array([c[0] for c in CASES])}
+    dev = torch.device("cpu")
+    bins = [0.5, 1.0]
+    for name, depth, iters, scripts in CASES:
+        n = len(scripts)
+        env = HUNLTensorEnv(num_envs=n, starting_stack=1000, sb=50, bb=100, default_bet_bins=list(bins), device=dev)
+        deck = torch.stack([torch.from_numpy(rng.permutation(52)[:9].copy()) for _ in range(n)])
+        env.reset(force_button=torch.tensor([s[0] for s in scripts]), force_deck=deck)
+        for step in range(max(len(s[1]) for s in scripts)):
+            env.step_bins(torch.tensor([s[1][step] if step < len(s[1]) else -1 for s in scripts], dtype=torch.long))
+        assert not env.done.any()
+
+        cfg = Config()
+        cfg.device = "cpu"
+        cfg.num_envs = n
+        cfg.train = TrainingConfig()
+        cfg.model = ModelConfig()
+        cfg.model.num_actions = len(bins) + 3
+        cfg.env = EnvConfig()
+        cfg.env.stack, cfg.env.sb, cfg.env.bb, cfg.env.bet_bins, cfg.env.flop_showdown = 1000, 50, 100, bins, False
+        cfg.search = SearchConfig()
+        cfg.search.iterations = iters
+        cfg.search.warm_start_iterations = 0
+        cfg.search.depth = depth
+        cfg.search.dcfr_alpha, cfg.search.dcfr_beta, cfg.search.dcfr_gamma = 1.5, 0.0, 2.0
+        cfg.search.dcfr_plus_delay = 0
+        cfg.search.cfr_type = CFRType["discounted"]
+        cfg.search.cfr_plus = False
+        cfg.search.cfr_avg = False
+        ev = SparseCFREvaluator(model=ValueNet(len(bins) + 3), device=dev, cfg=cfg)
+        ev.chance_helper.FLOP_SAMPLE_SIZE = 0
+        ev.chance_helper.NUM_PERM_SAMPLES = 0
+
+        bel = rng.gamma(0.5, size=(n, 2, NUM_HANDS)).astype(np.float32)
+        bel /= bel.sum(-1, keepdims=True)
+        for f in ENV_FIELDS:
+            out[f"{name}/root/{f}"] = getattr(env, f).clone().numpy()
+        ev.initialize_subgame(env, torch.arange(n), initial_beliefs=torch.from_numpy(bel.copy()))
+        ev.initialize_policy_and_beliefs()
+        ev.set_leaf_values(0)
+        ev.compute_expected_values()
+        ev.values_avg[:] = ev.latest_values
+        ev.t_sample = torch.full((ev.total_nodes,), -1, dtype=torch.long)
+        for t in range(iters):
+            ev.cfr_iteration(t)
+        for s in STATE:
+            x = getattr(ev, s).detach().numpy()
+            out[f"{name}/state/{s}"] = np.ascontiguousarray(x[..., cols]).astype(np.float32)
+            out[f"{name}/state/{s}_rowsum"] = x.astype(np.float64).sum(-1)
+        # the encoder alone, on every node, with the leaf rule for the board (cfr_evaluator.py:1031-1033)
+        enc = ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask)
+        out[f"{name}/encode_leaf/context"] = enc.context.numpy()
+        out[f"{name}/encode_leaf/board"] = enc.board.numpy()
+        out[f"{name}/encode_leaf/to_act"] = enc.to_act.numpy()
+        out[f"{name}/encode_leaf/street"] = enc.street.numpy()
+        out[f"{name}/new_street_mask"] = ev.new_street_mask.numpy()
+        out[f"{name}/leaf_mask"] = ev.leaf_mask.numpy()
+
+        batches = dict(zip(("value", "pre_value", "policy"), ev.training_data()))
+        for tag, batch in batches.items():
+            p = f"{name}/{tag}"
+            out[f"{p}/len"] = np.int64(len(batch))
+            out[f"{p}/context"] = batch.features.context.numpy()
+            out[f"{p}/board"] = batch.features.board.numpy()
+            out[f"{p}/to_act"] = batch.features.to_act.numpy()
+            out[f"{p}/street"] = batch.features.street.numpy()
+            fb = batch.features.beliefs.numpy().reshape(-1, 2, NUM_HANDS)
+            out[f"{p}/beliefs"] = np.ascontiguousarray(fb[..., cols])
+            out[f"{p}/beliefs_rowsum"] = fb.astype(np.float64).sum(-1)
+            out[f"{p}/legal_masks"] = batch.legal_masks.numpy()
+            if batch.value_targets is not None:
+                out[f"{p}/value_targets"] = batch.value_targets.numpy().astype(np.float32)
+            if batch.policy_targets is not None:
+                pt = batch.policy_targets.numpy()
+                out[f"{p}/policy_targets"] = np.ascontiguousarray(pt[:, cols, :]).astype(np.float32)
+                out[f"{p}/policy_targets_sum"] = pt.astype(np.float64).sum(axis=1)
+            for k, v in batch.statistics.items():
+                out[f"{p}/stat/{k}"] = v.numpy()
+        out[f"{name}/beliefs"] = bel
+        out[f"{name}/depth_offsets"] = np.array(ev.depth_offsets, dtype=np.int64)
+        out[f"{name}/settings"] = np.array([str(depth), str(iters)])
+        print(name, "nodes", ev.total_nodes, "depth offsets", ev.depth_offsets,
+              {k: len(b) for k, b in batches.items()}, flush=True)
+    path = os.path.join(HERE, "training_data_golden.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, os.path.getsize(path) // 1024, "KiB")
+
+
+if __name__ == "__main__":
+    main()

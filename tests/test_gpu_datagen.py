@@ -1,0 +1,263 @@
+"""GPU parity of the steps either side of the search in data generation: feature encoding, bet
+amounts, policy targets (kernels against the oracle on seeded inputs) and ``training_data`` of
+the evaluator against vectors written by running the reference's evaluator
+(tests/golden/training_data_golden.npz) and against the oracle on the same search."""
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cards as OC
+from oracle import cfr as OCFR
+from oracle import chance as OCH
+from oracle import datagen as ODG
+from tests.test_oracle_datagen import BINS, load_case, value_net_numpy
+
+pytestmark = pytest.mark.gpu
+H = 1326
+DEV = "cuda"
+
+
+class ValueNet:
+    """torch twin of ``ValueNet`` in tests/golden/gen_training_data_golden.py."""
+    enforce_zero_sum = False
+
+    def eval(self):
+        pass
+
+    def __call__(self, f):
+        b = f.beliefs.view(-1, 2, H).float()
+        ranks = torch.where(f.board >= 0, (f.board % 13 + 1).float(), torch.zeros_like(f.board, dtype=torch.float32))
+        w = (0.2 + 0.1 * f.context[:, 2] + 0.05 * f.context[:, 1] - 0.03 * f.context[:, 3]
+             + 0.01 / 13.0 * ranks.sum(dim=1))
+        opp = torch.flip(b, dims=[1])
+        sign = torch.tensor([1.0, -1.0], device=b.device)[None, :, None]
+        h = ((torch.arange(H, device=b.device) % 7).float() - 3.0) * 0.002
+        return SimpleNamespace(hand_values=sign * 0.05 * w[:, None, None] * (H * opp - 1.0) + h[None, None, :])
+
+
+def random_env(rng, m):
+    street = rng.integers(0, 4, m)
+    board = np.full((m, 5), -1, dtype=np.int64)
+    for i in range(m):
+        k = [0, 3, 4, 5][street[i]]
+        board[i, :k] = rng.permutation(52)[:k]
+    actions = rng.integers(0, 4, m)
+    env = {"to_act": rng.integers(0, 2, m), "button": rng.integers(0, 2, m),
+           "starting_stacks": rng.integers(0, 3, (m, 2)) * rng.integers(1, 30000, (m, 2)),
+           "pot": rng.integers(0, 50000, m), "committed": rng.integers(0, 3, (m, 2)) * rng.integers(0, 500, (m, 2)),
+           "stacks": rng.integers(0, 20000, (m, 2)), "actions_this_round": actions, "street": street,
+           "board_indices": board, "last_board_indices": ODG.previous_board(street, actions, board)}
+    return {k: v.astype(np.int64) for k, v in env.items()}
+
+
+def as_namespace(env):
+    return SimpleNamespace(**{k: torch.from_numpy(v).to(DEV) for k, v in env.items()})
+
+
+def test_encode_matches_oracle_all_argument_forms():
+    from poker2_amd.rebel_feature_encoder import RebelFeatureEncoder
+    rng = np.random.default_rng(40)
+    m = 777
+    env = random_env(rng, m)
+    bel = rng.random((m, 2, H)).astype(np.float32)
+    enc = RebelFeatureEncoder(as_namespace(env))
+    tb = torch.from_numpy(bel).to(DEV)
+    pre = rng.random(m) < 0.5
+    idx = rng.permutation(m)[:100]
+    for kw_o, kw_p in (({}, {}), ({"pre_chance_node": True}, {"pre_chance_node": True}),
+                       ({"pre_chance_node": pre}, {"pre_chance_node": torch.from_numpy(pre).to(DEV)}),
+                       ({"pre_chance_node": pre, "indices": idx},
+                        {"pre_chance_node": torch.from_numpy(pre).to(DEV), "indices": torch.from_numpy(idx).to(DEV)}),
+                       ({"pre_chance_node": False, "indices": idx}, {"pre_chance_node": False, "indices": torch.from_numpy(idx)})):
+        exp = ODG.encode(env, bel, **kw_o)
+        got = enc.encode(tb, **kw_p)
+        assert np.array_equal(got.context.cpu().numpy(), exp["context"])          # same float32 operations: exact
+        assert np.array_equal(got.board.cpu().numpy(), exp["board"])
+        assert np.array_equal(got.to_act.cpu().numpy(), exp["to_act"])
+        assert np.array_equal(got.street.cpu().numpy(), exp["street"])
+        assert np.array_equal(got.beliefs.cpu().numpy(), exp["beliefs"])
+    empty = enc.encode(tb, indices=torch.zeros(0, dtype=torch.long, device=DEV))
+    assert len(empty) == 0 and empty.context.shape == (0, 4)
+
+
+def test_bet_amounts_match_oracle():
+    from poker2_amd.evaluator import _TreeEnv
+    rng = np.random.default_rng(41)
+    m = 1000
+    env = random_env(rng, m)
+    for bins in ([0.5, 1.0], [0.33, 0.75, 1.5], [], [0.25, 0.5, 1.0, 2.0, 4.0]):
+        ns = as_namespace(env)
+        te = _TreeEnv(N=m, default_bet_bins=bins, legal_mask=None, **vars(ns))
+        got, _ = te.legal_bins_amounts_and_mask()
+        assert np.array_equal(got.cpu().numpy(), ODG.bet_amounts(env, bins)), bins    # int64: exact
+
+
+def golden_evaluator(case, fused):
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel
+    from poker2_amd.tree import RootStates
+    r = {k[5:]: v for k, v in case.items() if k.startswith("root/")}
+    n = len(r["street"])
+    roots = RootStates.from_env(SimpleNamespace(bb=100, **r), np.arange(n))
+    depth, iters = int(case["settings"][0]), int(case["settings"][1])
+    cfg = river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0)
+    model = NetworkLeafModel(ValueNet(), DEV)
+    ev = HipSparseCFREvaluator(model, torch.device(DEV), cfg, fused_iteration=fused)
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(case["beliefs"]))
+    ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+    for t in range(iters):
+        ev.cfr_iteration(t)
+    ev.chance_helper.FLOP_SAMPLE_SIZE, ev.chance_helper.NUM_PERM_SAMPLES = 0, 0
+    return ev, r
+
+
+def batch_as_dict(b):
+    out = {"features": {"context": b.features.context, "board": b.features.board, "to_act": b.features.to_act,
+                        "street": b.features.street, "beliefs": b.features.beliefs},
+           "legal_masks": b.legal_masks, "statistics": dict(b.statistics)}
+    if b.value_targets is not None:
+        out["value_targets"] = b.value_targets
+    if b.policy_targets is not None:
+        out["policy_targets"] = b.policy_targets
+
+    def host(x):
+        return {k: host(v) for k, v in x.items()} if isinstance(x, dict) else x.cpu().numpy()
+    return host(out)
+
+
+def close(got, exp, mask, rtol, atol, what):
+    """Agreement on the entries of ``mask``; elsewhere (hands the board blocks, where the
+    one-kernel evaluator and the base class legitimately differ) nothing is asserted."""
+    m = np.broadcast_to(mask, got.shape)
+    err = np.abs(got - exp) - (atol + rtol * np.abs(exp))
+    assert (err[m] <= 0).all(), f"{what}: max abs diff {np.abs(got - exp)[m].max():.3e}"
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("name", ["streets_mixed", "preflop"])
+def test_training_data_matches_vectors_from_the_reference(golden_dir, name, fused):
+    case, cols = load_case(golden_dir, name)
+    ev, r = golden_evaluator(case, fused)
+    assert list(ev.depth_offsets) == case["depth_offsets"].tolist()
+    n = ev.root_nodes
+    assert np.array_equal(ev.env.last_board_indices[:n].cpu().numpy(), r["last_board_indices"])
+    # the encoder alone on every node, board chosen by the leaf rule
+    f = ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask)
+    np.testing.assert_allclose(f.context.cpu().numpy(), case["encode_leaf/context"], rtol=1e-6, atol=0)
+    assert np.array_equal(f.board.cpu().numpy(), case["encode_leaf/board"])
+    assert np.array_equal(f.to_act.cpu().numpy(), case["encode_leaf/to_act"])
+    assert np.array_equal(f.street.cpu().numpy(), case["encode_leaf/street"])
+    allowed_root = OC.allowed_hands_for_boards(r["board_indices"])[0]              # [n, H]
+    batches = [batch_as_dict(b) for b in ev.training_data()]
+    rtol, atol = 3e-4, 3e-6          # float32; four iterations of regret matching behind the targets
+    for got, tag in zip(batches, ("value", "pre_value", "policy")):
+        k = int(case[f"{tag}/len"])
+        ft = got["features"]
+        assert ft["context"].shape[0] == k
+        if k == 0:
+            continue
+        np.testing.assert_allclose(ft["context"], case[f"{tag}/context"], rtol=1e-6, atol=0)
+        assert np.array_equal(ft["board"], case[f"{tag}/board"])
+        assert np.array_equal(ft["to_act"], case[f"{tag}/to_act"])
+        assert np.array_equal(ft["street"], case[f"{tag}/street"])
+        assert np.array_equal(got["legal_masks"], case[f"{tag}/legal_masks"])
+        for s, v in got["statistics"].items():
+            ref = case[f"{tag}/stat/{s}"]
+            if np.issubdtype(ref.dtype, np.floating):
+                np.testing.assert_allclose(v, ref, rtol=3e-3, atol=5e-5, err_msg=s)
+            else:
+                assert np.array_equal(v, ref), s
+        # rows of this batch -> their roots, for the mask of hands the board allows
+        if tag == "policy":
+            rows = np.nonzero(~ev.tree.leaf_mask[:ev.depth_offsets[-2]])[0]
+            root_of = ev.tree.root_index[rows]
+        elif tag == "value":
+            root_of = np.nonzero(~((r["street"] == 0) & (r["actions_this_round"] == 0)))[0]
+        else:
+            root_of = np.nonzero((r["actions_this_round"] == 0) & (r["street"] >= 1) & (r["street"] <= 3))[0]
+        ok = allowed_root[root_of]                                                   # [k, H]
+        fb = ft["beliefs"].reshape(k, 2, H)
+        if tag == "pre_value":      # ranges before the deal: the hands the dealt cards block still carry mass
+            np.testing.assert_allclose(fb[..., cols], case[f"{tag}/beliefs"], rtol=1e-6, atol=0)
+        else:
+            close(fb[..., cols], case[f"{tag}/beliefs"], ok[:, None, cols], rtol, atol, f"{tag} beliefs")
+        if "value_targets" in got:
+            mask = ok[:, None, :] if tag == "value" else np.ones((k, 1, H), bool)
+            close(got["value_targets"], case[f"{tag}/value_targets"], mask, rtol, atol, f"{tag} value targets")
+        if "policy_targets" in got:
+            pt = got["policy_targets"]
+            assert pt.shape == (k, H, len(BINS) + 3)
+            close(pt[:, cols, :], case[f"{tag}/policy_targets"], ok[:, cols, None], rtol, atol, "policy targets")
+            illegal = ~case[f"{tag}/legal_masks"]
+            assert not pt.transpose(0, 2, 1)[illegal].any()                          # no child, no probability
+
+
+@pytest.mark.parametrize("name", ["streets_mixed"])
+def test_training_data_matches_oracle_everywhere(golden_dir, name):
+    """Against the oracle following the one-kernel evaluator's conventions: every entry, blocked
+    hands included."""
+    from tests.test_gpu_evaluator import tree_as_dict
+    case, cols = load_case(golden_dir, name)
+    ev, r = golden_evaluator(case, True)
+    tree = tree_as_dict(ev.tree)
+    tree.update({k: v for k, v in ev.tree.state.items() if k not in tree})
+    env = ODG.tree_env(tree, r["board_indices"])
+
+    def leaf_fn(beliefs, rows):
+        f = ODG.encode(env, beliefs, pre_chance_node=tree["new_street_mask"], indices=rows)
+        return value_net_numpy(f["context"], f["street"], f["to_act"], f["board"], f["beliefs"])
+    iters = int(case["settings"][1])
+    o = OCFR.OracleCFR(tree, r["board_indices"], case["beliefs"], cfr_iterations=iters, leaf_value_fn=leaf_fn,
+                       t_sample_roots=np.full(ev.root_nodes, -1, dtype=np.int64), fused_variant=True)
+    o.prepare()
+    for t in range(iters):
+        o.cfr_iteration(t)
+    canonical, count, _ = OCH.canonical_flops()
+    exp = ODG.training_data(o, env, BINS, value_net_numpy, flop_tables=(canonical, count, OCH.combo_suit_perms()))
+    got = [batch_as_dict(b) for b in ev.training_data()]
+
+    def same(a, b, path):
+        if isinstance(b, dict):
+            assert set(a) == set(b), path
+            for k in b:
+                same(a[k], b[k], f"{path}/{k}")
+        elif np.issubdtype(np.asarray(b).dtype, np.floating):
+            # float32; regret matching divides by small regret sums, so a handful of policy entries
+            # (and what is built from them) move by more than the 3e-4 of the rest
+            tol = (3e-3, 5e-5) if "local_" in path else (3e-4, 3e-6)
+            err = np.abs(a - b) - (tol[1] + tol[0] * np.abs(b))
+            assert (err > 0).sum() <= max(2, 1e-4 * err.size) and np.abs(a - b).max() < 1e-3, \
+                f"{path}: {(err > 0).sum()} entries off, max abs diff {np.abs(a - b).max():.3e}"
+        else:
+            assert np.array_equal(a, b), path
+    for a, b, tag in zip(got, exp, ("value", "pre_value", "policy")):
+        same(a, b, tag)
+
+
+def test_policy_targets_kernel_matches_pull_back_on_a_deep_tree():
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    from oracle import best_response as OBR
+    from tests.helpers import random_boards
+    rng = np.random.default_rng(43)
+    n = 5
+    boards = random_boards(rng, n, 5)
+    roots = RootStates.at_round_start(3, rng.integers(100, 400, n), rng.integers(300, 2000, (n, 2)), boards)
+    ev = HipSparseCFREvaluator(None, torch.device(DEV), river_dcfr_config(n, iterations=2, depth=5))
+    ev.initialize_subgame(roots, np.arange(n))
+    ev.policy_probs_avg.copy_(torch.from_numpy(rng.random((ev.total_nodes, H)).astype(np.float32)))
+    top = ev.depth_offsets[-2]
+    shim = SimpleNamespace(num_actions=ev.num_actions, parent_index=ev.tree.parent_index,
+                           action_from_parent=ev.tree.action_from_parent,
+                           _level=lambda level: (0, top, ev.depth_offsets[1], ev.total_nodes))
+    exp = np.transpose(OBR.pull_back(shim, ev.policy_probs_avg.cpu().numpy()), (0, 2, 1))
+    rows = torch.from_numpy(rng.permutation(top)[: top // 2]).to(DEV)             # any rows, any order, leaves too
+    got = ev._policy_targets(rows).cpu().numpy()
+    assert np.array_equal(got, exp[rows.cpu().numpy()])                             # a gather: exact
+    assert ev._policy_targets(rows[:0]).shape == (0, H, ev.num_actions)
+    with pytest.raises(IndexError):
+        ev._policy_targets(torch.tensor([ev.total_nodes], device=DEV))
