@@ -22,4 +22,6 @@ Parity status
 * chance nodes (one card, flop): pinned by vectors written from the reference's own helper
   (``tests/golden/chance_golden.npz``, ``flop_chance_golden.npz``), per-sample loops and closed
   forms (``oracle/chance.py``).
+* feature encoding and training targets: pinned by vectors written from the reference's own
+  evaluator, encoder and chance helper (``tests/golden/training_data_golden.npz``; ``oracle/datagen.py``).
 """

@@ -78,6 +78,11 @@ class SampledLeaves:
     beliefs: torch.Tensor    # [K, 2, 1326]
     roots: RootStates        # K root states for ``initialize_subgame``
 
+    @property
+    def env(self) -> RootStates:
+        """The public states under the reference's attribute name (PublicBeliefState.env)."""
+        return self.roots
+
 
 class _TreeEnv(SimpleNamespace):
     """Per-node public states of the tree under the reference env's attribute names."""
@@ -752,15 +757,36 @@ class HipSparseCFREvaluator:
         keep = sampled[sampled >= n]            # roots that are leaves themselves are not continued
         rows = keep.cpu().numpy()
         tree = self.tree
-        fields = {}
+        root_of = tree.root_index[rows]
+        # The cards a sampled leaf sees: a leaf that closed a betting round stands on the next
+        # street, whose cards come from its root's runout (the reference env deals them from the
+        # deck it was reset with, hunl_tensor_env.py:900-975); roots without one get theirs drawn here.
+        if self._roots.runout is not None:
+            runout = self._roots.runout[root_of]
+        else:
+            runout = self._draw_runout(tree.board[root_of])
+        street = np.asarray(tree.state["street"])[rows]
+        shown = np.arange(5)[None, :] < CARDS_ON_STREET[np.clip(street, 0, 4)][:, None]
+        fields = {"board": np.where(shown, runout, -1), "last_board": tree.board[root_of].copy(), "runout": runout,
+                  "bb": int(self.env.bb)}
         for name in RootStates.__dataclass_fields__:
-            if name == "board":
-                fields[name] = tree.board[tree.root_index[rows]]
-            elif name == "bb":
-                fields[name] = int(self.env.bb)
-            else:
+            if name not in fields:
                 fields[name] = np.asarray(tree.state[name])[rows]
         return SampledLeaves(nodes=keep, beliefs=self.beliefs[keep].clone(), roots=RootStates(**fields))
+
+    def _draw_runout(self, boards: np.ndarray) -> np.ndarray:
+        """Complete each board [K,5] to five cards with uniformly drawn cards that are not on it."""
+        gen, dev = self.generator, self.device
+        gdev = gen.device if gen is not None else dev
+        b = torch.from_numpy(np.ascontiguousarray(boards)).to(gdev)
+        k = b.shape[0]
+        scores = torch.rand(k, 52, generator=gen, device=gdev)
+        dealt = b >= 0
+        scores[torch.arange(k, device=gdev)[:, None].expand(-1, 5)[dealt], b[dealt]] = -1.0
+        fresh = torch.topk(scores, 5, dim=1).indices               # five distinct cards off the board, random order
+        slot = (~dealt).long().cumsum(dim=1) - 1                    # which fresh card an empty slot takes
+        out = torch.where(dealt, b, fresh.gather(1, slot.clamp(min=0)))
+        return out.cpu().numpy()
 
     # ------------------------------------------------------------------ training data
     @property

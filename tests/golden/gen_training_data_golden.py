@@ -12,6 +12,7 @@ reset state is dropped from the value batch).  The leaf network is a closed-form
 encoded features (written out in ``ValueNet`` below; tests restate it), so the search, the
 encoder and the chance nodes all feed the stored targets.  The flop chance node runs in its
 exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
+A last section holds what the env's ``reset`` deals from a seeded CPU generator.
 """
 from __future__ import annotations
 
@@ -165,6 +166,15 @@ def main() -> None:
         out[f"{name}/settings"] = np.array([str(depth), str(iters)])
         print(name, "nodes", ev.total_nodes, "depth offsets", ev.depth_offsets,
               {k: len(b) for k, b in batches.items()}, flush=True)
+    # the env's own reset (hunl_tensor_env.py:219-346) from a seeded CPU generator: button, deck, stacks
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(99)
+    env = HUNLTensorEnv(num_envs=16, mean_stack=1000, sb=50, bb=100, default_bet_bins=list(bins), device=dev, rng=gen,
+                        randomize_stacks=True)
+    env.reset()
+    for f in ENV_FIELDS + ("deck",):
+        out[f"reset/{f}"] = getattr(env, f).clone().numpy()
+    out["reset/seed"] = np.int64(99)
     path = os.path.join(HERE, "training_data_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path) // 1024, "KiB")

@@ -261,3 +261,111 @@ def test_policy_targets_kernel_matches_pull_back_on_a_deep_tree():
     assert ev._policy_targets(rows[:0]).shape == (0, H, ev.num_actions)
     with pytest.raises(IndexError):
         ev._policy_targets(torch.tensor([ev.total_nodes], device=DEV))
+
+
+# ---- the loop around the search ---------------------------------------------------------------
+class ListBuffer:
+    def __init__(self):
+        self.batches = []
+
+    def add_batch(self, batch):
+        self.batches.append(batch)
+
+
+def test_sampled_leaves_are_dealt_from_the_runout_or_fresh_cards():
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel
+    from poker2_amd.tree import CARDS_ON_STREET, RootStates
+    rng = np.random.default_rng(50)
+    n = 64
+    runout = np.stack([rng.permutation(52)[:5] for _ in range(n)]).astype(np.int64)
+    boards = runout.copy()
+    boards[:, 4] = -1                                                    # turn roots
+    beliefs = torch.full((n, 2, H), 1.0 / H)
+    for with_runout in (True, False):
+        roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[900, 900]], (n, 1)), boards,
+                                          button=np.arange(n) % 2)
+        if with_runout:
+            roots.runout = runout
+        gen = torch.Generator(device=DEV)
+        gen.manual_seed(5)
+        ev = HipSparseCFREvaluator(NetworkLeafModel(ValueNet(), DEV), torch.device(DEV),
+                                   river_dcfr_config(n, iterations=4, depth=3, dcfr_delay=0), generator=gen)
+        ev.initialize_subgame(roots, np.arange(n), beliefs)
+        nxt = ev.evaluate_cfr()
+        k = nxt.nodes.numel()
+        assert 0 < k <= n and nxt.env is nxt.roots and nxt.beliefs.shape == (k, 2, H)
+        rows = nxt.nodes.cpu().numpy()
+        root_of = ev.tree.root_index[rows]
+        r = nxt.roots
+        closed = ev.tree.new_street_mask[rows]
+        assert closed.any() and (~closed).any()
+        assert np.array_equal(r.street, np.where(closed, 3, 2))
+        assert np.array_equal(r.last_board, boards[root_of])              # the board before any deal
+        assert np.array_equal(r.board[:, :4], boards[root_of][:, :4])
+        assert (r.board[~closed, 4] == -1).all()
+        river = r.board[closed, 4]
+        assert ((river >= 0) & (river < 52)).all()
+        assert not (river[:, None] == boards[root_of][closed][:, :4]).any()   # a card that was not out yet
+        if with_runout:
+            assert np.array_equal(river, runout[root_of][closed, 4])
+            assert np.array_equal(r.runout, runout[root_of])
+        shown = np.arange(5)[None, :] < CARDS_ON_STREET[r.street][:, None]
+        assert np.array_equal(np.where(shown, r.runout, -1), r.board)
+        # the sampled states are valid roots of the next search, ranges included
+        ev.initialize_subgame(r, np.arange(k), nxt.beliefs)
+        ev.prepare_search()
+        assert torch.isfinite(ev.values_avg).all()
+        on_board = torch.zeros(k, 52, dtype=torch.bool)
+        bb = torch.from_numpy(r.board)
+        on_board[torch.arange(k)[:, None].expand(-1, 5)[bb >= 0], bb[bb >= 0]] = True
+        from poker2_amd.card_utils import hand_combos_tensor
+        cm = hand_combos_tensor()
+        blocked = on_board[:, cm[:, 0]] | on_board[:, cm[:, 1]]
+        assert not ev.beliefs[:k].cpu()[blocked[:, None, :].expand(-1, 2, -1)].any()   # the new card blocks hands
+
+
+def test_data_generator_loop_plays_hands_forward():
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel
+    from poker2_amd.rebel_data_generator import EnvProto, RebelDataGenerator
+    n = 24
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(11)
+    cpu_gen = torch.Generator(device="cpu")
+    cpu_gen.manual_seed(12)
+    ev = HipSparseCFREvaluator(NetworkLeafModel(ValueNet(), DEV), torch.device(DEV),
+                               river_dcfr_config(n, iterations=4, depth=3, dcfr_delay=0), generator=gen)
+    ev.sample_epsilon = 0.25
+    values, policies = ListBuffer(), ListBuffer()
+    dg = RebelDataGenerator(EnvProto(mean_stack=1000, randomize_stacks=True, rng=cpu_gen), ev, values, policies)
+    dg.evaluator.chance_helper.FLOP_SAMPLE_SIZE = 32            # keep the flop chance node small here
+    assert dg.current_pbs.env.n == n and (dg.current_pbs.env.street == 0).all()
+    streets_seen = set()
+    total_value = 0
+    for _ in range(4):
+        value_batch, policy_batch = dg.generate_data(40)
+        assert value_batch is not None and policy_batch is not None
+        total_value += len(value_batch)
+        streets_seen |= set(value_batch.statistics["street"].cpu().tolist())
+        assert value_batch.value_targets.shape[1:] == (2, H) and policy_batch.policy_targets.shape[1:] == (H, 5)
+        assert torch.isfinite(value_batch.value_targets).all() and value_batch.value_targets.abs().max() <= 1.0
+        # a policy target row is a distribution over the legal actions for every hand the board allows
+        s = policy_batch.policy_targets.sum(dim=2)
+        assert ((s - 1.0).abs() < 1e-4).logical_or(s.abs() < 1e-6).all()
+        assert not policy_batch.policy_targets.permute(0, 2, 1)[~policy_batch.legal_masks].any()
+        assert dg.last_extra >= 0
+        pbs = dg.current_pbs
+        assert pbs.beliefs.shape[0] == pbs.env.n <= n
+    assert len(values.batches) == 2 * len(policies.batches) and total_value >= 160
+    assert {1, 2}.issubset(streets_seen)                         # hands move on to later streets
+    # pre-chance samples: the state before the deal, on the previous street's board and stage
+    pre = [b for b in values.batches[1::2] if len(b)]
+    assert pre
+    for b in pre:
+        st = b.statistics["street"]
+        assert (b.statistics["stage"] == 2 * st + 1).all()
+        cards = (b.features.board >= 0).sum(dim=1).cpu()
+        assert torch.equal(cards, torch.tensor([0, 3, 4, 5])[st.cpu()])
