@@ -62,6 +62,8 @@ def test_device_builder_from_mid_round_roots():
             fields[name] = first.board[first.root_index[rows]]
         elif name == "bb":
             fields[name] = 100
+        elif name in ("last_board", "runout"):
+            fields[name] = None
         else:
             fields[name] = np.asarray(first.state[name])[rows]
     roots = RootStates(**fields)
