@@ -127,6 +127,39 @@ def cases(repeats: int):
     yield ("chance_expand states=3584 x48", k * (2 + 2 * 48) * H * 4,
            lambda: CH.chance_expand(pre, roots, tb, cards_on_board=4))
     yield ("chance_mean states=3584 x48", k * (2 * 48 + 2) * H * 4, lambda: CH.chance_mean(post, offsets))
+    del post
+
+    # --- flop chance node: 64 preflop states x 256 drawn canonical flops, 6 of 24 suit permutations
+    from .card_utils import combo_suit_permutation_tensor
+    ks, kf = 64, 256
+    canonical, count, _, _ = CH.canonical_flops()
+    flops = torch.from_numpy(canonical[rng.integers(0, canonical.shape[0], kf)]).to(dev)
+    pre_f = bel[:ks].contiguous()
+    roots_f = torch.arange(ks, device=dev)
+    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops))
+    hv = CH.flop_expand(pre_f, roots_f, flops)
+    perms = combo_suit_permutation_tensor(dev)[:6].to(torch.int16).contiguous()
+    w = torch.full((kf,), 1.0 / kf, device=dev)
+    yield (f"perm_mean states={ks} x{kf} perms=6", ks * (2 * kf + 2) * H * 4, lambda: CH.perm_mean(hv, perms, w))
+    del hv
+
+    # --- data generation: policy targets and features of a 4096-root river search (21 nodes per root)
+    from .config import river_dcfr_config
+    from .evaluator import HipSparseCFREvaluator
+    from .tree import RootStates
+    n = 4096
+    roots_r = RootStates.at_round_start(3, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards.cpu().numpy())
+    ev = HipSparseCFREvaluator(None, dev, river_dcfr_config(n, iterations=1, depth=2))
+    ev.initialize_subgame(roots_r, np.arange(n), bel)
+    ev.policy_probs_avg.uniform_()
+    top = ev.depth_offsets[-2]
+    rows = torch.nonzero(~ev.leaf_mask[:top]).squeeze(1)
+    n_children = int(ev.child_count[rows].sum())
+    yield (f"policy_targets nodes={rows.numel()}", (n_children + rows.numel() * ev.num_actions) * H * 4,
+           lambda: ev._policy_targets(rows))
+    all_rows = torch.arange(ev.total_nodes, device=dev)
+    yield (f"encode nodes={ev.total_nodes}", ev.total_nodes * (13 * 8 + 16 + 5 * 8 + 10 * 8),
+           lambda: ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask))
 
 
 def main() -> None:

@@ -141,6 +141,9 @@ def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, fl
     return post
 
 
+PERM_MEAN_TARGET_WORKGROUPS = 2048   # 256 CUs x 8
+
+
 def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tensor,
               out: torch.Tensor | None = None) -> torch.Tensor:
     """hand_values [B,K,2,1326] fp32, perms [P,1326] hand-index maps (P <= 24), weight [K] ->
@@ -161,8 +164,11 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
         out = torch.empty(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     else:
         assert out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()
+    # enough workgroups to fill the chip: 2 per state, times shares of the flops
+    shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
+    workspace = torch.empty(shares, b, 2, NUM_HANDS, dtype=torch.float32, device=dev) if shares > 1 else None
     _lib.call("p2hip_perm_mean", _lib.ptr(hv), b, k, _lib.ptr(pt), int(pt.shape[0]), _lib.ptr(w), int(accumulate),
-              _lib.ptr(out), _lib.stream_ptr())
+              _lib.ptr(out), _lib.ptr(workspace), shares, _lib.stream_ptr())
     return out
 
 

@@ -257,49 +257,111 @@ __global__ __launch_bounds__(CH_BLOCK) void flop_expand_kernel(const float* __re
 
 // out[i][p][h] (+)= sum_f weight[f] * mean_q hand_values[i][f][p][perms[q][h]]
 // (the suit-orbit mean of _avg_over_perms, chance_node_helper.py:18-28, and the weighted sum over
-// flops, :352-357).  One workgroup per (state, player); the permutation table lives in LDS.
+// flops, :352-357).  A workgroup takes one (state, player) and one contiguous share of the flops:
+// each row goes through LDS once (the next one is already in flight in registers while the current
+// one is gathered), the permutation table is packed two hands per dword - in registers for up to
+// CH_REG_PERMS permutations, in LDS beyond - and the sums run in fp64.  With more than one share
+// the workgroups write partial sums that perm_reduce_kernel adds in a fixed order.
 constexpr int CH_MAX_PERMS = 24;
+constexpr int CH_REG_PERMS = 8;
 __global__ __launch_bounds__(CH_BLOCK) void perm_mean_kernel(const float* __restrict__ hand_values,
                                                               const int16_t* __restrict__ perms, int n_perms,
                                                               const float* __restrict__ weight, int64_t n_flops,
-                                                              int accumulate, float* __restrict__ out) {
+                                                              int64_t flops_per_share, int accumulate,
+                                                              float* __restrict__ dst, int64_t dst_share_stride) {
   extern __shared__ __align__(8) unsigned char lds_raw[];
-  float* row = reinterpret_cast<float*>(lds_raw);                          // [H + 2]
-  int16_t* ptab = reinterpret_cast<int16_t*>(lds_raw + (P2_H + 2) * 4);    // [n_perms][H]
-  const int64_t i = blockIdx.x;
-  const int p = blockIdx.y;
-  for (int e = threadIdx.x; e < n_perms * P2_H; e += CH_BLOCK) ptab[e] = perms[e];
+  float* rows = reinterpret_cast<float*>(lds_raw);                                  // [2][H + 2]
+  uint32_t* ptab = reinterpret_cast<uint32_t*>(lds_raw + 2 * (P2_H + 2) * 4);       // [n_perms][HPAIRS]
+  const int64_t i = blockIdx.x >> 1;
+  const int p = blockIdx.x & 1;
+  const int64_t f0 = (int64_t)blockIdx.y * flops_per_share;
+  const int64_t f1 = f0 + flops_per_share < n_flops ? f0 + flops_per_share : n_flops;
+  const bool in_regs = n_perms <= CH_REG_PERMS;
+  uint32_t preg[CH_REG_PERMS][CH_PPT];
+#pragma unroll
+  for (int q = 0; q < CH_REG_PERMS; ++q)
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      preg[q][k] = (in_regs && q < n_perms && idx < P2_HPAIRS)
+                       ? reinterpret_cast<const uint32_t*>(perms + (int64_t)q * P2_H)[idx] : 0u;
+    }
+  if (!in_regs)
+    for (int e = threadIdx.x; e < n_perms * P2_HPAIRS; e += CH_BLOCK) {
+      const int q = e / P2_HPAIRS, idx = e - q * P2_HPAIRS;
+      ptab[e] = reinterpret_cast<const uint32_t*>(perms + (int64_t)q * P2_H)[idx];
+    }
   double acc[CH_PPT][2];
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) acc[k][0] = acc[k][1] = 0.0;
   const float inv_perms = 1.0f / (float)n_perms;
-  for (int64_t f = 0; f < n_flops; ++f) {
-    p2_sync_lds();   // the previous row has been consumed (and, first time, ptab is complete)
+  float2 next[CH_PPT];
+  auto fetch = [&](int64_t f) {
     const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
-    for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += CH_BLOCK) reinterpret_cast<float2*>(row)[idx] = src[idx];
-    p2_sync_lds();
-    const float w = weight[f];
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      next[k] = idx < P2_HPAIRS ? src[idx] : make_float2(0.f, 0.f);
+    }
+  };
+  if (f0 < f1) fetch(f0);
+  int buf = 0;
+  for (int64_t f = f0; f < f1; ++f, buf ^= 1) {
+    float* row = rows + buf * (P2_H + 2);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx < P2_HPAIRS) reinterpret_cast<float2*>(row)[idx] = next[k];
+    }
+    if (f + 1 < f1) fetch(f + 1);
+    p2_sync_lds();   // row f is complete; the other buffer (row f-1) was consumed before this barrier
+    const float w = weight[f] * inv_perms;
 #pragma unroll
     for (int k = 0; k < CH_PPT; ++k) {
       const int idx = threadIdx.x + k * CH_BLOCK;
       if (idx >= P2_HPAIRS) continue;
+      float s0 = 0.f, s1 = 0.f;
+      if (in_regs) {
 #pragma unroll
-      for (int q2 = 0; q2 < 2; ++q2) {
-        const int h = 2 * idx + q2;
-        float s = 0.f;
-        for (int q = 0; q < n_perms; ++q) s += row[ptab[q * P2_H + h]];
-        acc[k][q2] += (double)(w * (s * inv_perms));
+        for (int q = 0; q < CH_REG_PERMS; ++q)
+          if (q < n_perms) {
+            s0 += row[preg[q][k] & 0xFFFFu];
+            s1 += row[preg[q][k] >> 16];
+          }
+      } else {
+        for (int q = 0; q < n_perms; ++q) {
+          const uint32_t e = ptab[q * P2_HPAIRS + idx];
+          s0 += row[e & 0xFFFFu];
+          s1 += row[e >> 16];
+        }
       }
+      acc[k][0] += (double)(w * s0);
+      acc[k][1] += (double)(w * s1);
     }
   }
-  float2* o = p2_row2(out, i * 2 + p);
+  float2* o = p2_row2(dst + (int64_t)blockIdx.y * dst_share_stride, i * 2 + p);
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) {
     const int idx = threadIdx.x + k * CH_BLOCK;
     if (idx >= P2_HPAIRS) continue;
-    float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
+    const float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
     o[idx] = make_float2(prev.x + (float)acc[k][0], prev.y + (float)acc[k][1]);
   }
+}
+
+// out (+)= sum over shares of partial[share], shares added in ascending order.
+__global__ __launch_bounds__(CH_BLOCK) void perm_reduce_kernel(const float2* __restrict__ partial, int shares,
+                                                                int64_t npairs, int accumulate,
+                                                                float2* __restrict__ out) {
+  const int64_t e = (int64_t)blockIdx.x * CH_BLOCK + threadIdx.x;
+  if (e >= npairs) return;
+  float2 s = accumulate ? out[e] : make_float2(0.f, 0.f);
+  for (int j = 0; j < shares; ++j) {
+    const float2 v = partial[(int64_t)j * npairs + e];
+    s.x += v.x;
+    s.y += v.y;
+  }
+  out[e] = s;
 }
 
 }  // namespace p2
@@ -346,19 +408,35 @@ int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int
 }
 
 int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
-                    const float* weight, int accumulate, float* out, void* stream) {
-  if (n < 0 || n_flops < 0 || n_perms < 1 || n_perms > p2::CH_MAX_PERMS) return P2_EINVAL;
+                    const float* weight, int accumulate, float* out, float* workspace, int shares, void* stream) {
+  if (n < 0 || n_flops < 0 || n_perms < 1 || n_perms > p2::CH_MAX_PERMS || shares < 1) return P2_EINVAL;
   if (n == 0) return 0;
   if (!hand_values || !perms || !weight || !out || !p2_aligned8(hand_values) || !p2_aligned8(out)) return P2_EINVAL;
-  if (n > 0x7FFFFFFF) return P2_EINVAL;
-  const size_t lds = (size_t)(P2_H + 2) * 4 + (size_t)n_perms * P2_H * 2;   // 69 KB with all 24 permutations
+  if (((uintptr_t)perms & 3) != 0) return P2_EINVAL;
+  if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
+  if (shares > 1 && (!workspace || !p2_aligned8(workspace))) return P2_EINVAL;
+  const size_t lds = (size_t)2 * (P2_H + 2) * 4 +
+                     (n_perms > p2::CH_REG_PERMS ? (size_t)n_perms * P2_HPAIRS * 4 : 0);   // 10.6 KB, or 74 KB with all 24
   if (lds > 64 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(p2::perm_mean_kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL(p2::perm_mean_kernel, dim3((unsigned)n, 2), dim3(p2::CH_BLOCK), lds, (hipStream_t)stream,
-                     hand_values, perms, n_perms, weight, n_flops, accumulate, out);
+  const int64_t per_share = (n_flops + shares - 1) / shares;
+  const int64_t npairs = n * 2 * P2_HPAIRS;
+  if (shares == 1) {
+    hipLaunchKernelGGL(p2::perm_mean_kernel, dim3((unsigned)(2 * n), 1), dim3(p2::CH_BLOCK), lds, (hipStream_t)stream,
+                       hand_values, perms, n_perms, weight, n_flops, per_share, accumulate, out, (int64_t)0);
+    P2_LAUNCH_CHECK();
+    return 0;
+  }
+  hipLaunchKernelGGL(p2::perm_mean_kernel, dim3((unsigned)(2 * n), (unsigned)shares), dim3(p2::CH_BLOCK), lds,
+                     (hipStream_t)stream, hand_values, perms, n_perms, weight, n_flops, per_share, 0, workspace,
+                     npairs * 2);
+  P2_LAUNCH_CHECK();
+  const int64_t grid = (npairs + p2::CH_BLOCK - 1) / p2::CH_BLOCK;
+  hipLaunchKernelGGL(p2::perm_reduce_kernel, dim3((unsigned)grid), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     (const float2*)workspace, shares, npairs, accumulate, (float2*)out);
   P2_LAUNCH_CHECK();
   return 0;
 }

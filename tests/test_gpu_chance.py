@@ -269,6 +269,16 @@ def test_perm_mean_matches_numpy(K, n_perms):
     again = K.perm_mean(torch.from_numpy(hv).cuda(), torch.from_numpy(perms).cuda(), torch.from_numpy(w).cuda(),
                         out=got.clone())
     np.testing.assert_allclose(again.cpu().numpy(), 2 * exp, rtol=1e-5, atol=4e-6)
+    # many states: one workgroup per (state, player) walks all flops and writes the result itself
+    hv = rng.standard_normal((1100, 3, 2, H)).astype(np.float32)
+    w = rng.random(3).astype(np.float32)
+    exp = np.zeros((1100, 2, H))
+    for k in range(3):
+        exp += w[k] * np.mean([hv[:, k][..., q] for q in perms], axis=0, dtype=np.float64)
+    base = rng.standard_normal((1100, 2, H)).astype(np.float32)
+    got = K.perm_mean(torch.from_numpy(hv).cuda(), torch.from_numpy(perms).cuda(), torch.from_numpy(w).cuda(),
+                      out=torch.from_numpy(base).cuda())
+    np.testing.assert_allclose(got.cpu().numpy(), base + exp, rtol=1e-5, atol=4e-6)
 
 
 def test_helper_flop_cache_matches_the_reference_cache(K, golden_dir):
