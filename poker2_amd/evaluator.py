@@ -730,15 +730,19 @@ class HipSparseCFREvaluator:
         sampling_masks[:top] &= ~done_src
         sampling_counts = sampling_masks.float().sum(dim=-1, keepdim=True)
         uniform = torch.where(sampling_masks, 1 / sampling_counts, torch.zeros_like(sampling_counts))
-        probs_by_src = self._pull_back(self.policy_probs_sample)
-        probs_by_src.masked_fill_(done_src[:, :, None], 0.0)
-        denom = probs_by_src.sum(dim=1, keepdim=True)
-        probs_by_src = torch.where(denom >= 1e-12, probs_by_src / denom, uniform[:top, :, None])
         child_action_index = self.child_mask.int().cumsum(dim=1) - self.child_mask.int()
         effective_leaf = self.leaf_mask | (sampling_counts.squeeze(1) == 0)
         actor_beliefs = self.beliefs[:n].gather(
             1, self.env.to_act[:n, None, None].expand(-1, -1, NUM_HANDS)).squeeze(1)
         selected_hands = multinomial(actor_beliefs)
+        # Only the column of each root's drawn hand is ever looked at: take it before pulling the
+        # sampling policy back to [node, action] (the reference pulls back all 1326 columns).
+        hand_of_node = selected_hands[self._root_index]
+        probs_node = self.policy_probs_sample.gather(1, hand_of_node[:, None]).squeeze(1)
+        probs_by_src = self._pull_back(probs_node)
+        probs_by_src.masked_fill_(done_src, 0.0)
+        denom = probs_by_src.sum(dim=1, keepdim=True)
+        probs_by_src = torch.where(denom >= 1e-12, probs_by_src / denom, uniform[:top])
         sampled = torch.arange(n, device=dev)
         depth = 0
         active = ~effective_leaf[sampled]
@@ -748,8 +752,7 @@ class HipSparseCFREvaluator:
             to_act = self.env.to_act[nodes]
             explore = torch.rand(nodes.numel(), generator=gen, device=gdev).to(dev) < sample_epsilon
             explore &= to_act == players[active]
-            p_active = probs_by_src[nodes, :, selected_hands[active]]
-            actions = multinomial(torch.where(explore[:, None], uniform[nodes], p_active))
+            actions = multinomial(torch.where(explore[:, None], uniform[nodes], probs_by_src[nodes]))
             sampled[active] = self.child_offsets[nodes] + child_action_index[nodes, actions]
             active = ~effective_leaf[sampled]
             depth += 1
