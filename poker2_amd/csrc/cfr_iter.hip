@@ -426,17 +426,15 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
         float vnext[2][SD_PPT];
         if (i + 1 < sd1) showdown_gather(leaf_beliefs + A.root_showdown_nodes[i + 1] * 2 * P2_H, sdr, vnext);
         // the EVs land in the sorted-range buffers, which the evaluation no longer needs by then
-        showdown_eval(vk, sdr, L.u.sd, L.u.sd.v[0], L.u.sd.v[1], A.potential[2 * c], A.potential[2 * c + 1],
-                      A.scale[c]);
+        showdown_eval(vk, sdr, L.u.sd, L.u.sd.v, A.potential[2 * c], A.potential[2 * c + 1], A.scale[c]);
         p2_sync_lds();
         float2 v[2][IT_PPT];
-        {
-          const float2* e0 = reinterpret_cast<const float2*>(L.u.sd.v[0]);
-          const float2* e1 = reinterpret_cast<const float2*>(L.u.sd.v[1]);
-          IT_FOR(j) {
-            v[0][j] = ln.ok[j] ? e0[ln.idx[j]] : make_float2(0.f, 0.f);
-            v[1][j] = ln.ok[j] ? e1[ln.idx[j]] : make_float2(0.f, 0.f);
-          }
+        IT_FOR(j) {
+          // hands 2*idx and 2*idx+1, each holding (hero 0, hero 1)
+          const float2 x = ln.ok[j] ? L.u.sd.v[2 * ln.idx[j]] : make_float2(0.f, 0.f);
+          const float2 y = ln.ok[j] ? L.u.sd.v[2 * ln.idx[j] + 1] : make_float2(0.f, 0.f);
+          v[0][j] = make_float2(x.x, y.x);
+          v[1][j] = make_float2(x.y, y.y);
         }
         st(A.latest, c * 2, v[0], ln);
         st(A.latest, c * 2 + 1, v[1], ln);

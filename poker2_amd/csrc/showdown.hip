@@ -216,11 +216,13 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_setup_kernel(const void* __
 // ---- per-call evaluation ---------------------------------------------------------
 constexpr int SD_PPT = 6;  // consecutive sorted positions per thread: 256 * 6 = 1536 >= 1326
 
-// Everything the evaluation of one node needs in LDS.
+// Everything the evaluation of one node needs in LDS.  The two heroes index every table alike
+// (positions, tie groups and card lists depend on the board only), so their values sit side by
+// side and one 64-bit LDS access serves both.
 struct ShowdownLds {
-  __align__(8) float v[2][P2_H + 2];        // villain-of-hero-p range in strength order: v[p] = beliefs[1-p] sorted
-  float P[2][P2_H + 2];        // exclusive prefix, P[p][k], k = 0..1326
-  float Pc[2][P2_CARDS][52];   // per-card exclusive prefix, Pc[p][c][j], j = 0..51
+  __align__(8) float2 v[P2_H + 2];        // .x / .y = villain-of-hero-0 / -1 range in strength order (beliefs[1] / [0] sorted)
+  float2 P[P2_H + 2];                     // exclusive prefix, k = 0..1326
+  float2 Pc[P2_CARDS][52];                // per-card exclusive prefix, Pc[c][j], j = 0..51
   float part[2][SD_WAVES];
 };
 
@@ -282,38 +284,37 @@ __device__ __forceinline__ void showdown_gather(const float* __restrict__ bel, c
   }
 }
 
-// Showdown EV of both players from gathered ranges, written in combo order to ev0 / ev1 (LDS,
-// 1326 floats each) already multiplied by mul0 / mul1 and divided by `div`; 0 for combos blocked
-// by the board.  ev0 / ev1 may be s.v[0] / s.v[1] (dead by the time they are written).  Uses LDS
-// barriers only; the caller puts an LDS barrier before reading ev0 / ev1 and another before the
-// next call.
+// Showdown EV of both players from gathered ranges, written in combo order to ev ((hero 0, hero 1)
+// per combo, 1326 float2 in LDS) already multiplied by mul0 / mul1 and divided by `div`; 0 for
+// combos blocked by the board.  ev may be s.v (dead by the time it is written).  Uses LDS barriers
+// only; the caller puts an LDS barrier before reading ev and another before the next call.
 // First half of showdown_eval: sorted ranges, their prefix and the per-card prefixes into LDS.
 // Ends with an LDS barrier.
 __device__ __forceinline__ void showdown_scans(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int k0 = threadIdx.x * SD_PPT;
-  float local[2], incl[2];
+  float local[2] = {0.f, 0.f}, incl[2];
+#pragma unroll
+  for (int i = 0; i < SD_PPT; ++i) {
+    if (k0 + i < P2_H) s.v[k0 + i] = make_float2(vk[0][i], vk[1][i]);
+    local[0] += vk[0][i];
+    local[1] += vk[1][i];
+  }
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
-    local[p] = 0.f;
-#pragma unroll
-    for (int i = 0; i < SD_PPT; ++i) {
-      if (k0 + i < P2_H) s.v[p][k0 + i] = vk[p][i];
-      local[p] += vk[p][i];
-    }
     incl[p] = p2_wave_scan_incl(local[p]);
     if (lane == 63) s.part[p][wave] = incl[p];
   }
   p2_sync_lds();
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    float base = 0.f;
-    for (int w = 0; w < wave; ++w) base += s.part[p][w];
-    float run = base + (incl[p] - local[p]);
+  {
+    float base0 = 0.f, base1 = 0.f;
+    for (int w = 0; w < wave; ++w) { base0 += s.part[0][w]; base1 += s.part[1][w]; }
+    float run0 = base0 + (incl[0] - local[0]), run1 = base1 + (incl[1] - local[1]);
 #pragma unroll
     for (int i = 0; i < SD_PPT; ++i) {
-      if (k0 + i <= P2_H) s.P[p][k0 + i] = run;
-      run += vk[p][i];
+      if (k0 + i <= P2_H) s.P[k0 + i] = make_float2(run0, run1);
+      run0 += vk[0][i];
+      run1 += vk[1][i];
     }
   }
   // per-card prefixes: one wave scan per (player, card); this wave owns cards wave, wave+4, ...
@@ -323,25 +324,18 @@ __device__ __forceinline__ void showdown_scans(const float (&vk)[2][SD_PPT], con
     const int c = wave + 4 * i;
     const uint32_t pos = R.clist[i];
     const bool in = pos < (uint32_t)P2_H;
-    float x0 = in ? s.v[0][pos] : 0.f;
-    float x1 = in ? s.v[1][pos] : 0.f;
+    const float2 x = in ? s.v[pos] : make_float2(0.f, 0.f);
+    float x0 = x.x, x1 = x.y;
     p2_wave_scan_incl2(x0, x1);
-    if (lane < 51) {
-      s.Pc[0][c][lane + 1] = x0;
-      s.Pc[1][c][lane + 1] = x1;
-    }
-    if (lane == 0) {
-      s.Pc[0][c][0] = 0.f;
-      s.Pc[1][c][0] = 0.f;
-    }
+    if (lane < 51) s.Pc[c][lane + 1] = make_float2(x0, x1);
+    if (lane == 0) s.Pc[c][0] = make_float2(0.f, 0.f);
   }
   p2_sync_lds();
 }
 
-// Second half: six LDS reads per hand and player, EVs written in combo order to ev0 / ev1.
+// Second half: eight 64-bit LDS reads per hand serve both players; EVs written in combo order to ev.
 __device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], const ShowdownRegs& R,
-                                                const ShowdownLds& s, float* ev0, float* ev1, float mul0, float mul1,
-                                                float div) {
+                                                const ShowdownLds& s, float2* ev, float mul0, float mul1, float div) {
   const float r0 = mul0 / div, r1 = mul1 / div;  // potential / scale of the node, one division each
 #pragma unroll
   for (int i = 0; i < SD_PPT; ++i) {
@@ -352,16 +346,19 @@ __device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], co
     const int a = (int)(R.ab[i] & 0xFFu), b = (int)(R.ab[i] >> 8);
     const int iLa = (int)(R.cidx[i] & 0xFFu), iRa = (int)((R.cidx[i] >> 8) & 0xFFu);
     const int iLb = (int)((R.cidx[i] >> 16) & 0xFFu), iRb = (int)(R.cidx[i] >> 24);
+    const float2 PL2 = s.P[L], PR2 = s.P[Rr];
+    const float2 aL2 = s.Pc[a][iLa], aR2 = s.Pc[a][iRa], bL2 = s.Pc[b][iLb], bR2 = s.Pc[b][iRb];
+    const float2 aT2 = s.Pc[a][51], bT2 = s.Pc[b][51];
     float e[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
       const float v0 = vk[p][i];
-      const float PL = s.P[p][L], PR = s.P[p][Rr];
-      const float aL = s.Pc[p][a][iLa], aR = s.Pc[p][a][iRa];
-      const float bL = s.Pc[p][b][iLb], bR = s.Pc[p][b][iRb];
+      const float PL = p ? PL2.y : PL2.x, PR = p ? PR2.y : PR2.x;
+      const float aL = p ? aL2.y : aL2.x, aR = p ? aR2.y : aR2.x;
+      const float bL = p ? bL2.y : bL2.x, bR = p ? bR2.y : bR2.x;
       const float win = PL - aL - bL;
       const float tie = (PR - PL) - (aR - aL) - (bR - bL) + v0;
-      float den = 1.0f - s.Pc[p][a][51] - s.Pc[p][b][51] + v0;
+      float den = 1.0f - (p ? aT2.y : aT2.x) - (p ? bT2.y : bT2.x) + v0;
       den = fmaxf(den, 1e-8f);
       // The kernel is VALU-issue bound and an IEEE division is about ten instructions, so both
       // quotients share one hardware reciprocal and are corrected by one fused residual step
@@ -374,15 +371,14 @@ __device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], co
       const float lp = valid ? 1.0f - wp - tp : 0.f;
       e[p] = (wp - lp) * keep;
     }
-    ev0[h] = e[0] * r0;
-    ev1[h] = e[1] * r1;
+    ev[h] = make_float2(e[0] * r0, e[1] * r1);
   }
 }
 
 __device__ __forceinline__ void showdown_eval(const float (&vk)[2][SD_PPT], const ShowdownRegs& R, ShowdownLds& s,
-                                              float* ev0, float* ev1, float mul0, float mul1, float div) {
+                                              float2* ev, float mul0, float mul1, float div) {
   showdown_scans(vk, R, s);
-  showdown_finish(vk, R, s, ev0, ev1, mul0, mul1, div);
+  showdown_finish(vk, R, s, ev, mul0, mul1, div);
 }
 
 // out[n] = showdown EV of both players at node n.
@@ -423,15 +419,14 @@ __global__ __launch_bounds__(SD_BLOCK, 3) void showdown_both_kernel(const float*
     showdown_scans(vk, R, s);
     if (more) showdown_gather(beliefs + nn * 2 * P2_H, Rn, vkn);
     // the EVs go over the sorted ranges, which are dead once the card scans are done
-    showdown_finish(vk, R, s, s.v[0], s.v[1], mul0, mul1, div);
+    showdown_finish(vk, R, s, s.v, mul0, mul1, div);
     p2_sync_lds();
     float2* o0 = p2_row2(out, n * 2);
     float2* o1 = p2_row2(out, n * 2 + 1);
-    const float2* e0 = reinterpret_cast<const float2*>(s.v[0]);
-    const float2* e1 = reinterpret_cast<const float2*>(s.v[1]);
     for (int i = threadIdx.x; i < P2_HPAIRS; i += SD_BLOCK) {
-      o0[i] = e0[i];
-      o1[i] = e1[i];
+      const float2 x = s.v[2 * i], y = s.v[2 * i + 1];   // hands 2i, 2i+1: (hero 0, hero 1) each
+      o0[i] = make_float2(x.x, y.x);
+      o1[i] = make_float2(x.y, y.y);
     }
     p2_sync_lds();  // the next node overwrites s.v
   }
