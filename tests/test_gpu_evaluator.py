@@ -404,3 +404,85 @@ def test_one_kernel_and_per_op_paths_agree_on_random_subgames(seed):
         bad = ((x - y).abs() > 2e-5 + 2e-4 * y.abs()).float().mean().item()
         assert bad <= 1e-3, f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type}: {name} {bad:.2e} " \
                             f"max {float((x - y).abs().max()):.3e}"
+
+
+# ---- full benchmark sizes: properties that do not depend on the size -------------------------
+def river_evaluator(n_roots, depth, max_raises, seed, iters, select=None):
+    """Evaluator on seeded river roots without the oracle (too slow at these sizes); `select`
+    keeps a subset of the SAME seeded roots."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(seed)
+    boards = random_boards(rng, n_roots)
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(3, np.full(n_roots, 200), np.tile([[800, 800]], (n_roots, 1)), boards,
+                                      button=np.arange(n_roots) % 2)
+    idx = np.arange(n_roots) if select is None else np.asarray(select)
+    cfg = river_dcfr_config(len(idx), iterations=iters, depth=depth)
+    ev = HipSparseCFREvaluator(None, torch.device("cuda"), cfg, max_raises=max_raises)
+    ev.initialize_subgame(roots, idx, torch.from_numpy(beliefs[idx]))
+    ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+    return ev
+
+
+def test_b4096_results_do_not_depend_on_the_batch():
+    """The benchmark workload (B=4096 river roots, 21 nodes each): a root's search is the same,
+    bit for bit, whether it runs among 4096 roots or among 256 of them."""
+    iters = 6
+    big = river_evaluator(4096, 2, None, seed=123, iters=iters)
+    sel = np.arange(1500, 1756)
+    small = river_evaluator(4096, 2, None, seed=123, iters=iters, select=sel)
+    for t in range(iters):
+        big.cfr_iteration(t)
+        small.cfr_iteration(t)
+    rows_big = np.nonzero(np.isin(big.tree.root_index, sel))[0]
+    # level-major layout, roots ascending inside a level: the subset's rows appear in the same order
+    assert np.array_equal(sel[small.tree.root_index], big.tree.root_index[rows_big])
+    rows_big = torch.from_numpy(rows_big).cuda()
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        assert torch.equal(getattr(big, name)[rows_big], getattr(small, name)), name
+    a, b = big._compute_exploitability(), small._compute_exploitability()
+    assert torch.equal(a.local_exploitability[torch.from_numpy(sel).cuda()], b.local_exploitability)
+
+
+def test_b1024_three_raise_tree_200_iterations_invariants():
+    """B=1024 river roots on the three-raise tree (105 nodes per root), 200 discounted-CFR
+    iterations: what holds at any size."""
+    iters, n = 200, 1024
+    ev = river_evaluator(n, 16, 3, seed=321, iters=iters)
+    assert ev.total_nodes == 105 * n
+    before = ev._compute_exploitability().local_exploitability
+    for t in range(iters):
+        ev.cfr_iteration(t)
+    top = ev.depth_offsets[-2]
+    for pol in (ev.policy_probs, ev.policy_probs_avg):
+        s = torch.zeros(top, 1326, device="cuda").index_add_(0, ev.parent_index[n:], pol[n:])
+        s = s[ev.child_count[:top] > 0]
+        assert (s - 1.0).abs().max() <= 1e-5
+        assert (pol[n:] >= 0).all()
+    for b in (ev.beliefs, ev.beliefs_avg):
+        assert (b.sum(-1) - 1.0).abs().max() <= 1e-5
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        assert torch.isfinite(getattr(ev, name)).all(), name
+    # Values are chips over the starting stack, so at most 1 in exact arithmetic.  The showdown EV
+    # divides by the opponent mass compatible with the hand, computed as 1 - cs[a] - cs[b] + v in
+    # float32 like the reference (cfr_evaluator.py:577-587): where that mass is zero up to
+    # rounding the quotient is noise of any size (the reference asserts only that win and tie mass
+    # are small there), and values_avg, which weighs the newest iteration about one half
+    # (t^gamma against (t+1)^gamma), carries it for a few iterations.  So: no entry above 1 where
+    # the opponent has real compatible mass, and few anywhere.
+    from poker2_amd.card_utils import calculate_unblocked_mass
+    compat = calculate_unblocked_mass(torch.flip(ev.beliefs, dims=[1]).reshape(-1, 1326)).reshape(ev.beliefs.shape)
+    over = ev.latest_values.abs() > 1.0 + 1e-4
+    assert not (over & (compat > 1e-2)).any()
+    assert over.float().mean() < 1e-4 and (ev.values_avg.abs() > 1.0 + 1e-4).float().mean() < 1e-4
+    blocked = ~ev.allowed_hands[n:]
+    assert (ev.self_reach[n:, 0][blocked] == 0).all() and (ev.self_reach[n:, 1][blocked] == 0).all()
+    # the game is zero-sum: the two players' range-weighted root values cancel
+    w = ev.beliefs_avg[:n]
+    total = (ev.values_avg[:n] * w).sum(-1).sum(-1)
+    assert total.abs().max() < 5e-3
+    # and the search did its job on every root: far less exploitable than the uniform start
+    after = ev._compute_exploitability().local_exploitability
+    assert (after < 0.5 * before).all() and after.max() < 0.15 and (after > -1e-4).all()
