@@ -55,3 +55,24 @@ def test_wrappers_fail_loudly_without_gpu():
         rules_hip.rank_7_cards_single_batch_triton(torch.zeros(4, 7, dtype=torch.int16))
     with pytest.raises((RuntimeError, ValueError)):
         fused_cfr_hip.unblocked_mass_triton(torch.zeros(2, 1326))
+    # the chance-node and data-generation wrappers have no CPU path either
+    from types import SimpleNamespace
+    from poker2_amd import chance_node_helper as CH
+    from poker2_amd.rebel_feature_encoder import RebelFeatureEncoder
+    z = torch.zeros(1, 2, 1326)
+    with pytest.raises((RuntimeError, ValueError)):
+        CH.chance_expand(z, torch.zeros(1, dtype=torch.long), torch.full((1, 5), -1))
+    with pytest.raises((RuntimeError, ValueError)):
+        CH.chance_mean(z, torch.tensor([0, 1]))
+    with pytest.raises((RuntimeError, ValueError)):
+        CH.flop_expand(z, torch.zeros(1, dtype=torch.long), torch.tensor([[0, 1, 2]]))
+    with pytest.raises((RuntimeError, ValueError)):
+        CH.perm_mean(torch.zeros(1, 1, 2, 1326), torch.arange(1326)[None], torch.ones(1))
+    env = SimpleNamespace(**{k: torch.zeros(1, dtype=torch.long) for k in ("to_act", "button", "pot", "actions_this_round")},
+                          starting_stacks=torch.ones(1, 2, dtype=torch.long), committed=torch.zeros(1, 2, dtype=torch.long),
+                          board_indices=torch.full((1, 5), -1), last_board_indices=torch.full((1, 5), -1))
+    with pytest.raises((RuntimeError, ValueError)):
+        RebelFeatureEncoder(env).encode(z)
+    helper = CH.ChanceNodeHelper(torch.device("cpu"), torch.float32, 2, model=None, autocast_dtype=None)
+    with pytest.raises((RuntimeError, ValueError)):
+        helper.flop_chance_values(torch.zeros(1, dtype=torch.long), None, z)
