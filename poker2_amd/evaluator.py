@@ -158,6 +158,7 @@ class HipSparseCFREvaluator:
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
         self._chance_helper = None
+        self.subgame_serial = 0
 
     @property
     def enforce_zero_sum(self) -> bool:
@@ -183,6 +184,7 @@ class HipSparseCFREvaluator:
         else:
             tree = build_sparse_tree(roots, self.bet_bins, self.max_depth, max_raises=self.max_raises)
         self.tree: SparseTree = tree
+        self.subgame_serial += 1           # lets leaf models drop what they cached for the previous subgame
         resident = getattr(tree, "device_arrays", None) or {}
 
         def tt(name, host_array):

@@ -57,10 +57,21 @@ class NetworkLeafModel:
         self.device = torch.device(device)
         self.enforce_zero_sum = enforce_zero_sum
         self.autocast_dtype = autocast_dtype
+        self._cached_for = None
+        self._cached = None
 
     @torch.no_grad()
     def leaf_values(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
-        feats = ev.feature_encoder.encode_rows(beliefs.contiguous(), rows, ev.new_street_mask[rows])
+        # Context and board of a leaf are public state: encoded once per subgame, only the ranges
+        # change from iteration to iteration (the reference re-encodes every time).
+        key = (id(ev), ev.subgame_serial, rows.data_ptr(), rows.numel())
+        beliefs = beliefs.contiguous()
+        if self._cached_for != key:
+            self._cached = ev.feature_encoder.encode_rows(beliefs, rows, ev.new_street_mask[rows])
+            self._cached_for = key
+        c = self._cached
+        feats = MLPFeatures(context=c.context, street=c.street, to_act=c.to_act, board=c.board,
+                            beliefs=beliefs.reshape(beliefs.shape[0], -1))
         if hasattr(self.net, "eval"):
             self.net.eval()
         if self.autocast_dtype is not None:
@@ -113,7 +124,7 @@ class ChanceLeafModel:
 
     @torch.no_grad()
     def leaf_values(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
-        key = (id(ev), id(ev.tree), rows.data_ptr(), rows.numel())
+        key = (id(ev), ev.subgame_serial, rows.data_ptr(), rows.numel())
         if self._plan_for != key:
             self._plan, self._plan_for = self._make_plan(rows, ev), key
         plan = self._plan

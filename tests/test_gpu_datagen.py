@@ -369,3 +369,35 @@ def test_data_generator_loop_plays_hands_forward():
         assert (b.statistics["stage"] == 2 * st + 1).all()
         cards = (b.features.board >= 0).sum(dim=1).cpu()
         assert torch.equal(cards, torch.tensor([0, 3, 4, 5])[st.cpu()])
+
+
+def test_leaf_model_does_not_reuse_features_of_the_previous_subgame():
+    """Two subgames of identical shape on one evaluator: the second must see its own pots and boards."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import ChanceLeafModel, NetworkLeafModel, RangeBoardMLP
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(60)
+    n = 8
+    beliefs = torch.full((n, 2, H), 1.0 / H)
+
+    def roots_of(pot, seed):
+        r = np.random.default_rng(seed)
+        boards = np.full((n, 5), -1, dtype=np.int64)
+        boards[:, :4] = np.stack([r.permutation(52)[:4] for _ in range(n)])
+        return RootStates.at_round_start(2, np.full(n, pot), np.tile([[900, 900]], (n, 1)), boards)
+    first, second = roots_of(200, 1), roots_of(600, 2)
+    net = RangeBoardMLP(hidden=32, layers=1, seed=1).to(DEV)
+    for make in (lambda: NetworkLeafModel(ValueNet(), DEV), lambda: ChanceLeafModel(net, DEV)):
+        cfg = river_dcfr_config(n, iterations=2, depth=2, dcfr_delay=0)
+        ev = HipSparseCFREvaluator(make(), torch.device(DEV), cfg, max_raises=1)
+        ev.initialize_subgame(first, np.arange(n), beliefs)
+        ev.prepare_search()
+        ev.initialize_subgame(second, np.arange(n), beliefs)
+        ev.prepare_search()
+        fresh = HipSparseCFREvaluator(make(), torch.device(DEV), cfg, max_raises=1)
+        fresh.initialize_subgame(second, np.arange(n), beliefs)
+        fresh.prepare_search()
+        assert torch.equal(ev.model_indices, fresh.model_indices)
+        assert torch.equal(ev.latest_values, fresh.latest_values)
+        assert ev.latest_values[ev.model_indices].abs().max() > 0
