@@ -73,6 +73,7 @@ struct IterArgs {
 };
 
 constexpr int IT_VSTRIDE = P2_H + 2;  // floats between vectors staged in LDS
+constexpr int IT_RED = 20;            // block-reduction slots: 2 + 2 * 8 children, rounded up
 
 template <int CH>
 struct IterLds {
@@ -81,7 +82,7 @@ struct IterLds {
     ShowdownLds sd;              // showdown scans (never live at the same time)
   } u;
   double cs[CH * P2_CARDS];
-  float red[IT_WAVES][4];
+  float red[2][IT_WAVES][IT_RED];   // two buffers, used alternately by consecutive block reductions
 };
 
 #define IT_FOR(j) _Pragma("unroll") for (int j = 0; j < IT_PPT; ++j)
@@ -127,7 +128,7 @@ __device__ __forceinline__ void unblocked_regs(float2 (&out)[IT_PPT], const floa
 }
 
 // Sums of up to four per-thread partials over the block; results to all threads.
-__device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[4]) {
+__device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[IT_RED]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int q = 0; q < 4; ++q) v[q] = p2_wave_sum(v[q]);
@@ -143,6 +144,32 @@ __device__ __forceinline__ void block_sum4(float (&v)[4], float (*red)[4]) {
 #pragma unroll
     for (int w = 0; w < IT_WAVES; ++w) s += red[w][q];
     v[q] = s;
+  }
+}
+
+// Sums of the first `n` (<= N) per-thread partials over the block; results to all threads.  One
+// barrier: the caller alternates between two `red` buffers from call to call, so a buffer is
+// rewritten only after a later barrier has seen every thread finish reading it.
+template <int N>
+__device__ __forceinline__ void block_sums(float (&v)[N], int n, float (*red)[IT_RED]) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int q = 0; q < N; ++q)
+    if (q < n) v[q] = p2_wave_sum(v[q]);
+  if (lane == 0) {
+#pragma unroll
+    for (int q = 0; q < N; ++q)
+      if (q < n) red[wave][q] = v[q];
+  }
+  p2_sync_lds();
+#pragma unroll
+  for (int q = 0; q < N; ++q) {
+    if (q < n) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < IT_WAVES; ++w) s += red[w][q];
+      v[q] = s;
+    }
   }
 }
 
@@ -366,42 +393,115 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
           st(A.policy_avg, first + k, pav[k], ln);
         }
       }
+      // Belief normalisers of the whole family in one block reduction: the player who does not
+      // act has the same reach at every child (two sums), the actor's differ per child.  The rows
+      // are then written array by array, so that each array receives the family's children as one
+      // contiguous run.
+      float2 rn_opp[IT_PPT], ran_opp[IT_PPT], ran_act[IT_PPT], rb_act[IT_PPT], rb_opp[IT_PPT], rba_act[IT_PPT],
+          rba_opp[IT_PPT];
+      IT_FOR(j) {
+        const bool a0 = actor == 0;
+        rn_opp[j] = a0 ? rn[1][j] : rn[0][j];
+        ran_act[j] = a0 ? ran[0][j] : ran[1][j];
+        ran_opp[j] = a0 ? ran[1][j] : ran[0][j];
+        rb_act[j] = a0 ? rb[0][j] : rb[1][j];
+        rb_opp[j] = a0 ? rb[1][j] : rb[0][j];
+        rba_act[j] = a0 ? rba[0][j] : rba[1][j];
+        rba_opp[j] = a0 ? rba[1][j] : rba[0][j];
+        rn_opp[j] = make_float2(am[j].x ? rn_opp[j].x : 0.f, am[j].y ? rn_opp[j].y : 0.f);
+        ran_opp[j] = make_float2(am[j].x ? ran_opp[j].x : 0.f, am[j].y ? ran_opp[j].y : 0.f);
+      }
+      float sums[2 + 2 * MAXC];
+#pragma unroll
+      for (int q = 0; q < 2 + 2 * MAXC; ++q) sums[q] = 0.f;
+      IT_FOR(j) {
+        const float2 vb = mul2(rb_opp[j], rn_opp[j]), vba = mul2(rba_opp[j], ran_opp[j]);
+        sums[0] += vb.x + vb.y;
+        sums[1] += vba.x + vba.y;
+      }
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          IT_FOR(j) {
+            float2 x = mul2(rn_act[j], cur[k][j]), y = mul2(ran_act[j], pav[k][j]);
+            x = make_float2(am[j].x ? x.x : 0.f, am[j].y ? x.y : 0.f);
+            y = make_float2(am[j].x ? y.x : 0.f, am[j].y ? y.y : 0.f);
+            const float2 vb = mul2(rb_act[j], x), vba = mul2(rba_act[j], y);
+            sums[2 + 2 * k] += vb.x + vb.y;
+            sums[3 + 2 * k] += vba.x + vba.y;
+          }
+        }
+      }
+      PROF_BEGIN(t_b2);
+      block_sums<2 + 2 * MAXC>(sums, 2 + 2 * cnt, L.red[(i - pp0) & 1]);
+      PROF_END(6, t_b2);
+      const float so = sums[0], soa = sums[1];
+      // reach
 #pragma unroll
       for (int k = 0; k < MAXC; ++k) {
         if (k < cnt) {
           const int64_t c = first + k;
-          float2 rc[2][IT_PPT], rca[2][IT_PPT], vb[2][IT_PPT], vba[2][IT_PPT];
-          float s4[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int pl = 0; pl < 2; ++pl) {
-            IT_FOR(j) {
-              float2 x = rn[pl][j], y = ran[pl][j];
-              if (pl == actor) { x = mul2(x, cur[k][j]); y = mul2(y, pav[k][j]); }
-              x = make_float2(am[j].x ? x.x : 0.f, am[j].y ? x.y : 0.f);
-              y = make_float2(am[j].x ? y.x : 0.f, am[j].y ? y.y : 0.f);
-              rc[pl][j] = x;
-              rca[pl][j] = y;
-              vb[pl][j] = mul2(rb[pl][j], x);
-              vba[pl][j] = mul2(rba[pl][j], y);
-              s4[pl] += vb[pl][j].x + vb[pl][j].y;
-              s4[2 + pl] += vba[pl][j].x + vba[pl][j].y;
-            }
-            st(A.reach, c * 2 + pl, rc[pl], ln);
-            st(A.reach_avg, c * 2 + pl, rca[pl], ln);
+          float2 xa[IT_PPT];
+          IT_FOR(j) {
+            const float2 x = mul2(rn_act[j], cur[k][j]);
+            xa[j] = make_float2(am[j].x ? x.x : 0.f, am[j].y ? x.y : 0.f);
           }
-          PROF_BEGIN(t_b2);
-          block_sum4(s4, L.red);
-          PROF_END(6, t_b2);
+          if (actor == 0) { st(A.reach, c * 2, xa, ln); st(A.reach, c * 2 + 1, rn_opp, ln); }
+          else { st(A.reach, c * 2, rn_opp, ln); st(A.reach, c * 2 + 1, xa, ln); }
+        }
+      }
+      // reach_avg
 #pragma unroll
-          for (int pl = 0; pl < 2; ++pl) {
-            float2 o[IT_PPT], oa[IT_PPT];
-            IT_FOR(j) {
-              o[j] = s4[pl] > 1e-5f ? make_float2(vb[pl][j].x / s4[pl], vb[pl][j].y / s4[pl]) : ap[j];
-              oa[j] = s4[2 + pl] > 1e-5f ? make_float2(vba[pl][j].x / s4[2 + pl], vba[pl][j].y / s4[2 + pl]) : ap[j];
-            }
-            st(A.beliefs, c * 2 + pl, o, ln);
-            st(A.beliefs_avg, c * 2 + pl, oa, ln);
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          const int64_t c = first + k;
+          float2 ya[IT_PPT];
+          IT_FOR(j) {
+            const float2 y = mul2(ran_act[j], pav[k][j]);
+            ya[j] = make_float2(am[j].x ? y.x : 0.f, am[j].y ? y.y : 0.f);
           }
+          if (actor == 0) { st(A.reach_avg, c * 2, ya, ln); st(A.reach_avg, c * 2 + 1, ran_opp, ln); }
+          else { st(A.reach_avg, c * 2, ran_opp, ln); st(A.reach_avg, c * 2 + 1, ya, ln); }
+        }
+      }
+      // beliefs
+      float2 bo[IT_PPT], boa[IT_PPT];
+      IT_FOR(j) {
+        const float2 vb = mul2(rb_opp[j], rn_opp[j]), vba = mul2(rba_opp[j], ran_opp[j]);
+        bo[j] = so > 1e-5f ? make_float2(vb.x / so, vb.y / so) : ap[j];
+        boa[j] = soa > 1e-5f ? make_float2(vba.x / soa, vba.y / soa) : ap[j];
+      }
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          const int64_t c = first + k;
+          const float sa = sums[2 + 2 * k];
+          float2 o[IT_PPT];
+          IT_FOR(j) {
+            float2 x = mul2(rn_act[j], cur[k][j]);
+            x = make_float2(am[j].x ? x.x : 0.f, am[j].y ? x.y : 0.f);
+            const float2 vb = mul2(rb_act[j], x);
+            o[j] = sa > 1e-5f ? make_float2(vb.x / sa, vb.y / sa) : ap[j];
+          }
+          if (actor == 0) { st(A.beliefs, c * 2, o, ln); st(A.beliefs, c * 2 + 1, bo, ln); }
+          else { st(A.beliefs, c * 2, bo, ln); st(A.beliefs, c * 2 + 1, o, ln); }
+        }
+      }
+      // beliefs_avg
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k) {
+        if (k < cnt) {
+          const int64_t c = first + k;
+          const float saa = sums[3 + 2 * k];
+          float2 oa[IT_PPT];
+          IT_FOR(j) {
+            float2 y = mul2(ran_act[j], pav[k][j]);
+            y = make_float2(am[j].x ? y.x : 0.f, am[j].y ? y.y : 0.f);
+            const float2 vba = mul2(rba_act[j], y);
+            oa[j] = saa > 1e-5f ? make_float2(vba.x / saa, vba.y / saa) : ap[j];
+          }
+          if (actor == 0) { st(A.beliefs_avg, c * 2, oa, ln); st(A.beliefs_avg, c * 2 + 1, boa, ln); }
+          else { st(A.beliefs_avg, c * 2, boa, ln); st(A.beliefs_avg, c * 2 + 1, oa, ln); }
         }
       }
     }
@@ -522,7 +622,7 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
           }
           float shift = 0.f;
           if (enforce_zs) {
-            block_sum4(s4, L.red);
+            block_sum4(s4, L.red[0]);
             shift = (A.node_flags[c] & NODE_DONE) ? 0.f : 0.5f * s4[0];
           }
 #pragma unroll
@@ -552,7 +652,7 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
         }
         float shift = 0.f;
         if (enforce_zs) {
-          block_sum4(s4, L.red);
+          block_sum4(s4, L.red[0]);
           shift = (A.node_flags[p] & NODE_DONE) ? 0.f : 0.5f * s4[0];
         }
 #pragma unroll
