@@ -354,9 +354,11 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
       float2 psum[IT_PPT];
       IT_FOR(j) psum[j] = make_float2(0.f, 0.f);
 #pragma unroll
+      for (int k = 0; k < MAXC; ++k)
+        if (k < cnt) ld(cur[k], A.policy, first + k, ln);
+#pragma unroll
       for (int k = 0; k < MAXC; ++k) {
         if (k < cnt) {
-          ld(cur[k], A.policy, first + k, ln);
           if (avg_copy) {
             IT_FOR(j) pav[k][j] = cur[k][j];
           } else {
