@@ -34,7 +34,7 @@ TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2), "raise3": (1
 # HBM bytes per launch of the iteration kernel from two rocprofv3 --pmc passes (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy): an offline
 # measurement per workload, quoted in the JSON line; None where no counter run exists.
-MEASURED_TRAFFIC_BYTES = {("depth2", 4096): 6.03e9 + 6.81e9}
+MEASURED_TRAFFIC_BYTES = {("depth2", 4096): 6.00e9 + 6.80e9}
 
 
 def synth_roots(n: int, seed: int):
