@@ -203,30 +203,33 @@ class HipSparseCFREvaluator:
         self.action_from_parent = tt("action_from_parent", tree.action_from_parent)
         self.child_count = tt("child_count", tree.child_count)
         self.child_offsets = tt("child_offsets", tree.child_offsets)
-        self.prev_actor = self._t(tree.prev_actor)
+        self.prev_actor = tt("prev_actor", tree.prev_actor)
         self.legal_mask = tt("legal_mask", tree.legal_mask)
-        self.leaf_mask = self._t(tree.leaf_mask)
-        self.new_street_mask = self._t(tree.new_street_mask)
+        self.leaf_mask = tt("leaf_mask", tree.leaf_mask)
+        self.new_street_mask = tt("new_street_mask", tree.new_street_mask)
         self.child_mask = self.legal_mask & (~self.leaf_mask)[:, None]
         st = tree.state
         # Boards per node.  Every action saves the board before cards are dealt
         # (hunl_tensor_env.py:862): below the roots the previous board is the root's board.  The
         # current board of a node that closed a betting round shows the next cards only when the
         # roots carry their runout.
-        node_board = tree.board[tree.root_index]
-        last_board = node_board.copy()
-        last_board[:N] = roots.previous_board()
+        d_root_index = tt("root_index", tree.root_index)
+        d_last_board = self._t(tree.board)[d_root_index]
+        d_last_board[:N] = self._t(roots.previous_board())
         if roots.runout is not None:
-            shown = np.arange(5)[None, :] < CARDS_ON_STREET[np.clip(st["street"], 0, 4)][:, None]
-            node_board = np.where(shown, roots.runout[tree.root_index], -1)
+            cards = self._t(CARDS_ON_STREET)[tt("street", st["street"]).clamp(0, 4)]
+            shown = torch.arange(5, device=dev)[None, :] < cards[:, None]
+            d_node_board = torch.where(shown, self._t(roots.runout)[d_root_index], torch.full_like(d_last_board, -1))
+        else:
+            d_node_board = self._t(tree.board)[d_root_index]
         self._roots = roots
         self.env = _TreeEnv(
-            N=T, to_act=tt("to_act", st["to_act"]), done=self._t(st["done"]), street=tt("street", st["street"]),
-            pot=tt("pot", st["pot"]), stacks=self._t(st["stacks"]), committed=self._t(st["committed"]),
-            starting_stacks=self._t(st["starting_stacks"]), scale=self._t(st["scale"]),
+            N=T, to_act=tt("to_act", st["to_act"]), done=tt("done", st["done"]), street=tt("street", st["street"]),
+            pot=tt("pot", st["pot"]), stacks=tt("stacks", st["stacks"]), committed=tt("committed", st["committed"]),
+            starting_stacks=tt("starting_stacks", st["starting_stacks"]), scale=tt("scale", st["scale"]),
             actions_this_round=tt("actions_this_round", st["actions_this_round"]), button=tt("button", st["button"]),
-            min_raise=tt("min_raise", st["min_raise"]), is_allin=self._t(st["is_allin"]),
-            board_indices=self._t(node_board), last_board_indices=self._t(last_board), bb=roots.bb,
+            min_raise=tt("min_raise", st["min_raise"]), is_allin=tt("is_allin", st["is_allin"]),
+            board_indices=d_node_board, last_board_indices=d_last_board, bb=roots.bb,
             default_bet_bins=list(self.bet_bins), legal_mask=self.legal_mask)
         self.feature_encoder = (self.model.create_feature_encoder(self.env, device=dev, dtype=self.float_dtype)
                                 if hasattr(self.model, "create_feature_encoder")
@@ -236,8 +239,11 @@ class HipSparseCFREvaluator:
         self.model_indices = self._t(np.nonzero(model_mask)[0].astype(np.int64))
         self.showdown_indices = self._t(np.nonzero(tree.showdown_mask)[0].astype(np.int64))
         self.showdown_actors = self.env.to_act[self.showdown_indices]
-        self.showdown_potential = self._t(tree.showdown_potential[tree.showdown_mask])
-        self._potential_all = self._t(tree.showdown_potential.astype(np.float32))
+        d_potential = resident.get("showdown_potential")
+        if d_potential is None:
+            d_potential = self._t(tree.showdown_potential)
+        self.showdown_potential = d_potential[self.showdown_indices]
+        self._potential_all = d_potential.to(torch.float32)
 
         def z1():
             return torch.zeros(T, NUM_HANDS, dtype=self.float_dtype, device=dev)
@@ -256,8 +262,8 @@ class HipSparseCFREvaluator:
         self.self_reach[:N] = 1.0
         self.self_reach_avg = self.self_reach.clone()
         self.latest_values = z2()
-        folded = self._t(tree.fold_mask)
-        rew = self._t(tree.reward)
+        folded = tt("fold_mask", tree.fold_mask)
+        rew = tt("reward", tree.reward)
         self.latest_values[folded, 0] = rew[folded][:, None]
         self.latest_values[folded, 1] = -rew[folded][:, None]
         self.values_avg = self.latest_values.clone()

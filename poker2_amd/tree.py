@@ -406,10 +406,12 @@ def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: in
     child_count = torch.cat(count_l)
     total = offsets[-1]
     child_offsets = (n + torch.cumsum(child_count, 0) - child_count).contiguous()
-    table = nodes.cpu().numpy()                     # the one bulk copy back to the host
+    # the one bulk copy back to the host, column-major so that every column is a contiguous row
+    columns = nodes.t().contiguous()
+    table = columns.cpu().numpy()
 
     def c(name):
-        return np.ascontiguousarray(table[:, col[name]])
+        return table[col[name]]
     state = {
         "street": c("street"), "to_act": c("to_act"), "button": c("button"), "pot": c("pot"),
         "stacks": np.stack([c("stack0"), c("stack1")], axis=1),
@@ -437,10 +439,31 @@ def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: in
                       fold_mask=(action == 0) & state["done"], showdown_mask=state["street"] == 4,
                       reward=reward, state=state, board=np.array(roots.board))
     object.__setattr__(tree, "device_arrays", {
-        "parent_index": nodes[:, col["parent"]].contiguous(), "action_from_parent": nodes[:, col["action"]].contiguous(),
-        "child_count": child_count, "child_offsets": child_offsets, "root_index": nodes[:, col["root"]].contiguous(),
-        "legal_mask": legal, "to_act": nodes[:, col["to_act"]].contiguous(), "street": nodes[:, col["street"]].contiguous(),
-        "pot": nodes[:, col["pot"]].contiguous(), "button": nodes[:, col["button"]].contiguous(),
-        "actions_this_round": nodes[:, col["actions_this_round"]].contiguous(),
+        "parent_index": columns[col["parent"]], "action_from_parent": columns[col["action"]],
+        "child_count": child_count, "child_offsets": child_offsets, "root_index": columns[col["root"]],
+        "legal_mask": legal, "to_act": columns[col["to_act"]], "street": columns[col["street"]],
+        "pot": columns[col["pot"]], "button": columns[col["button"]],
+        "actions_this_round": columns[col["actions_this_round"]], "min_raise": columns[col["min_raise"]],
+        "stacks": torch.stack([columns[col["stack0"]], columns[col["stack1"]]], dim=1),
+        "committed": torch.stack([columns[col["comm0"]], columns[col["comm1"]]], dim=1),
+        "starting_stacks": torch.stack([columns[col["start0"]], columns[col["start1"]]], dim=1),
+        "is_allin": torch.stack([columns[col["allin0"]], columns[col["allin1"]]], dim=1).bool(),
+        "done": columns[col["done"]].bool(),
+        "scale": columns[col["scale"]].to(torch.int32).view(torch.float32),
+        "reward": columns[col["reward"]].to(torch.int32).view(torch.float32),
+    })
+    # masks the evaluator keeps on the device, derived there instead of copied back
+    d_done = tree.device_arrays["done"]
+    d_new_street = (columns[col["actions_this_round"]] == 0)
+    d_new_street[:n] = False
+    d_leaf = d_done | d_new_street
+    d_leaf[offsets[-2]:] = True
+    d_prev = torch.full((total,), -1, dtype=torch.int64, device=dev)
+    d_prev[n:] = columns[col["to_act"]][columns[col["parent"]][n:]]
+    d_pot = tree.device_arrays["stacks"] + columns[col["pot"]][:, None] - tree.device_arrays["starting_stacks"]
+    tree.device_arrays.update({
+        "new_street_mask": d_new_street, "leaf_mask": d_leaf, "prev_actor": d_prev,
+        "fold_mask": (columns[col["action"]] == 0) & d_done, "showdown_mask": columns[col["street"]] == 4,
+        "showdown_potential": d_pot,
     })
     return tree
