@@ -157,6 +157,8 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
     b, k = hand_values.shape[0], hand_values.shape[1]
     assert weight.shape == (k,)
     hv = hand_values.contiguous().float()
+    if int(perms.min()) < 0 or int(perms.max()) >= NUM_HANDS:
+        raise IndexError("perms must map hands to hand indices 0..1325")
     pt = perms.to(device=dev, dtype=torch.int16).contiguous()
     w = weight.to(device=dev, dtype=torch.float32).contiguous()
     accumulate = out is not None

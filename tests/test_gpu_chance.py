@@ -124,6 +124,8 @@ def test_helper_edge_cases(K):
     assert out.shape == (0, 2, H)
     with pytest.raises(IndexError):                          # a state index beyond the ranges is refused on the host
         K.flop_expand(torch.rand(2, 2, H, device=dev), torch.tensor([2], device=dev), torch.tensor([[0, 1, 2]], device=dev))
+    with pytest.raises(IndexError):                          # so is a permutation that points outside the hands
+        K.perm_mean(torch.rand(1, 1, 2, H, device=dev), torch.full((1, H), H, device=dev), torch.ones(1, device=dev))
     # the fixed-count fast path gives the same samples
     rng = np.random.default_rng(9)
     boards, pre = inputs(rng, 3, [4])
