@@ -103,6 +103,14 @@ int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int
 int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
                     const float* weight, int accumulate, float* out, float* workspace, int shares, void* stream);
 
+/* p2hip_perm_mean for the case of ALL 24 suit permutations (the rows of combo_suit_permutation_tensor,
+ * env/card_utils.py:161-181): the mean over the orbit of a hand is the mean over its class of
+ * starting hands (13 pairs, 78 suited, 78 offsuit), so
+ * out[i][p][h] (+)= sum_f weight[f] * mean over the class of h of hand_values[i][f][p][.].
+ * Same arguments otherwise; the class tables are built into the library. */
+int p2hip_orbit_mean(const float* hand_values, int64_t n, int64_t n_flops, const float* weight, int accumulate,
+                     float* out, float* workspace, int shares, void* stream);
+
 /* ---- either side of the search in data generation ------------------------------------------ */
 
 /* Context features and board of RebelFeatureEncoder.encode (models/mlp/rebel_feature_encoder.py:55-127)

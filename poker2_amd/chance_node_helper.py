@@ -174,6 +174,30 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
     return out
 
 
+def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``perm_mean`` over ALL 24 suit permutations: the orbit of a hand is its class of starting
+    hands (pair / suited / offsuit of the same ranks), so the mean is taken per class."""
+    if not _lib.hip_is_available():
+        raise RuntimeError("orbit_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
+    _lib.require_gpu(hand_values, "orbit_mean")
+    dev = hand_values.device
+    assert hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)
+    b, k = hand_values.shape[0], hand_values.shape[1]
+    assert weight.shape == (k,)
+    hv = hand_values.contiguous().float()
+    w = weight.to(device=dev, dtype=torch.float32).contiguous()
+    accumulate = out is not None
+    if out is None:
+        out = torch.empty(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
+    else:
+        assert out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()
+    shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
+    workspace = torch.empty(shares, b, 2, NUM_HANDS, dtype=torch.float32, device=dev) if shares > 1 else None
+    _lib.call("p2hip_orbit_mean", _lib.ptr(hv), b, k, _lib.ptr(w), int(accumulate), _lib.ptr(out),
+              _lib.ptr(workspace), shares, _lib.stream_ptr())
+    return out
+
+
 def canonical_flops():
     """The suit-canonical flops (src/p2/search/chance_node_helper.py:76-216), on the host.
 
@@ -286,9 +310,9 @@ class ChanceNodeHelper:
             p = self.NUM_PERM_SAMPLES
             if 0 < p < self.num_permutations:
                 perm_idx = torch.randperm(self.num_permutations, device=gdev, generator=self.generator)[:p].to(dev)
+                perm_mean(hv, self._combo_perm_i16[perm_idx], weight, out=out)
             else:
-                perm_idx = torch.arange(self.num_permutations, device=dev)
-            perm_mean(hv, self._combo_perm_i16[perm_idx], weight, out=out)
+                orbit_mean(hv, weight, out=out)       # all 24 permutations: the mean over each hand's class
 
         s = self.FLOP_SAMPLE_SIZE
         if 0 < s < num_flops:

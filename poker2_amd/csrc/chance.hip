@@ -355,6 +355,95 @@ __global__ __launch_bounds__(CH_BLOCK) void perm_reduce_kernel(const float2* __r
   out[e] = s;
 }
 
+// ---- mean over the whole suit orbit ------------------------------------------------------------
+// With all 24 suit permutations the mean of hv[perm_q[h]] over q is the mean of hv over the orbit of
+// h (every orbit member is hit 24 / |orbit| times), and the orbits are the 169 classes of starting
+// hands: 13 pairs (6 hands each), 78 suited (4), 78 offsuit (12).  So one accumulator per class
+// replaces 24 look-ups per hand and flop.
+constexpr int ORB_CLASSES = 169;
+constexpr int ORB_MAX = 12;
+struct P2OrbitTable {
+  int16_t member[ORB_CLASSES][ORB_MAX];   // hands of the class, ascending; -1 past its size
+  uint8_t size[ORB_CLASSES];
+  uint8_t cls[P2_H];                       // class of every hand
+  constexpr P2OrbitTable() : member(), size(), cls() {
+    for (int c = 0; c < ORB_CLASSES; ++c) {
+      size[c] = 0;
+      for (int j = 0; j < ORB_MAX; ++j) member[c][j] = -1;
+    }
+    int h = 0;
+    for (int a = 0; a < P2_CARDS; ++a) {
+      for (int b = a + 1; b < P2_CARDS; ++b, ++h) {
+        const int ra = a % 13, rb = b % 13, sa = a / 13, sb = b / 13;
+        const int lo = ra < rb ? ra : rb, hi = ra < rb ? rb : ra;
+        const int pair_index = lo * (25 - lo) / 2 + (hi - lo - 1);   // 0..77 over rank pairs lo < hi
+        const int c = ra == rb ? ra : (sa == sb ? 13 + pair_index : 91 + pair_index);
+        cls[h] = (uint8_t)c;
+        member[c][size[c]] = (int16_t)h;
+        size[c] = (uint8_t)(size[c] + 1);
+      }
+    }
+  }
+};
+__device__ const P2OrbitTable p2_orbit = P2OrbitTable();
+
+// dst[i][p][h] (+)= sum_f weight[f] * (mean of hand_values[i][f][p] over the orbit class of h).
+// Workgroup layout and the share / workspace scheme are those of perm_mean_kernel.
+__global__ __launch_bounds__(CH_BLOCK) void orbit_mean_kernel(const float* __restrict__ hand_values,
+                                                               const float* __restrict__ weight, int64_t n_flops,
+                                                               int64_t flops_per_share, int accumulate,
+                                                               float* __restrict__ dst, int64_t dst_share_stride) {
+  __shared__ __align__(8) float rows[2][P2_H + 2];
+  __shared__ float class_acc[ORB_CLASSES];
+  const int64_t i = blockIdx.x >> 1;
+  const int p = blockIdx.x & 1;
+  const int64_t f0 = (int64_t)blockIdx.y * flops_per_share;
+  const int64_t f1 = f0 + flops_per_share < n_flops ? f0 + flops_per_share : n_flops;
+  const int c = threadIdx.x;                 // lanes 0..168 own one class each
+  int mem[ORB_MAX];
+  float inv_size = 0.f;
+#pragma unroll
+  for (int j = 0; j < ORB_MAX; ++j) mem[j] = c < ORB_CLASSES ? (int)p2_orbit.member[c][j] : -1;
+  if (c < ORB_CLASSES) inv_size = 1.0f / (float)p2_orbit.size[c];
+  double acc = 0.0;
+  float2 next[CH_PPT];
+  auto fetch = [&](int64_t f) {
+    const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      next[k] = idx < P2_HPAIRS ? src[idx] : make_float2(0.f, 0.f);
+    }
+  };
+  if (f0 < f1) fetch(f0);
+  int buf = 0;
+  for (int64_t f = f0; f < f1; ++f, buf ^= 1) {
+    float* row = rows[buf];
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx < P2_HPAIRS) reinterpret_cast<float2*>(row)[idx] = next[k];
+    }
+    if (f + 1 < f1) fetch(f + 1);
+    p2_sync_lds();   // row f is complete; the other buffer was consumed before this barrier
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < ORB_MAX; ++j)
+      if (mem[j] >= 0) s += row[mem[j]];
+    acc += (double)(weight[f] * (s * inv_size));
+  }
+  if (c < ORB_CLASSES) class_acc[c] = (float)acc;
+  p2_sync_lds();
+  float2* o = p2_row2(dst + (int64_t)blockIdx.y * dst_share_stride, i * 2 + p);
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    if (idx >= P2_HPAIRS) continue;
+    const float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
+    o[idx] = make_float2(prev.x + class_acc[p2_orbit.cls[2 * idx]], prev.y + class_acc[p2_orbit.cls[2 * idx + 1]]);
+  }
+}
+
 }  // namespace p2
 
 extern "C" {
@@ -427,6 +516,31 @@ int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const 
   hipLaunchKernelGGL(p2::perm_mean_kernel, dim3((unsigned)(2 * n), (unsigned)shares), dim3(p2::CH_BLOCK), lds,
                      (hipStream_t)stream, hand_values, perms, n_perms, weight, n_flops, per_share, 0, workspace,
                      npairs * 2);
+  P2_LAUNCH_CHECK();
+  const int64_t grid = (npairs + p2::CH_BLOCK - 1) / p2::CH_BLOCK;
+  hipLaunchKernelGGL(p2::perm_reduce_kernel, dim3((unsigned)grid), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     (const float2*)workspace, shares, npairs, accumulate, (float2*)out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_orbit_mean(const float* hand_values, int64_t n, int64_t n_flops, const float* weight, int accumulate,
+                     float* out, float* workspace, int shares, void* stream) {
+  if (n < 0 || n_flops < 0 || shares < 1) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!hand_values || !weight || !out || !p2_aligned8(hand_values) || !p2_aligned8(out)) return P2_EINVAL;
+  if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
+  if (shares > 1 && (!workspace || !p2_aligned8(workspace))) return P2_EINVAL;
+  const int64_t per_share = (n_flops + shares - 1) / shares;
+  const int64_t npairs = n * 2 * P2_HPAIRS;
+  if (shares == 1) {
+    hipLaunchKernelGGL(p2::orbit_mean_kernel, dim3((unsigned)(2 * n), 1), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                       hand_values, weight, n_flops, per_share, accumulate, out, (int64_t)0);
+    P2_LAUNCH_CHECK();
+    return 0;
+  }
+  hipLaunchKernelGGL(p2::orbit_mean_kernel, dim3((unsigned)(2 * n), (unsigned)shares), dim3(p2::CH_BLOCK), 0,
+                     (hipStream_t)stream, hand_values, weight, n_flops, per_share, 0, workspace, npairs * 2);
   P2_LAUNCH_CHECK();
   const int64_t grid = (npairs + p2::CH_BLOCK - 1) / p2::CH_BLOCK;
   hipLaunchKernelGGL(p2::perm_reduce_kernel, dim3((unsigned)grid), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,

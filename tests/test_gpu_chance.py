@@ -409,3 +409,26 @@ def test_preflop_subgame_with_flop_leaves_matches_oracle(K):
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
         compare(ev, orc, rtol=1e-3, atol=3e-4)      # network through hipBLASLt vs numpy: GEMM summation order
+
+
+def test_orbit_mean_equals_the_mean_over_all_24_permutations(K):
+    """The class-mean shortcut against the literal mean over the 24 permuted copies (numpy, fp64)
+    and against the generic kernel fed with the full permutation table."""
+    rng = np.random.default_rng(71)
+    perms = OCH.combo_suit_perms()
+    classes = {tuple(sorted(set(perms[:, h].tolist()))) for h in range(H)}
+    assert len(classes) == 169 and sorted({len(c) for c in classes}) == [4, 6, 12]   # suited, pairs, offsuit
+    for b, k in ((3, 11), (1100, 2)):            # flops shared out over workgroups / one workgroup per (state, player)
+        hv = rng.standard_normal((b, k, 2, H)).astype(np.float32)
+        w = rng.random(k).astype(np.float32)
+        exp = np.zeros((b, 2, H))
+        for f in range(k):
+            exp += w[f] * np.mean([hv[:, f][..., q] for q in perms], axis=0, dtype=np.float64)
+        t_hv, t_w = torch.from_numpy(hv).cuda(), torch.from_numpy(w).cuda()
+        got = K.orbit_mean(t_hv, t_w)
+        np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=2e-6)
+        generic = K.perm_mean(t_hv, torch.from_numpy(perms).cuda(), t_w)
+        np.testing.assert_allclose(got.cpu().numpy(), generic.cpu().numpy(), rtol=1e-5, atol=2e-6)
+        base = torch.from_numpy(rng.standard_normal((b, 2, H)).astype(np.float32)).cuda()
+        again = K.orbit_mean(t_hv, t_w, out=base.clone())
+        np.testing.assert_allclose(again.cpu().numpy(), base.cpu().numpy() + exp, rtol=1e-5, atol=4e-6)
