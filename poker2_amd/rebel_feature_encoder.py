@@ -50,11 +50,14 @@ class RebelFeatureEncoder:
             raise RuntimeError("RebelFeatureEncoder.encode needs libp2hip.so and a GPU (no CPU fallback exists).")
         _lib.require_gpu(beliefs, "RebelFeatureEncoder.encode")
 
+        widths = {"starting_stacks": 2, "committed": 2, "last_board_indices": 5, "board_indices": 5}
+
         def get(name: str) -> torch.Tensor:
             val = getattr(self.env, name)
             val = val[indices] if indices is not None else val
-            if val.shape[0] != m:
-                raise ValueError(f"env.{name} has {val.shape[0]} rows, beliefs {m}")
+            want = (m, widths[name]) if name in widths else (m,)
+            if tuple(val.shape) != want:
+                raise ValueError(f"env.{name} has shape {tuple(val.shape)}, expected {want}")
             return val.to(device=dev, dtype=torch.int64).contiguous()
 
         pre_ptr, pre_all, pre_keep = None, 0, None
