@@ -140,8 +140,19 @@ def cases(repeats: int):
     hv = CH.flop_expand(pre_f, roots_f, flops)
     perms = combo_suit_permutation_tensor(dev)[:6].to(torch.int16).contiguous()
     w = torch.full((kf,), 1.0 / kf, device=dev)
-    yield (f"perm_mean states={ks} x{kf} perms=6", ks * (2 * kf + 2) * H * 4, lambda: CH.perm_mean(hv, perms, w))
+    yield (f"perm_mean states={ks} x{kf} perms=6", ks * (2 * kf + 2) * H * 4, lambda: CH.perm_mean(hv, perms, w, check_perms=False))
+    yield (f"orbit_mean states={ks} x{kf} (all 24)", ks * (2 * kf + 2) * H * 4, lambda: CH.orbit_mean(hv, w))
     del hv
+    # the same at 1024 states (2.9 GB of network answers)
+    ks = 1024
+    pre_f = (torch.rand(ks, 2, H, device=dev) + 1e-3)
+    pre_f = pre_f / pre_f.sum(-1, keepdim=True)
+    roots_f = torch.arange(ks, device=dev)
+    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops))
+    hv = CH.flop_expand(pre_f, roots_f, flops)
+    yield (f"perm_mean states={ks} x{kf} perms=6", ks * (2 * kf + 2) * H * 4, lambda: CH.perm_mean(hv, perms, w, check_perms=False))
+    yield (f"orbit_mean states={ks} x{kf} (all 24)", ks * (2 * kf + 2) * H * 4, lambda: CH.orbit_mean(hv, w))
+    del hv, pre_f
 
     # --- data generation: policy targets and features of a 4096-root river search (21 nodes per root)
     from .config import river_dcfr_config

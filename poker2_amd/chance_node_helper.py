@@ -145,7 +145,7 @@ PERM_MEAN_TARGET_WORKGROUPS = 2048   # 256 CUs x 8
 
 
 def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tensor,
-              out: torch.Tensor | None = None) -> torch.Tensor:
+              out: torch.Tensor | None = None, check_perms: bool = True) -> torch.Tensor:
     """hand_values [B,K,2,1326] fp32, perms [P,1326] hand-index maps (P <= 24), weight [K] ->
     [B,2,1326]: sum_k weight[k] * mean_q hand_values[b,k,p,perms[q,h]]; added to ``out`` if given."""
     if not _lib.hip_is_available():
@@ -157,7 +157,7 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
     b, k = hand_values.shape[0], hand_values.shape[1]
     assert weight.shape == (k,)
     hv = hand_values.contiguous().float()
-    if int(perms.min()) < 0 or int(perms.max()) >= NUM_HANDS:
+    if check_perms and (int(perms.min()) < 0 or int(perms.max()) >= NUM_HANDS):   # two device reads: skip for known tables
         raise IndexError("perms must map hands to hand indices 0..1325")
     pt = perms.to(device=dev, dtype=torch.int16).contiguous()
     w = weight.to(device=dev, dtype=torch.float32).contiguous()
@@ -310,7 +310,7 @@ class ChanceNodeHelper:
             p = self.NUM_PERM_SAMPLES
             if 0 < p < self.num_permutations:
                 perm_idx = torch.randperm(self.num_permutations, device=gdev, generator=self.generator)[:p].to(dev)
-                perm_mean(hv, self._combo_perm_i16[perm_idx], weight, out=out)
+                perm_mean(hv, self._combo_perm_i16[perm_idx], weight, out=out, check_perms=False)
             else:
                 orbit_mean(hv, weight, out=out)       # all 24 permutations: the mean over each hand's class
 
