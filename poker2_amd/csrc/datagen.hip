@@ -65,33 +65,42 @@ __global__ __launch_bounds__(DG_BLOCK) void bet_amounts_kernel(const int64_t* __
 }
 
 // out[k, h, a] = policy_avg[c, h] for the child c of node rows[k] reached by action a, 0 where the
-// action has no child.  One workgroup per node: the children's rows are read whole (coalesced),
-// transposed through LDS and written as one contiguous [H * A] run.
+// action has no child.  One workgroup per node: the children's rows are read whole (coalesced
+// float2), transposed through LDS and written as one contiguous [H * A] run of float2.  A is a
+// template parameter so that the (hand, action) split of an output index is a multiplication.
+template <int A>
 __global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* __restrict__ policy_avg,
                                                                    const int64_t* __restrict__ rows,
                                                                    const int64_t* __restrict__ child_offsets,
                                                                    const int64_t* __restrict__ child_count,
                                                                    const int64_t* __restrict__ action_from_parent,
-                                                                   int num_actions, float* __restrict__ out) {
-  extern __shared__ __align__(8) float tile[];   // [num_actions][H + 1]
+                                                                   float* __restrict__ out) {
+  constexpr int STRIDE = P2_H + 2;                 // floats between action rows in LDS (keeps float2 alignment)
+  __shared__ __align__(8) float tile[A][STRIDE];
   const int64_t k = blockIdx.x;
   const int64_t r = rows[k];
-  const int stride = P2_H + 1;
-  for (int e = threadIdx.x; e < num_actions * stride; e += DG_BLOCK) tile[e] = 0.f;
-  p2_sync_lds();
   const int64_t first = child_offsets[r];
   const int n_children = (int)child_count[r];
+  uint32_t present = 0;
   for (int j = 0; j < n_children; ++j) {
     const int a = (int)action_from_parent[first + j];
-    if (a < 0 || a >= num_actions) continue;
-    const float* src = policy_avg + (first + j) * P2_H;
-    for (int h = threadIdx.x; h < P2_H; h += DG_BLOCK) tile[a * stride + h] = src[h];
+    if (a < 0 || a >= A) continue;
+    present |= 1u << a;
+    const float2* src = p2_row2(policy_avg, first + j);
+    for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += DG_BLOCK) reinterpret_cast<float2*>(tile[a])[idx] = src[idx];
   }
+#pragma unroll
+  for (int a = 0; a < A; ++a)
+    if (!((present >> a) & 1u))
+      for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += DG_BLOCK)
+        reinterpret_cast<float2*>(tile[a])[idx] = make_float2(0.f, 0.f);
   p2_sync_lds();
-  float* dst = out + k * (int64_t)P2_H * num_actions;
-  for (int e = threadIdx.x; e < P2_H * num_actions; e += DG_BLOCK) {
-    const int h = e / num_actions, a = e - h * num_actions;
-    dst[e] = tile[a * stride + h];
+  float2* dst = reinterpret_cast<float2*>(out + k * (int64_t)P2_H * A);   // 8-byte aligned: H * A * 4 is a multiple of 8
+  for (int e2 = threadIdx.x; e2 < P2_H * A / 2; e2 += DG_BLOCK) {
+    const int e = 2 * e2;
+    const int h0 = e / A, a0 = e - h0 * A;
+    const int h1 = (e + 1) / A, a1 = (e + 1) - h1 * A;
+    dst[e2] = make_float2(tile[a0][h0], tile[a1][h1]);
   }
 }
 
@@ -141,9 +150,18 @@ int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n
   if (n_rows == 0) return 0;
   if (!policy_avg || !rows || !child_offsets || !child_count || !action_from_parent || !out) return P2_EINVAL;
   if (n_rows > 0x7FFFFFFF) return P2_EINVAL;
-  const size_t lds = (size_t)num_actions * (P2_H + 1) * sizeof(float);   // at most 42.5 KB
-  hipLaunchKernelGGL(p2::policy_targets_kernel, dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), lds, (hipStream_t)stream,
-                     policy_avg, rows, child_offsets, child_count, action_from_parent, num_actions, out);
+  if ((reinterpret_cast<uintptr_t>(policy_avg) & 7u) || (reinterpret_cast<uintptr_t>(out) & 7u)) return P2_EINVAL;
+#define P2_PT_CASE(A)                                                                                          \
+  case A:                                                                                                      \
+    hipLaunchKernelGGL(p2::policy_targets_kernel<A>, dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), 0,            \
+                       (hipStream_t)stream, policy_avg, rows, child_offsets, child_count, action_from_parent,  \
+                       out);                                                                                   \
+    break;
+  switch (num_actions) {
+    P2_PT_CASE(1) P2_PT_CASE(2) P2_PT_CASE(3) P2_PT_CASE(4) P2_PT_CASE(5) P2_PT_CASE(6) P2_PT_CASE(7) P2_PT_CASE(8)
+    default: return P2_EINVAL;
+  }
+#undef P2_PT_CASE
   P2_LAUNCH_CHECK();
   return 0;
 }
