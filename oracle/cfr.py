@@ -35,8 +35,11 @@ tests/test_oracle_cfr_golden.py holds this restatement to them (1e-5 relative on
 iterations).  Further pinned by (tests/test_oracle_cfr.py) an explicit hand-pair game that
 reproduces reach, conditional values and regrets at depths 2-4, the closed form of the average
 policy, a textbook CFR / best response, and structural identities.  The ``fused_variant``
-switches (what FusedSparseCFREvaluator does differently on rows / hands without probability
-mass) are read off the source and agree with the base variant wherever mass lives.
+switches (what FusedSparseCFREvaluator does differently: root rows of self_reach keep 1.0 on
+board-blocked hands, root beliefs are not re-normalised, average values use (a*old + v*new) *
+(1/(old+new)), linear CFR accumulates without the CFR+ clamp) are PARITY UNPINNED: they are read
+off the source — its Triton kernels cannot run in the CPU-only build container — and checked only
+to agree with the pinned base variant wherever probability mass lives.
 """
 from __future__ import annotations
 
