@@ -29,17 +29,23 @@ with Python-scalar operands rounded to float32 first, as torch does.
 PINNED by vectors written from the reference itself: tests/golden/cfr_golden.npz holds the
 11 state tensors of the reference's own SparseCFREvaluator (run on the CPU of the build
 container by tests/golden/gen_cfr_golden.py) after the preparation step and after iterations
-of six searches — discounted, discounted_plus with delay, linear + CFR+ + cfr_avg, standard,
-warm start ``model_br`` and ``model``; depths 2 and 3 — and its local exploitability;
+of eight searches — discounted, discounted_plus with delay, linear + cfr_avg with and without
+CFR+, standard, warm start ``model_br`` and ``model`` (twice); depths 2 and 3 — and its local exploitability;
 tests/test_oracle_cfr_golden.py holds this restatement to them (1e-5 relative on the first
 iterations).  Further pinned by (tests/test_oracle_cfr.py) an explicit hand-pair game that
 reproduces reach, conditional values and regrets at depths 2-4, the closed form of the average
-policy, a textbook CFR / best response, and structural identities.  The ``fused_variant``
-switches (what FusedSparseCFREvaluator does differently: root rows of self_reach keep 1.0 on
-board-blocked hands, root beliefs are not re-normalised, average values use (a*old + v*new) *
-(1/(old+new)), linear CFR accumulates without the CFR+ clamp) are PARITY UNPINNED: they are read
-off the source — its Triton kernels cannot run in the CPU-only build container — and checked only
-to agree with the pinned base variant wherever probability mass lives.
+policy, a textbook CFR / best response, and structural identities.
+
+The ``fused_variant`` switches (what FusedSparseCFREvaluator does differently: root rows of
+self_reach keep 1.0 on board-blocked hands, root beliefs are not re-normalised, average values
+use (a*old + v*new) * (1/(old+new)), linear CFR accumulates without the CFR+ clamp) are PINNED by
+tests/golden/fused_cfr_golden.npz: the same eight searches run through the reference's own
+FusedSparseCFREvaluator, its Triton kernels executing under Triton's CPU interpreter
+(``gen_cfr_golden.py --fused``); with ``fused_variant=True`` this restatement is held to those
+vectors on every entry, board-blocked hands included (tests/test_oracle_cfr_golden.py).  One of the
+eight (model warm start with a discount delay shorter than the warm start) leaves NaN in the
+reference's average policy — its device scalars are still zero at that point — so the four
+tensors derived from it are compared with the base class's vectors only.
 """
 from __future__ import annotations
 

@@ -19,7 +19,10 @@ in the arithmetic order of that kernel:
   reach_weights_depth        <- _fused_reach_weights_kernel           :1900-1941
   deep_beliefs               <- _fused_deep_beliefs_kernel            :1996-2036
 
-Pinned by: the same identities the reference's own tests assert in
+Pinned by tests/golden/fused_ops_golden.npz: outputs of the reference's own Triton kernels,
+run on seeded inputs under Triton's CPU interpreter by tests/golden/gen_fused_ops_golden.py
+(every function above, through the reference's public wrappers; tests/test_oracle_fused_ops.py
+holds these restatements to them at 1e-5 relative).  Also by: the same identities the reference's own tests assert in
 ``tests/test_fused_cfr_triton.py`` (each of those tests spells the op out with
 plain torch ops; the spellings agree with these), and by ``oracle/cfr.py``,
 whose whole-iteration results are built from the un-fused forms of the same

@@ -32,6 +32,12 @@ rank-order lists of the reference's ``tests/test_rules.py`` (restated as data in
 ``tests/golden/rules_pairs.json``); (3) the exhaustive C(52,7) category
 histogram equalling the textbook table; (4) agreement with an independent
 best-5-of-7 evaluator (``oracle/std_eval.c``) outside the quirk classes.
+
+PARITY UNPINNED: what ``rank_cards`` returns for a hand that repeats a card id.  That rule is read
+off ``_evaluate_cards_player``; the kernels of ``rules_triton.py`` hold PTX inline assembly
+(:364-385), so they run neither under Triton's CPU interpreter nor on this hardware, and
+``rules.py`` takes card planes, which cannot express a repeated card.  No caller on the search
+path passes one (boards and hole cards are distinct).
 """
 from __future__ import annotations
 

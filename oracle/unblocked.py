@@ -15,7 +15,10 @@
 Pinned by the reference's known answers (tests/test_card_utils.py:472-614:
 uniform -> 1225/1326 = 0.9238311052322388, delta -> 0 on itself and its
 blockers and 1 elsewhere, two half deltas -> 0.5 ...), by the identity of the
-two formulations, and by an explicit double loop on a few rows.
+two formulations, by an explicit double loop on a few rows, and by outputs of the
+reference's own unblocked-mass kernels (plain, opponent-at-parents, ratio direct
+and indirect) run under Triton's CPU interpreter (tests/golden/fused_ops_golden.npz,
+tests/test_oracle_fused_ops.py).
 """
 from __future__ import annotations
 

@@ -18,6 +18,24 @@ inputs (boards, ranges, chips, settings), the tree arrays, and after the prepara
 the first two iterations, the sampling iteration and the last one, the 11 state tensors
 restricted to 64 seeded hand columns plus their full row sums (float64).  Two cases start from
 the reference's warm start (``model_br`` and ``model``).
+
+With ``--fused`` the same searches run through the reference's ``FusedSparseCFREvaluator`` (the
+class the search path uses on a GPU) and go to ``fused_cfr_golden.npz``:
+
+    python -O tests/golden/gen_cfr_golden.py --fused
+
+Its Triton kernels execute on CPU tensors under Triton's interpreter (TRITON_INTERPRET=1).  The
+evaluator is built as a ``SparseCFREvaluator`` and its ``__class__`` is then set to the fused
+class and ``_ensure_fused_attrs()`` called, which is how the reference's own tests construct it
+(tests/test_fused_cfr_triton.py:600, 646-647); the hand ranker therefore stays ``rules.py``.
+``-O`` is needed because one wrapper guards its launch with ``assert target.is_cuda``
+(fused_cfr_triton.py:307).
+
+In the fused fixture the case ``warm_model_d2`` holds NaN in ``policy_probs_avg`` and what derives
+from it: the fused class mixes the average policy with the device scalars of ``TScalars``, which are
+still all zero when ``warm_start`` calls ``update_policy`` before the first ``cfr_iteration``
+(fused_sparse_cfr_evaluator.py:368-378, fused_cfr_triton.py:2109-2128), unless the discount delay
+sends that call down the copy branch (:356-361) as the reference's own settings do.
 """
 from __future__ import annotations
 
@@ -42,6 +60,9 @@ CASES = [
     ("standard_d2", "standard", False, False, 0, 2, 4, [(450, 300, 300, 1)], (0, "model_br", 1.0)),
     ("warm_br_d2", "discounted_plus", False, False, 4, 2, 7, [(200, 800, 800, 1)], (3, "model_br", 1.0)),
     ("warm_model_d2", "discounted", False, False, 0, 2, 6, [(260, 700, 900, 0)], (3, "model", 10.0)),
+    # the shape of the reference's own search settings (conf/config_rebel_cfr.yaml:77-86): model warm start under
+    # discounted_plus with a delay that outlasts the warm start iterations
+    ("warm_model_dplus_d2", "discounted_plus", False, False, 5, 2, 8, [(240, 900, 650, 1)], (3, "model", 10.0)),
 ]
 
 
@@ -74,8 +95,12 @@ def install_stand_ins() -> None:
     sys.modules.update({"hydra": hydra, "hydra.core": core, "hydra.core.config_store": store, "omegaconf": omega})
 
 
-def main() -> None:
+def main(fused: bool = False) -> None:
     os.environ.setdefault("TORCHDYNAMO_DISABLE", "1")
+    if fused:
+        if __debug__:
+            raise SystemExit("run as: python -O tests/golden/gen_cfr_golden.py --fused")
+        os.environ["TRITON_INTERPRET"] = "1"          # before triton is imported
     install_stand_ins()
     sys.path.insert(0, REF_SRC)
     import torch
@@ -85,6 +110,8 @@ def main() -> None:
     from p2.env.hunl_tensor_env import HUNLTensorEnv
     from p2.models.model_output import ModelOutput
     from p2.search.sparse_cfr_evaluator import SparseCFREvaluator
+    if fused:
+        from p2.search.fused_sparse_cfr_evaluator import FusedSparseCFREvaluator
 
     class MockModel:
         def __init__(self, num_actions):
@@ -144,6 +171,9 @@ def main() -> None:
         cfg.search.cfr_plus = cfr_plus
         cfg.search.cfr_avg = cfr_avg
         ev = SparseCFREvaluator(model=MockModel(len(bins) + 3), device=dev, cfg=cfg)
+        if fused:
+            ev.__class__ = FusedSparseCFREvaluator
+            ev._ensure_fused_attrs()                                  # as tests/test_fused_cfr_triton.py:646-647 does
 
         board = env.board_indices.clone().numpy()
         bel = rng.gamma(0.5, size=(n, 2, NUM_HANDS)).astype(np.float32)
@@ -185,10 +215,10 @@ def main() -> None:
         out[f"{name}/settings"] = np.array([cfr_type, str(cfr_plus), str(cfr_avg), str(delay), str(depth), str(iters),
                                             str(warm), warm_type, str(warm_mult)])
         print(name, "nodes", ev.total_nodes, "depth offsets", ev.depth_offsets, flush=True)
-    path = os.path.join(HERE, "cfr_golden.npz")
+    path = os.path.join(HERE, "fused_cfr_golden.npz" if fused else "cfr_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path) // 1024, "KiB")
 
 
 if __name__ == "__main__":
-    main()
+    main(fused="--fused" in sys.argv[1:])

@@ -1,8 +1,12 @@
 """CPU: the oracle's whole CFR iteration against vectors written by RUNNING the reference's own
-SparseCFREvaluator in the build container (tests/golden/gen_cfr_golden.py).  Seven searches
-(discounted, discounted_plus with delay, linear + cfr_avg with and without CFR+, standard, and two that start
+SparseCFREvaluator in the build container (tests/golden/gen_cfr_golden.py).  Eight searches
+(discounted, discounted_plus with delay, linear + cfr_avg with and without CFR+, standard, and three that start
 from the reference's warm start; depths 2 and 3): the preparation step, the first iterations,
-the sampling iteration and the last one, all 11 state tensors."""
+the sampling iteration and the last one, all 11 state tensors.
+
+The same seven searches run through the reference's FusedSparseCFREvaluator (its Triton kernels
+under Triton's CPU interpreter, ``gen_cfr_golden.py --fused``) are in fused_cfr_golden.npz; the
+oracle's ``fused_variant=True`` is held to those on every entry, board-blocked hands included."""
 import numpy as np
 import pytest
 
@@ -12,9 +16,10 @@ from oracle import tree as OT
 STATE = OCFR.OracleCFR.STATE_NAMES
 
 
-@pytest.fixture(scope="module")
-def golden(golden_dir):
-    return np.load(str(golden_dir) + "/cfr_golden.npz")
+@pytest.fixture(scope="module", params=["base", "fused"])
+def golden(golden_dir, request):
+    g = np.load(str(golden_dir) + ("/fused_cfr_golden.npz" if request.param == "fused" else "/cfr_golden.npz"))
+    return {**{k: g[k] for k in g.files}, "fused_variant": request.param == "fused"}
 
 
 def build(golden, name):
@@ -33,8 +38,14 @@ def build(golden, name):
                        cfr_plus=cfr_plus == "True", cfr_avg=cfr_avg == "True", dcfr_delay=int(delay),
                        dcfr_alpha=1.5, dcfr_beta=0.0, dcfr_gamma=2.0, cfr_iterations=50, enforce_zero_sum=True,
                        t_sample_roots=t_sample, warm_start_iterations=int(warm), warm_start_type=str(warm_type),
-                       warm_start_multiplier=float(warm_mult))
+                       warm_start_multiplier=float(warm_mult), fused_variant=golden["fused_variant"])
     return o, int(warm), int(iters)
+
+
+# In the fused fixture this case holds NaN in the average policy and what is computed from it: the
+# reference's fused class mixes with device scalars that are still zero when its warm start runs
+# (tests/golden/gen_cfr_golden.py explains).  Those tensors are left out there; the rest is compared.
+NAN_IN_FUSED_REFERENCE = {"warm_model_d2": ("policy_probs_avg", "self_reach_avg", "beliefs_avg", "values_avg")}
 
 
 def check(o, golden, name, tag, rtol, atol):
@@ -42,6 +53,11 @@ def check(o, golden, name, tag, rtol, atol):
     for s in STATE:
         got = getattr(o, s)
         exp = golden[f"{name}/{tag}/{s}"]
+        if golden["fused_variant"] and s in NAN_IN_FUSED_REFERENCE.get(name, ()):
+            if s == "policy_probs_avg":
+                assert np.isnan(exp).any(), "the fixture no longer shows the reference's NaN: compare this case too"
+            continue
+        assert not np.isnan(exp).any(), (name, tag, s)
         err = np.abs(got[..., cols] - exp) - (atol + rtol * np.abs(exp))
         # hands whose regret sums are tiny amplify rounding (and some sit on the algorithm's hard
         # thresholds): up to 0.2 % of the entries may miss the tolerance, none by more than 1e-3
@@ -53,7 +69,7 @@ def check(o, golden, name, tag, rtol, atol):
 
 
 @pytest.mark.parametrize("name", ["discounted_d2", "dplus_d3", "linear_avg_d2", "linear_noplus_d2", "standard_d2",
-                                  "warm_br_d2", "warm_model_d2"])
+                                  "warm_br_d2", "warm_model_d2", "warm_model_dplus_d2"])
 def test_oracle_iterations_match_reference_vectors(golden, name):
     o, warm, iters = build(golden, name)
     o.prepare()                                   # includes the warm start of the last two cases
@@ -71,6 +87,9 @@ def test_oracle_iterations_match_reference_vectors(golden, name):
             check(o, golden, name, f"t{t}", rtol=tol, atol=tol / 2)
     # the reference's own local exploitability of the final average strategy (:718-764)
     from oracle import best_response as OBR
+    if np.isnan(golden[f"{name}/local_exploitability"]).any():
+        assert golden["fused_variant"] and name in NAN_IN_FUSED_REFERENCE
+        return
     expl, br = OBR.compute_exploitability(o)
     np.testing.assert_allclose(expl, golden[f"{name}/local_exploitability"], rtol=1e-3, atol=2e-5)
     np.testing.assert_allclose(br, golden[f"{name}/local_best_response_values"], rtol=1e-3, atol=2e-5)
