@@ -13,6 +13,11 @@ encoded features (written out in ``ValueNet`` below; tests restate it), so the s
 encoder and the chance nodes all feed the stored targets.  The flop chance node runs in its
 exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
 A last section holds what the env's ``reset`` deals from a seeded CPU generator.
+
+With ``--fused`` the same searches run through the reference's ``FusedSparseCFREvaluator``, its
+Triton kernels executing under Triton's CPU interpreter, and go to
+``fused_training_data_golden.npz`` (how, and why ``-O``: see gen_cfr_golden.py):
+    python -O tests/golden/gen_training_data_golden.py --fused
 """
 from __future__ import annotations
 
@@ -37,8 +42,12 @@ CASES = [
 ]
 
 
-def main() -> None:
+def main(fused: bool = False) -> None:
     os.environ.setdefault("TORCHDYNAMO_DISABLE", "1")
+    if fused:
+        if __debug__:
+            raise SystemExit("run as: python -O tests/golden/gen_training_data_golden.py --fused")
+        os.environ["TRITON_INTERPRET"] = "1"          # before triton is imported
     install_stand_ins()
     sys.path.insert(0, REF_SRC)
     import warnings
@@ -49,6 +58,8 @@ def main() -> None:
     from p2.models.model_output import ModelOutput
     from p2.models.mlp.rebel_feature_encoder import RebelFeatureEncoder
     from p2.search.sparse_cfr_evaluator import SparseCFREvaluator
+    if fused:
+        from p2.search.fused_sparse_cfr_evaluator import FusedSparseCFREvaluator
     warnings.filterwarnings("ignore")
 
     class ValueNet:
@@ -113,6 +124,9 @@ def main() -> None:
         cfg.search.cfr_plus = False
         cfg.search.cfr_avg = False
         ev = SparseCFREvaluator(model=ValueNet(len(bins) + 3), device=dev, cfg=cfg)
+        if fused:
+            ev.__class__ = FusedSparseCFREvaluator
+            ev._ensure_fused_attrs()
         ev.chance_helper.FLOP_SAMPLE_SIZE = 0
         ev.chance_helper.NUM_PERM_SAMPLES = 0
 
@@ -175,10 +189,10 @@ def main() -> None:
     for f in ENV_FIELDS + ("deck",):
         out[f"reset/{f}"] = getattr(env, f).clone().numpy()
     out["reset/seed"] = np.int64(99)
-    path = os.path.join(HERE, "training_data_golden.npz")
+    path = os.path.join(HERE, "fused_training_data_golden.npz" if fused else "training_data_golden.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path) // 1024, "KiB")
 
 
 if __name__ == "__main__":
-    main()
+    main(fused="--fused" in sys.argv[1:])
