@@ -132,7 +132,7 @@ def cases(repeats: int):
     # --- flop chance node: 64 preflop states x 256 drawn canonical flops, 6 of 24 suit permutations
     from .card_utils import combo_suit_permutation_tensor
     ks, kf = 64, 256
-    canonical, count, _, _ = CH.canonical_flops()
+    canonical = CH.canonical_flops()[0]
     flops = torch.from_numpy(canonical[rng.integers(0, canonical.shape[0], kf)]).to(dev)
     pre_f = bel[:ks].contiguous()
     roots_f = torch.arange(ks, device=dev)
@@ -168,7 +168,6 @@ def cases(repeats: int):
     n_children = int(ev.child_count[rows].sum())
     yield (f"policy_targets nodes={rows.numel()}", (n_children + rows.numel() * ev.num_actions) * H * 4,
            lambda: ev._policy_targets(rows))
-    all_rows = torch.arange(ev.total_nodes, device=dev)
     yield (f"encode nodes={ev.total_nodes}", ev.total_nodes * (13 * 8 + 16 + 5 * 8 + 10 * 8),
            lambda: ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask))
 

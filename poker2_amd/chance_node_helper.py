@@ -21,6 +21,7 @@ import numpy as np
 
 from . import _lib
 from .card_utils import NUM_HANDS, combo_suit_permutation_tensor, suit_permutations_tensor
+from ._guards import require as _req
 
 
 @dataclass
@@ -35,10 +36,10 @@ class MLPFeatures:
 
     def __post_init__(self) -> None:
         n = self.context.shape[0]
-        assert self.street.shape == (n,)
-        assert self.to_act.shape == (n,)
-        assert self.board.shape == (n, 5)
-        assert self.beliefs.shape == (n, 2 * NUM_HANDS)
+        _req(self.street.shape == (n,), "self.street.shape == (n,)")
+        _req(self.to_act.shape == (n,), "self.to_act.shape == (n,)")
+        _req(self.board.shape == (n, 5), "self.board.shape == (n, 5)")
+        _req(self.beliefs.shape == (n, 2 * NUM_HANDS), "self.beliefs.shape == (n, 2 * NUM_HANDS)")
 
     def __len__(self) -> int:
         return self.context.shape[0]
@@ -80,8 +81,9 @@ def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, 
         raise RuntimeError("chance_expand needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(pre_chance_beliefs, "chance_expand")
     dev = pre_chance_beliefs.device
-    assert pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS)
-    assert board_pre.dim() == 2 and board_pre.shape[1] == 5
+    _req(pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS),
+         "pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS)")
+    _req(board_pre.dim() == 2 and board_pre.shape[1] == 5, "board_pre.dim() == 2 and board_pre.shape[1] == 5")
     pre = pre_chance_beliefs.contiguous().float()
     board = board_pre.to(device=dev, dtype=torch.int64).contiguous()
     roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
@@ -110,7 +112,8 @@ def chance_mean(hand_values: torch.Tensor, sample_offsets: torch.Tensor) -> torc
     if not _lib.hip_is_available():
         raise RuntimeError("chance_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(hand_values, "chance_mean")
-    assert hand_values.dim() == 3 and tuple(hand_values.shape[1:]) == (2, NUM_HANDS)
+    _req(hand_values.dim() == 3 and tuple(hand_values.shape[1:]) == (2, NUM_HANDS),
+         "hand_values.dim() == 3 and tuple(hand_values.shape[1:]) == (2, NUM_HANDS)")
     hv = hand_values.contiguous().float()
     offsets = sample_offsets.to(device=hv.device, dtype=torch.int64).contiguous()
     b = offsets.numel() - 1
@@ -127,8 +130,9 @@ def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, fl
         raise RuntimeError("flop_expand needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(pre_chance_beliefs, "flop_expand")
     dev = pre_chance_beliefs.device
-    assert pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS)
-    assert flops.dim() == 2 and flops.shape[1] == 3
+    _req(pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS),
+         "pre_chance_beliefs.dim() == 3 and tuple(pre_chance_beliefs.shape[1:]) == (2, NUM_HANDS)")
+    _req(flops.dim() == 2 and flops.shape[1] == 3, "flops.dim() == 2 and flops.shape[1] == 3")
     pre = pre_chance_beliefs.contiguous().float()
     roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
     if roots.numel() and (int(roots.min()) < 0 or int(roots.max()) >= pre.shape[0]):
@@ -152,10 +156,12 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
         raise RuntimeError("perm_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(hand_values, "perm_mean")
     dev = hand_values.device
-    assert hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)
-    assert perms.dim() == 2 and perms.shape[1] == NUM_HANDS and 1 <= perms.shape[0] <= 24
+    _req(hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS),
+         "hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)")
+    _req(perms.dim() == 2 and perms.shape[1] == NUM_HANDS and 1 <= perms.shape[0] <= 24,
+         "perms.dim() == 2 and perms.shape[1] == NUM_HANDS and 1 <= perms.shape[0] <= 24")
     b, k = hand_values.shape[0], hand_values.shape[1]
-    assert weight.shape == (k,)
+    _req(weight.shape == (k,), "weight.shape == (k,)")
     hv = hand_values.contiguous().float()
     if check_perms and (int(perms.min()) < 0 or int(perms.max()) >= NUM_HANDS):   # two device reads: skip for known tables
         raise IndexError("perms must map hands to hand indices 0..1325")
@@ -165,7 +171,8 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
     if out is None:
         out = torch.empty(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     else:
-        assert out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()
+        _req(out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous(),
+             "out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()")
     # enough workgroups to fill the chip: 2 per state, times shares of the flops
     shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
     workspace = torch.empty(shares, b, 2, NUM_HANDS, dtype=torch.float32, device=dev) if shares > 1 else None
@@ -181,16 +188,18 @@ def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tenso
         raise RuntimeError("orbit_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(hand_values, "orbit_mean")
     dev = hand_values.device
-    assert hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)
+    _req(hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS),
+         "hand_values.dim() == 4 and tuple(hand_values.shape[2:]) == (2, NUM_HANDS)")
     b, k = hand_values.shape[0], hand_values.shape[1]
-    assert weight.shape == (k,)
+    _req(weight.shape == (k,), "weight.shape == (k,)")
     hv = hand_values.contiguous().float()
     w = weight.to(device=dev, dtype=torch.float32).contiguous()
     accumulate = out is not None
     if out is None:
         out = torch.empty(b, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     else:
-        assert out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()
+        _req(out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous(),
+             "out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()")
     shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
     workspace = torch.empty(shares, b, 2, NUM_HANDS, dtype=torch.float32, device=dev) if shares > 1 else None
     _lib.call("p2hip_orbit_mean", _lib.ptr(hv), b, k, _lib.ptr(w), int(accumulate), _lib.ptr(out),

@@ -42,6 +42,7 @@ from .chance_node_helper import ChanceNodeHelper
 from .rebel_batch import RebelBatch
 from .rebel_feature_encoder import RebelFeatureEncoder
 from .tree import CARDS_ON_STREET, RootStates, SparseTree, build_sparse_tree, build_sparse_tree_device
+from ._guards import require as _req
 
 STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
                "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",
@@ -755,7 +756,7 @@ class HipSparseCFREvaluator:
         depth = 0
         active = ~effective_leaf[sampled]
         while bool(active.any()):
-            assert depth <= self.tree_depth
+            _req(depth <= self.tree_depth, "depth <= self.tree_depth")
             nodes = sampled[active]
             to_act = self.env.to_act[nodes]
             explore = torch.rand(nodes.numel(), generator=gen, device=gdev).to(dev) < sample_epsilon
@@ -764,7 +765,8 @@ class HipSparseCFREvaluator:
             sampled[active] = self.child_offsets[nodes] + child_action_index[nodes, actions]
             active = ~effective_leaf[sampled]
             depth += 1
-        assert bool(effective_leaf[sampled].all()) and not bool(self.env.done[sampled].any())
+        _req(bool(effective_leaf[sampled].all()) and not bool(self.env.done[sampled].any()),
+             "bool(effective_leaf[sampled].all()) and not bool(self.env.done[sampled].any())")
         keep = sampled[sampled >= n]            # roots that are leaves themselves are not continued
         rows = keep.cpu().numpy()
         tree = self.tree
@@ -903,7 +905,7 @@ class HipSparseCFREvaluator:
         if deviating_player is None:
             deviating_player = self._fan_out_deep(self.env.to_act[:n])
         deviating_player = deviating_player.to(device=self.device, dtype=torch.int64).contiguous()
-        assert deviating_player.shape == (self.total_nodes,)
+        _req(deviating_player.shape == (self.total_nodes,), "deviating_player.shape == (self.total_nodes,)")
         policy = policy.contiguous()
         beliefs = beliefs.contiguous()
         values_br = torch.where(self.leaf_mask[:, None, None], base_values, torch.zeros_like(base_values)).contiguous()

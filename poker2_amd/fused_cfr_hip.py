@@ -18,6 +18,7 @@ import torch
 
 from . import _lib
 from ._lib import hip_is_available
+from ._guards import require as _req
 
 _H = 1326
 
@@ -58,6 +59,28 @@ _S = _lib.stream_ptr
 _p = _lib.ptr
 
 
+def _f32(**tensors) -> None:
+    """Every named tensor is contiguous float32 on the GPU (the kernels read raw fp32 rows)."""
+    for name, t in tensors.items():
+        _req(t.dtype == torch.float32 and t.is_contiguous() and t.device.type == "cuda",
+             f"{name} must be a contiguous float32 GPU tensor, got {t.dtype} on {t.device}")
+
+
+def _i64(rows: int, **tensors) -> None:
+    """Every named tensor is a contiguous int64 GPU vector with at least ``rows`` entries (the
+    kernels read index arrays as 8-byte integers)."""
+    for name, t in tensors.items():
+        _req(t.dtype == torch.int64 and t.is_contiguous() and t.dim() == 1 and t.shape[0] >= rows
+             and t.device.type == "cuda", f"{name} must be a contiguous int64 GPU vector of >= {rows} entries, "
+             f"got {t.dtype} {tuple(t.shape)} on {t.device}")
+
+
+def _scalar_ptrs(**tensors) -> None:
+    for name, t in tensors.items():
+        _req(t.dtype == torch.float32 and t.numel() >= 1 and t.device.type == "cuda",
+             f"{name} must be a float32 GPU scalar tensor")
+
+
 # --------------------------------------------------------------------------- K1
 def fused_dcfr_update_(cumulative_regrets, regret_weight_sums, regrets, t: int, cfr_type, dcfr_alpha: float,
                        dcfr_beta: float, cfr_plus: bool, positive_regrets_out=None, block_size: int = 1024) -> None:
@@ -67,10 +90,11 @@ def fused_dcfr_update_(cumulative_regrets, regret_weight_sums, regrets, t: int, 
         raise ValueError("fused_dcfr_update_ requires GPU tensors.")
     if getattr(cfr_type, "name", cfr_type) == "linear":
         raise NotImplementedError("Linear CFR path not supported; default config uses discounted_plus.")
-    assert cumulative_regrets.is_contiguous()
-    assert regret_weight_sums.is_contiguous()
-    assert regrets.is_contiguous()
-    assert cumulative_regrets.shape == regret_weight_sums.shape == regrets.shape
+    _req(cumulative_regrets.is_contiguous(), "cumulative_regrets.is_contiguous()")
+    _req(regret_weight_sums.is_contiguous(), "regret_weight_sums.is_contiguous()")
+    _req(regrets.is_contiguous(), "regrets.is_contiguous()")
+    _req(cumulative_regrets.shape == regret_weight_sums.shape == regrets.shape,
+         "cumulative_regrets.shape == regret_weight_sums.shape == regrets.shape")
     apply_dcfr = getattr(cfr_type, "name", cfr_type) in ("discounted", "discounted_plus")
     if apply_dcfr:
         a = float(t ** dcfr_alpha)
@@ -88,6 +112,12 @@ def fused_dcfr_update_with_tensors_(cumulative_regrets, regret_weight_sums, regr
                                     positive_regrets_out=None, block_size: int = 1024) -> None:
     """fused_cfr_triton.py:200-235."""
     _need()
+    _f32(cumulative_regrets=cumulative_regrets, regret_weight_sums=regret_weight_sums, regrets=regrets)
+    _req(cumulative_regrets.shape == regret_weight_sums.shape == regrets.shape, "regret tensors differ in shape")
+    _scalar_ptrs(t_alpha_num=t_alpha_num, t_beta_num=t_beta_num, t_alpha_den=t_alpha_den, t_beta_den=t_beta_den)
+    if positive_regrets_out is not None:
+        _f32(positive_regrets_out=positive_regrets_out)
+        _req(positive_regrets_out.shape == cumulative_regrets.shape, "positive_regrets_out differs in shape")
     _lib.call("p2hip_dcfr_update", _p(cumulative_regrets), _p(regret_weight_sums), _p(regrets), _p(t_alpha_num),
               _p(t_beta_num), _p(t_alpha_den), _p(t_beta_den), cumulative_regrets.numel(), int(bool(apply_dcfr)),
               int(bool(cfr_plus)), _p(positive_regrets_out), _S())
@@ -98,10 +128,10 @@ def fused_block_and_normalize_beliefs_(target, allowed_hands, allowed_hands_prob
     """Mask by ``allowed_hands``, normalise rows, fall back to ``allowed_hands_prob`` where the
     row sum is <= eps (fused_cfr_triton.py:286-335)."""
     _need()
-    assert target.is_contiguous()
-    assert allowed_hands.is_contiguous()
-    assert allowed_hands_prob.is_contiguous()
-    assert target.device.type == "cuda"
+    _req(target.is_contiguous(), "target.is_contiguous()")
+    _req(allowed_hands.is_contiguous(), "allowed_hands.is_contiguous()")
+    _req(allowed_hands_prob.is_contiguous(), "allowed_hands_prob.is_contiguous()")
+    _req(target.device.type == "cuda", "target.device.type == \"cuda\"")
     if target.dim() == 3:
         n, p, h = target.shape
         rows, stride = n * p, p
@@ -110,9 +140,11 @@ def fused_block_and_normalize_beliefs_(target, allowed_hands, allowed_hands_prob
         rows, stride = n, 1
     else:
         raise ValueError(f"target must be 2D or 3D, got {target.shape}")
-    assert h == _H
-    assert allowed_hands.shape == (n, h) and allowed_hands.dtype == torch.bool
-    assert allowed_hands_prob.shape == (n, h)
+    _req(h == _H, "h == _H")
+    _req(allowed_hands.shape == (n, h) and allowed_hands.dtype == torch.bool,
+         "allowed_hands.shape == (n, h) and allowed_hands.dtype == torch.bool")
+    _req(allowed_hands_prob.shape == (n, h), "allowed_hands_prob.shape == (n, h)")
+    _f32(target=target, allowed_hands_prob=allowed_hands_prob)
     _lib.call("p2hip_block_and_normalize", _p(target), _p(allowed_hands), _p(allowed_hands_prob), rows, stride,
               float(eps), _S())
 
@@ -122,11 +154,13 @@ def fused_regret_matching_divide_(positive_regrets, denom, uniform_fallback, out
                                   block_size: int = 1024) -> None:
     """out = where(denom > eps, pos / max(denom, eps), uniform) (fused_cfr_triton.py:369-399)."""
     _need()
-    assert positive_regrets.is_contiguous()
-    assert denom.is_contiguous()
-    assert uniform_fallback.is_contiguous()
-    assert out.is_contiguous()
-    assert positive_regrets.shape == denom.shape == uniform_fallback.shape == out.shape
+    _req(positive_regrets.is_contiguous(), "positive_regrets.is_contiguous()")
+    _req(denom.is_contiguous(), "denom.is_contiguous()")
+    _req(uniform_fallback.is_contiguous(), "uniform_fallback.is_contiguous()")
+    _req(out.is_contiguous(), "out.is_contiguous()")
+    _req(positive_regrets.shape == denom.shape == uniform_fallback.shape == out.shape,
+         "positive_regrets.shape == denom.shape == uniform_fallback.shape == out.shape")
+    _f32(positive_regrets=positive_regrets, denom=denom, uniform_fallback=uniform_fallback, out=out)
     _lib.call("p2hip_regret_matching_divide", _p(positive_regrets), _p(denom), _p(uniform_fallback), _p(out),
               positive_regrets.numel(), float(eps), _S())
 
@@ -136,14 +170,19 @@ def fused_weight_child_values(values_src, prev_actor, policy_hero, policy_opp, o
     """out[m,p] = values_src[m,p] * (policy_hero[m] if p == prev_actor[m] else policy_opp[m])
     (fused_cfr_triton.py:438-477)."""
     _need()
-    assert values_src.is_contiguous() and values_src.dim() == 3
-    assert out.is_contiguous() and out.shape == values_src.shape
-    assert prev_actor.is_contiguous() and prev_actor.dim() == 1
-    assert policy_hero.is_contiguous() and policy_opp.is_contiguous()
+    _req(values_src.is_contiguous() and values_src.dim() == 3, "values_src.is_contiguous() and values_src.dim() == 3")
+    _req(out.is_contiguous() and out.shape == values_src.shape,
+         "out.is_contiguous() and out.shape == values_src.shape")
+    _req(prev_actor.is_contiguous() and prev_actor.dim() == 1, "prev_actor.is_contiguous() and prev_actor.dim() == 1")
+    _req(policy_hero.is_contiguous() and policy_opp.is_contiguous(),
+         "policy_hero.is_contiguous() and policy_opp.is_contiguous()")
     m, p, h = values_src.shape
-    assert p == 2, "Only supports 2 players."
-    assert prev_actor.shape[0] == m
-    assert policy_hero.shape == (m, h) and policy_opp.shape == (m, h)
+    _req(p == 2, "Only supports 2 players.")
+    _req(prev_actor.shape[0] == m, "prev_actor.shape[0] == m")
+    _req(policy_hero.shape == (m, h) and policy_opp.shape == (m, h),
+         "policy_hero.shape == (m, h) and policy_opp.shape == (m, h)")
+    _f32(values_src=values_src, policy_hero=policy_hero, policy_opp=policy_opp, out=out)
+    _i64(m, prev_actor=prev_actor)
     _lib.call("p2hip_weight_child_values", _p(values_src), _p(prev_actor), _p(policy_hero), _p(policy_opp), _p(out),
               m, _S())
 
@@ -152,11 +191,11 @@ def fused_weight_child_values(values_src, prev_actor, policy_hero, policy_opp, o
 def fused_update_average_values_(values_avg, latest_values, old: float, new: float, block_size: int = 1024) -> None:
     """values_avg = (values_avg*old + latest*new) * (1/(old+new)) (fused_cfr_triton.py:509-535)."""
     _need()
-    assert values_avg.is_contiguous()
-    assert latest_values.is_contiguous()
-    assert values_avg.shape == latest_values.shape
+    _req(values_avg.is_contiguous(), "values_avg.is_contiguous()")
+    _req(latest_values.is_contiguous(), "latest_values.is_contiguous()")
+    _req(values_avg.shape == latest_values.shape, "values_avg.shape == latest_values.shape")
     total = float(old) + float(new)
-    assert total != 0.0
+    _req(total != 0.0, "total != 0.0")
     o_t, n_t, inv_t = _scalars([old, new, 1.0 / total], values_avg)
     fused_update_average_values_with_tensors_(values_avg, latest_values, o_t, n_t, inv_t, block_size=block_size)
 
@@ -165,6 +204,9 @@ def fused_update_average_values_with_tensors_(values_avg, latest_values, old, ne
                                               block_size: int = 1024) -> None:
     """fused_cfr_triton.py:538-560."""
     _need()
+    _f32(values_avg=values_avg, latest_values=latest_values)
+    _req(values_avg.shape == latest_values.shape, "values_avg.shape == latest_values.shape")
+    _scalar_ptrs(old=old, new=new, inv_total=inv_total)
     _lib.call("p2hip_update_average_values", _p(values_avg), _p(latest_values), _p(old), _p(new), _p(inv_total),
               values_avg.numel(), _S())
 
@@ -174,14 +216,19 @@ def fused_avg_values_zero_sum_(values_avg, latest_values, beliefs, old, new, inv
     """Mix, then optionally subtract 0.5 * sum_p sum_h v_p*b_p per node (0 where ``ignore_mask``)
     (fused_cfr_triton.py:623-668)."""
     _need()
-    assert values_avg.is_contiguous() and latest_values.is_contiguous()
-    assert beliefs.is_contiguous()
-    assert values_avg.shape == latest_values.shape == beliefs.shape
-    assert values_avg.dim() == 3 and values_avg.shape[1] == 2
+    _req(values_avg.is_contiguous() and latest_values.is_contiguous(),
+         "values_avg.is_contiguous() and latest_values.is_contiguous()")
+    _req(beliefs.is_contiguous(), "beliefs.is_contiguous()")
+    _req(values_avg.shape == latest_values.shape == beliefs.shape,
+         "values_avg.shape == latest_values.shape == beliefs.shape")
+    _req(values_avg.dim() == 3 and values_avg.shape[1] == 2, "values_avg.dim() == 3 and values_avg.shape[1] == 2")
     n_rows, _, h = values_avg.shape
-    assert h == _H
+    _req(h == _H, "h == _H")
     if ignore_mask is not None:
-        assert ignore_mask.is_contiguous() and ignore_mask.shape == (n_rows,) and ignore_mask.dtype == torch.bool
+        _req(ignore_mask.is_contiguous() and ignore_mask.shape == (n_rows,) and ignore_mask.dtype == torch.bool,
+             "ignore_mask.is_contiguous() and ignore_mask.shape == (n_rows,) and ignore_mask.dtype == torch.bool")
+    _f32(values_avg=values_avg, latest_values=latest_values, beliefs=beliefs)
+    _scalar_ptrs(old=old, new=new, inv_total=inv_total)
     _lib.call("p2hip_avg_values_zero_sum", _p(values_avg), _p(latest_values), _p(beliefs), _p(ignore_mask), _p(old),
               _p(new), _p(inv_total), n_rows, int(bool(enforce_zero_sum)), _S())
 
@@ -192,18 +239,26 @@ def fused_regret_tail_(regrets, values_achieved, actor_values, src_weights, pare
     """regrets[c] = src_weights[parent(c)] * (values_achieved[c, prev_actor[c]] - actor_values[parent(c)])
     for c >= bottom (fused_cfr_triton.py:712-766)."""
     _need()
-    assert regrets.is_contiguous() and regrets.dim() == 2
-    assert values_achieved.is_contiguous() and values_achieved.dim() == 3
-    assert values_achieved.shape[1] == 2
-    assert actor_values.is_contiguous() and actor_values.dim() == 2
-    assert src_weights.is_contiguous() and src_weights.dim() == 2
-    assert actor_values.shape == src_weights.shape
-    assert parent_index.is_contiguous() and parent_index.dim() == 1
-    assert prev_actor.is_contiguous() and prev_actor.dim() == 1
+    _req(regrets.is_contiguous() and regrets.dim() == 2, "regrets.is_contiguous() and regrets.dim() == 2")
+    _req(values_achieved.is_contiguous() and values_achieved.dim() == 3,
+         "values_achieved.is_contiguous() and values_achieved.dim() == 3")
+    _req(values_achieved.shape[1] == 2, "values_achieved.shape[1] == 2")
+    _req(actor_values.is_contiguous() and actor_values.dim() == 2,
+         "actor_values.is_contiguous() and actor_values.dim() == 2")
+    _req(src_weights.is_contiguous() and src_weights.dim() == 2,
+         "src_weights.is_contiguous() and src_weights.dim() == 2")
+    _req(actor_values.shape == src_weights.shape, "actor_values.shape == src_weights.shape")
+    _req(parent_index.is_contiguous() and parent_index.dim() == 1,
+         "parent_index.is_contiguous() and parent_index.dim() == 1")
+    _req(prev_actor.is_contiguous() and prev_actor.dim() == 1, "prev_actor.is_contiguous() and prev_actor.dim() == 1")
     total, h = regrets.shape
-    assert values_achieved.shape == (total, 2, h)
-    assert parent_index.shape == (total,)
-    assert prev_actor.shape == (total,)
+    _req(values_achieved.shape == (total, 2, h), "values_achieved.shape == (total, 2, h)")
+    _req(parent_index.shape == (total,), "parent_index.shape == (total,)")
+    _req(prev_actor.shape == (total,), "prev_actor.shape == (total,)")
+    _f32(regrets=regrets, values_achieved=values_achieved, actor_values=actor_values, src_weights=src_weights)
+    _i64(total, parent_index=parent_index, prev_actor=prev_actor)
+    _req(0 <= int(bottom) <= total, f"bottom={bottom} outside the {total} rows")
+    _req(actor_values.shape[1] == h, "actor_values.shape[1] == h")
     _lib.call("p2hip_regret_tail", _p(regrets), _p(values_achieved), _p(actor_values), _p(src_weights),
               _p(parent_index), _p(prev_actor), int(bottom), total, _S())
 
@@ -213,19 +268,23 @@ def fused_average_policy_mix_(policy_probs_avg, policy_probs, self_reach, self_r
                               old: float, new: float, bottom: int, eps: float = 1e-5, block_h: int = 512) -> None:
     """Reach-weighted average-policy mix before renormalisation (fused_cfr_triton.py:823-876)."""
     _need()
-    assert policy_probs_avg.is_contiguous() and policy_probs_avg.dim() == 2
-    assert policy_probs.is_contiguous() and policy_probs.dim() == 2
-    assert self_reach.is_contiguous() and self_reach.dim() == 3
-    assert self_reach_avg.is_contiguous() and self_reach_avg.dim() == 3
-    assert self_reach.shape[1] == 2 and self_reach_avg.shape[1] == 2
+    _req(policy_probs_avg.is_contiguous() and policy_probs_avg.dim() == 2,
+         "policy_probs_avg.is_contiguous() and policy_probs_avg.dim() == 2")
+    _req(policy_probs.is_contiguous() and policy_probs.dim() == 2,
+         "policy_probs.is_contiguous() and policy_probs.dim() == 2")
+    _req(self_reach.is_contiguous() and self_reach.dim() == 3, "self_reach.is_contiguous() and self_reach.dim() == 3")
+    _req(self_reach_avg.is_contiguous() and self_reach_avg.dim() == 3,
+         "self_reach_avg.is_contiguous() and self_reach_avg.dim() == 3")
+    _req(self_reach.shape[1] == 2 and self_reach_avg.shape[1] == 2,
+         "self_reach.shape[1] == 2 and self_reach_avg.shape[1] == 2")
     total, h = policy_probs_avg.shape
-    assert policy_probs.shape == (total, h)
-    assert self_reach.shape == (total, 2, h)
-    assert self_reach_avg.shape == (total, 2, h)
-    assert to_act.shape == (total,)
-    assert parent_index.shape == (total,)
+    _req(policy_probs.shape == (total, h), "policy_probs.shape == (total, h)")
+    _req(self_reach.shape == (total, 2, h), "self_reach.shape == (total, 2, h)")
+    _req(self_reach_avg.shape == (total, 2, h), "self_reach_avg.shape == (total, 2, h)")
+    _req(to_act.shape == (total,), "to_act.shape == (total,)")
+    _req(parent_index.shape == (total,), "parent_index.shape == (total,)")
     total_weight = float(old) + float(new)
-    assert total_weight != 0.0
+    _req(total_weight != 0.0, "total_weight != 0.0")
     o_t, n_t, tot_t = _scalars([old, new, total_weight], policy_probs_avg)
     fused_average_policy_mix_with_tensors_(policy_probs_avg, policy_probs, self_reach, self_reach_avg, to_act,
                                            parent_index, o_t, n_t, tot_t, bottom=bottom, eps=eps, block_h=block_h)
@@ -236,7 +295,15 @@ def fused_average_policy_mix_with_tensors_(policy_probs_avg, policy_probs, self_
                                            block_h: int = 512) -> None:
     """fused_cfr_triton.py:879-914."""
     _need()
-    total, _ = policy_probs_avg.shape
+    _req(policy_probs_avg.dim() == 2, "policy_probs_avg.dim() == 2")
+    total, h = policy_probs_avg.shape
+    _f32(policy_probs_avg=policy_probs_avg, policy_probs=policy_probs, self_reach=self_reach,
+         self_reach_avg=self_reach_avg)
+    _req(policy_probs.shape == (total, h) and self_reach.shape == (total, 2, h)
+         and self_reach_avg.shape == (total, 2, h), "policy / reach tensors differ in shape")
+    _i64(total, to_act=to_act, parent_index=parent_index)
+    _scalar_ptrs(old=old, new=new, total_weight=total_weight)
+    _req(0 <= int(bottom) <= total, f"bottom={bottom} outside the {total} rows")
     _lib.call("p2hip_average_policy_mix", _p(policy_probs_avg), _p(policy_probs), _p(self_reach), _p(self_reach_avg),
               _p(to_act), _p(parent_index), _p(old), _p(new), _p(total_weight), int(bottom), total, float(eps), _S())
 
@@ -248,7 +315,7 @@ def unblocked_mass_triton(target: torch.Tensor) -> torch.Tensor:
     if target.device.type != "cuda":
         raise ValueError("unblocked_mass requires GPU tensors.")
     orig_shape = target.shape
-    assert orig_shape[-1] == _H, f"last dim must be {_H}, got {orig_shape}"
+    _req(orig_shape[-1] == _H, f"last dim must be {_H}, got {orig_shape}")
     flat = target.reshape(-1, _H).contiguous()
     out = torch.empty_like(flat)
     _lib.call("p2hip_unblocked_mass", _p(flat), flat.shape[0], _p(out), _S())
@@ -263,8 +330,12 @@ def unblocked_mass_opp_at_parents_triton(beliefs, to_act, top: int, cached_stats
     (fused_cfr_triton.py:1067-1107).  ``cached_stats`` is accepted and ignored."""
     _need()
     total, p, h = beliefs.shape
-    assert p == 2 and h == _H
-    assert beliefs.is_contiguous() and to_act.is_contiguous() and to_act.dtype == torch.int64
+    _req(p == 2 and h == _H, "p == 2 and h == _H")
+    _req(beliefs.is_contiguous() and to_act.is_contiguous() and to_act.dtype == torch.int64,
+         "beliefs.is_contiguous() and to_act.is_contiguous() and to_act.dtype == torch.int64")
+    _req(0 <= int(top) <= total, f"top={top} outside the {total} rows of beliefs")
+    _i64(int(top), to_act=to_act)
+    _f32(beliefs=beliefs)
     out = torch.empty((top, h), device=beliefs.device, dtype=beliefs.dtype)
     _lib.call("p2hip_unblocked_mass_by_player", _p(beliefs), _p(to_act), int(top), 1, _p(out), _S())
     return out
@@ -275,14 +346,19 @@ def unblocked_mass_ratio_indirect_triton(numer_target, denom_target, parent_inde
     """where(unblk(denom[parent]) > eps, unblk(numer) / unblk(denom[parent]), 0)
     (fused_cfr_triton.py:1499-1556).  ``denom_stats`` is accepted and ignored."""
     _need()
-    assert numer_target.is_contiguous() and numer_target.dim() == 2
-    assert denom_target.is_contiguous() and denom_target.dim() == 2
-    assert parent_index.is_contiguous() and parent_index.dim() == 1
+    _req(numer_target.is_contiguous() and numer_target.dim() == 2,
+         "numer_target.is_contiguous() and numer_target.dim() == 2")
+    _req(denom_target.is_contiguous() and denom_target.dim() == 2,
+         "denom_target.is_contiguous() and denom_target.dim() == 2")
+    _req(parent_index.is_contiguous() and parent_index.dim() == 1,
+         "parent_index.is_contiguous() and parent_index.dim() == 1")
     num_children, h = numer_target.shape
     top = denom_target.shape[0]
-    assert denom_target.shape == (top, h)
-    assert parent_index.shape == (num_children,)
-    assert h == _H
+    _req(denom_target.shape == (top, h), "denom_target.shape == (top, h)")
+    _req(parent_index.shape == (num_children,), "parent_index.shape == (num_children,)")
+    _req(h == _H, "h == _H")
+    _f32(numer_target=numer_target, denom_target=denom_target)
+    _i64(num_children, parent_index=parent_index)
     out = torch.empty_like(numer_target)
     _lib.call("p2hip_unblocked_mass_ratio", _p(numer_target), _p(denom_target), _p(parent_index), num_children,
               float(eps), _p(out), _S())
@@ -292,7 +368,7 @@ def unblocked_mass_ratio_indirect_triton(numer_target, denom_target, parent_inde
 def unblocked_mass_ratio_triton(numer_target, denom_target, eps: float = 1e-5) -> torch.Tensor:
     """fused_cfr_triton.py:1559-1602."""
     _need()
-    assert numer_target.shape == denom_target.shape
+    _req(numer_target.shape == denom_target.shape, "numer_target.shape == denom_target.shape")
     orig = numer_target.shape
     n = numer_target.reshape(-1, _H).contiguous()
     d = denom_target.reshape(-1, _H).contiguous()
@@ -305,10 +381,15 @@ def unblocked_mass_ratio_triton(numer_target, denom_target, eps: float = 1e-5) -
 def fused_parent_sum(values, child_offsets, child_count, max_children: int = 8, block_h: int = 512) -> torch.Tensor:
     """Per-parent sum over its contiguous child rows -> [num_parents, H] (fused_cfr_triton.py:1279-1313)."""
     _need()
-    assert values.is_contiguous() and values.dim() == 2
-    assert child_offsets.is_contiguous() and child_offsets.dim() == 1
-    assert child_count.is_contiguous() and child_count.shape == child_offsets.shape
+    _req(values.is_contiguous() and values.dim() == 2, "values.is_contiguous() and values.dim() == 2")
+    _req(child_offsets.is_contiguous() and child_offsets.dim() == 1,
+         "child_offsets.is_contiguous() and child_offsets.dim() == 1")
+    _req(child_count.is_contiguous() and child_count.shape == child_offsets.shape,
+         "child_count.is_contiguous() and child_count.shape == child_offsets.shape")
     num_parents = child_offsets.shape[0]
+    _f32(values=values)
+    _req(values.shape[1] == _H, "values.shape[1] == 1326")
+    _i64(num_parents, child_offsets=child_offsets, child_count=child_count)
     out = torch.empty(num_parents, values.shape[1], device=values.device, dtype=values.dtype)
     _lib.call("p2hip_parent_sum", _p(values), _p(child_offsets), _p(child_count), num_parents, _p(out), _S())
     return out
@@ -319,12 +400,18 @@ def fused_divide_by_parent_sum_(pos, fallback, parent_sum, parent_index, out, ep
     """out[c] = where(parent_sum[parent(c)] > eps, pos[c] / max(parent_sum, eps), fallback[c])
     (fused_cfr_triton.py:1316-1352); ``out`` may alias ``pos`` or ``fallback``."""
     _need()
-    assert pos.is_contiguous() and fallback.is_contiguous() and out.is_contiguous()
-    assert parent_sum.is_contiguous() and parent_index.is_contiguous()
-    assert pos.dim() == 2 and fallback.shape == pos.shape == out.shape
-    assert parent_sum.dim() == 2 and parent_sum.shape[1] == pos.shape[1]
+    _req(pos.is_contiguous() and fallback.is_contiguous() and out.is_contiguous(),
+         "pos.is_contiguous() and fallback.is_contiguous() and out.is_contiguous()")
+    _req(parent_sum.is_contiguous() and parent_index.is_contiguous(),
+         "parent_sum.is_contiguous() and parent_index.is_contiguous()")
+    _req(pos.dim() == 2 and fallback.shape == pos.shape == out.shape,
+         "pos.dim() == 2 and fallback.shape == pos.shape == out.shape")
+    _req(parent_sum.dim() == 2 and parent_sum.shape[1] == pos.shape[1],
+         "parent_sum.dim() == 2 and parent_sum.shape[1] == pos.shape[1]")
     num_children, _ = pos.shape
-    assert parent_index.shape == (num_children,)
+    _req(parent_index.shape == (num_children,), "parent_index.shape == (num_children,)")
+    _f32(pos=pos, fallback=fallback, parent_sum=parent_sum, out=out)
+    _i64(num_children, parent_index=parent_index)
     _lib.call("p2hip_divide_by_parent_sum", _p(pos), _p(fallback), _p(parent_sum), _p(parent_index), _p(out),
               num_children, float(eps), _S())
 
@@ -333,10 +420,17 @@ def fused_sibling_sum(values, child_offsets, child_count, bottom: int, num_child
                       block_h: int = 512) -> torch.Tensor:
     """Sum over each child's siblings, child-aligned -> [num_children, H] (fused_cfr_triton.py:1355-1398)."""
     _need()
-    assert values.is_contiguous() and values.dim() == 2
-    assert child_offsets.is_contiguous() and child_offsets.dim() == 1
-    assert child_count.is_contiguous() and child_count.dim() == 1
-    assert child_offsets.shape == child_count.shape
+    _req(values.is_contiguous() and values.dim() == 2, "values.is_contiguous() and values.dim() == 2")
+    _req(child_offsets.is_contiguous() and child_offsets.dim() == 1,
+         "child_offsets.is_contiguous() and child_offsets.dim() == 1")
+    _req(child_count.is_contiguous() and child_count.dim() == 1,
+         "child_count.is_contiguous() and child_count.dim() == 1")
+    _req(child_offsets.shape == child_count.shape, "child_offsets.shape == child_count.shape")
+    _f32(values=values)
+    _req(values.shape[1] == _H, "values.shape[1] == 1326")
+    _i64(child_offsets.shape[0], child_offsets=child_offsets, child_count=child_count)
+    _req(0 <= int(bottom) and 0 <= int(num_children) and int(bottom) + int(num_children) <= values.shape[0],
+         f"children [{bottom}, {bottom}+{num_children}) outside the {values.shape[0]} rows of values")
     out = torch.empty(num_children, values.shape[1], device=values.device, dtype=values.dtype)
     _lib.call("p2hip_sibling_sum", _p(values), _p(child_offsets), _p(child_count), child_offsets.shape[0],
               int(bottom), _p(out), _S())
@@ -348,9 +442,10 @@ def fused_model_values_mix(hand_values, last_model_values, old: float, new: floa
                            block_size: int = 1024) -> torch.Tensor:
     """((old+new)*hand - old*last)/new with pre-divided scalars (fused_cfr_triton.py:1633-1655)."""
     _need()
-    assert hand_values.is_contiguous() and last_model_values.is_contiguous()
-    assert hand_values.shape == last_model_values.shape
-    assert new != 0.0
+    _req(hand_values.is_contiguous() and last_model_values.is_contiguous(),
+         "hand_values.is_contiguous() and last_model_values.is_contiguous()")
+    _req(hand_values.shape == last_model_values.shape, "hand_values.shape == last_model_values.shape")
+    _req(new != 0.0, "new != 0.0")
     out = torch.empty_like(hand_values)
     onon_t, oon_t = _scalars([(old + new) / new, old / new], hand_values)
     fused_model_values_mix_with_tensors(hand_values, last_model_values, onon_t, oon_t, out, block_size=block_size)
@@ -361,6 +456,9 @@ def fused_model_values_mix_with_tensors(hand_values, last_model_values, old_plus
                                         block_size: int = 1024) -> None:
     """fused_cfr_triton.py:1658-1680."""
     _need()
+    _f32(hand_values=hand_values, last_model_values=last_model_values, out=out)
+    _req(hand_values.shape == last_model_values.shape == out.shape, "hand_values / last_model_values / out differ")
+    _scalar_ptrs(old_plus_new_over_new=old_plus_new_over_new, old_over_new=old_over_new)
     _lib.call("p2hip_model_values_mix", _p(hand_values), _p(last_model_values), _p(old_plus_new_over_new),
               _p(old_over_new), _p(out), hand_values.numel(), _S())
 
@@ -369,12 +467,16 @@ def fused_model_values_mix_zero_sum(hand_values, last_model_values, beliefs, old
                                     out, enforce_zero_sum: bool, block_h: int = 2048) -> None:
     """fused_cfr_triton.py:1739-1775."""
     _need()
-    assert hand_values.is_contiguous() and last_model_values.is_contiguous()
-    assert beliefs.is_contiguous() and out.is_contiguous()
-    assert hand_values.shape == last_model_values.shape == beliefs.shape == out.shape
-    assert hand_values.dim() == 3 and hand_values.shape[1] == 2
+    _req(hand_values.is_contiguous() and last_model_values.is_contiguous(),
+         "hand_values.is_contiguous() and last_model_values.is_contiguous()")
+    _req(beliefs.is_contiguous() and out.is_contiguous(), "beliefs.is_contiguous() and out.is_contiguous()")
+    _req(hand_values.shape == last_model_values.shape == beliefs.shape == out.shape,
+         "hand_values.shape == last_model_values.shape == beliefs.shape == out.shape")
+    _req(hand_values.dim() == 3 and hand_values.shape[1] == 2, "hand_values.dim() == 3 and hand_values.shape[1] == 2")
     m, _, h = hand_values.shape
-    assert h == _H
+    _req(h == _H, "h == _H")
+    _f32(hand_values=hand_values, last_model_values=last_model_values, beliefs=beliefs, out=out)
+    _scalar_ptrs(old_plus_new_over_new=old_plus_new_over_new, old_over_new=old_over_new)
     _lib.call("p2hip_model_values_mix_zero_sum", _p(hand_values), _p(last_model_values), _p(beliefs),
               _p(old_plus_new_over_new), _p(old_over_new), _p(out), m, int(bool(enforce_zero_sum)), _S())
 
@@ -385,12 +487,23 @@ def fused_weighted_parent_sum(values, prev_actor, policy_hero, policy_opp, child
     """values[parent_base+p, pl] = sum_children values[c, pl] * (policy_hero[c] if pl == prev_actor[c]
     else policy_opp[c]); parents without children keep their value (fused_cfr_triton.py:1838-1889)."""
     _need()
-    assert values.is_contiguous() and values.dim() == 3 and values.shape[1] == 2
-    assert policy_hero.is_contiguous() and policy_opp.is_contiguous()
-    assert child_offsets.is_contiguous() and child_count.is_contiguous()
+    _req(values.is_contiguous() and values.dim() == 3 and values.shape[1] == 2,
+         "values.is_contiguous() and values.dim() == 3 and values.shape[1] == 2")
+    _req(policy_hero.is_contiguous() and policy_opp.is_contiguous(),
+         "policy_hero.is_contiguous() and policy_opp.is_contiguous()")
+    _req(child_offsets.is_contiguous() and child_count.is_contiguous(),
+         "child_offsets.is_contiguous() and child_count.is_contiguous()")
     total, _, h = values.shape
-    assert policy_hero.shape == (total, h) and policy_opp.shape == (total, h)
-    assert prev_actor.shape == (total,)
+    _req(policy_hero.shape == (total, h) and policy_opp.shape == (total, h),
+         "policy_hero.shape == (total, h) and policy_opp.shape == (total, h)")
+    _req(prev_actor.shape == (total,), "prev_actor.shape == (total,)")
+    _f32(values=values, policy_hero=policy_hero, policy_opp=policy_opp)
+    _req(h == _H, "values.shape[2] == 1326")
+    num_parents = child_offsets.shape[0]
+    _i64(total, prev_actor=prev_actor)
+    _i64(num_parents, child_offsets=child_offsets, child_count=child_count)
+    _req(0 <= int(parent_base) and int(parent_base) + num_parents <= total,
+         f"parents [{parent_base}, {parent_base}+{num_parents}) outside the {total} rows")
     _lib.call("p2hip_weighted_parent_sum", _p(values), _p(prev_actor), _p(policy_hero), _p(policy_opp),
               _p(child_offsets), _p(child_count), child_offsets.shape[0], int(parent_base), _S())
 
@@ -400,14 +513,21 @@ def fused_reach_weights_depth_(reach, policy, allowed_mask, parent_index, prev_a
     """reach[c,p] = reach[parent(c),p] * (policy[c] if p == prev_actor[c] else 1), zero where
     ``allowed_mask[c]`` is False, for c in [start, end) (fused_cfr_triton.py:1944-1986)."""
     _need()
-    assert reach.is_contiguous() and reach.dim() == 3 and reach.shape[1] == 2
-    assert policy.is_contiguous() and policy.dim() == 2
+    _req(reach.is_contiguous() and reach.dim() == 3 and reach.shape[1] == 2,
+         "reach.is_contiguous() and reach.dim() == 3 and reach.shape[1] == 2")
+    _req(policy.is_contiguous() and policy.dim() == 2, "policy.is_contiguous() and policy.dim() == 2")
     total, _, h = reach.shape
-    assert policy.shape == (total, h)
-    assert allowed_mask.shape == (total, h) and allowed_mask.is_contiguous() and allowed_mask.dtype == torch.bool
-    assert parent_index.shape == (total,) and prev_actor.shape == (total,)
+    _req(policy.shape == (total, h), "policy.shape == (total, h)")
+    _req(allowed_mask.shape == (total, h) and allowed_mask.is_contiguous() and allowed_mask.dtype == torch.bool,
+         "allowed_mask.shape == (total, h) and allowed_mask.is_contiguous() and allowed_mask.dtype == torch.bool")
+    _req(parent_index.shape == (total,) and prev_actor.shape == (total,),
+         "parent_index.shape == (total,) and prev_actor.shape == (total,)")
+    _f32(reach=reach, policy=policy)
+    _req(h == _H, "reach.shape[2] == 1326")
+    _i64(total, parent_index=parent_index, prev_actor=prev_actor)
     if end - start <= 0:
         return
+    _req(0 <= int(start) and int(end) <= total, f"rows [{start}, {end}) outside the {total} rows")
     _lib.call("p2hip_reach_weights_depth", _p(reach), _p(policy), _p(allowed_mask), _p(parent_index),
               _p(prev_actor), int(start), int(end), _S())
 
@@ -417,14 +537,23 @@ def fused_deep_beliefs_(out, root_beliefs, reach_weights, allowed_prob, root_ind
     """out[i,p] = normalise(root_beliefs[root_index[i],p] * reach_weights[i,p]) with fallback
     ``allowed_prob[i]``; root rows are left untouched (fused_cfr_triton.py:2039-2092)."""
     _need()
-    assert out.is_contiguous() and out.dim() == 3 and out.shape[1] == 2
-    assert root_beliefs.is_contiguous() and root_beliefs.dim() == 3
-    assert reach_weights.is_contiguous() and reach_weights.shape == out.shape
+    _req(out.is_contiguous() and out.dim() == 3 and out.shape[1] == 2,
+         "out.is_contiguous() and out.dim() == 3 and out.shape[1] == 2")
+    _req(root_beliefs.is_contiguous() and root_beliefs.dim() == 3,
+         "root_beliefs.is_contiguous() and root_beliefs.dim() == 3")
+    _req(reach_weights.is_contiguous() and reach_weights.shape == out.shape,
+         "reach_weights.is_contiguous() and reach_weights.shape == out.shape")
     total, _, h = out.shape
     n = num_roots if num_roots is not None else root_beliefs.shape[0]
-    assert root_beliefs.shape[0] >= n and tuple(root_beliefs.shape[1:]) == (2, h)
-    assert allowed_prob.shape == (total, h) and allowed_prob.is_contiguous()
-    assert root_index.shape == (total,) and root_index.is_contiguous()
+    _req(root_beliefs.shape[0] >= n and tuple(root_beliefs.shape[1:]) == (2, h),
+         "root_beliefs.shape[0] >= n and tuple(root_beliefs.shape[1:]) == (2, h)")
+    _req(allowed_prob.shape == (total, h) and allowed_prob.is_contiguous(),
+         "allowed_prob.shape == (total, h) and allowed_prob.is_contiguous()")
+    _req(root_index.shape == (total,) and root_index.is_contiguous(),
+         "root_index.shape == (total,) and root_index.is_contiguous()")
+    _f32(out=out, root_beliefs=root_beliefs, reach_weights=reach_weights, allowed_prob=allowed_prob)
+    _req(h == _H, "out.shape[2] == 1326")
+    _i64(total, root_index=root_index)
     if total <= n:
         return
     _lib.call("p2hip_deep_beliefs", _p(out), _p(root_beliefs), _p(reach_weights), _p(allowed_prob), _p(root_index),
@@ -435,9 +564,15 @@ def fused_sample_snapshot_(policy_probs_sample, policy_probs, t_sample, t_tensor
     """policy_probs_sample <- where(t_sample == t, policy_probs, policy_probs_sample)
     (fused_sparse_cfr_evaluator.py:494-499); ``t_tensor`` is a 0-D int64 device tensor."""
     _need()
-    assert policy_probs_sample.is_contiguous() and policy_probs.is_contiguous()
-    assert policy_probs_sample.shape == policy_probs.shape
-    assert t_sample.is_contiguous() and t_sample.dtype == torch.int64 and t_tensor.dtype == torch.int64
+    _req(policy_probs_sample.is_contiguous() and policy_probs.is_contiguous(),
+         "policy_probs_sample.is_contiguous() and policy_probs.is_contiguous()")
+    _req(policy_probs_sample.shape == policy_probs.shape, "policy_probs_sample.shape == policy_probs.shape")
+    _req(t_sample.is_contiguous() and t_sample.dtype == torch.int64 and t_tensor.dtype == torch.int64,
+         "t_sample.is_contiguous() and t_sample.dtype == torch.int64 and t_tensor.dtype == torch.int64")
+    _f32(policy_probs_sample=policy_probs_sample, policy_probs=policy_probs)
+    _req(policy_probs.dim() == 2 and policy_probs.shape[1] == _H, "policy_probs must be [rows, 1326]")
+    _i64(policy_probs.shape[0], t_sample=t_sample)
+    _req(t_tensor.numel() >= 1 and t_tensor.device.type == "cuda", "t_tensor must be a GPU scalar tensor")
     _lib.call("p2hip_sample_snapshot", _p(policy_probs), _p(policy_probs_sample), _p(t_sample), _p(t_tensor),
               policy_probs.shape[0], _S())
 
@@ -489,7 +624,8 @@ class ParentBeliefUnblockedStats:
     passing this object as ``cached_stats`` changes nothing; it exists for callers that build it."""
 
     def __init__(self, beliefs_parents: torch.Tensor) -> None:
-        assert beliefs_parents.dim() == 3 and beliefs_parents.shape[1] == 2
+        _req(beliefs_parents.dim() == 3 and beliefs_parents.shape[1] == 2,
+             "beliefs_parents.dim() == 3 and beliefs_parents.shape[1] == 2")
         self.top = beliefs_parents.shape[0]
         self.beliefs_parents = beliefs_parents
 

@@ -12,6 +12,7 @@ from typing import Optional
 import torch
 
 from .chance_node_helper import MLPFeatures
+from ._guards import require as _req
 
 
 @dataclass
@@ -23,15 +24,16 @@ class RebelBatch:
     statistics: dict[str, torch.Tensor] = field(default_factory=dict)
 
     def __post_init__(self) -> None:
-        assert self.value_targets is not None or self.policy_targets is not None
+        _req(self.value_targets is not None or self.policy_targets is not None,
+             "self.value_targets is not None or self.policy_targets is not None")
         n = len(self.features)
-        assert n == self.legal_masks.shape[0]
+        _req(n == self.legal_masks.shape[0], "n == self.legal_masks.shape[0]")
         if self.policy_targets is not None:
-            assert n == self.policy_targets.shape[0]
+            _req(n == self.policy_targets.shape[0], "n == self.policy_targets.shape[0]")
         if self.value_targets is not None:
-            assert n == self.value_targets.shape[0]
+            _req(n == self.value_targets.shape[0], "n == self.value_targets.shape[0]")
         for key in self.statistics:
-            assert n == self.statistics[key].shape[0], key
+            _req(n == self.statistics[key].shape[0], key)
 
     def __len__(self) -> int:
         return len(self.features)

@@ -19,6 +19,7 @@ import torch
 from .card_utils import NUM_HANDS
 from .rebel_batch import RebelBatch
 from .tree import RootStates
+from ._guards import require as _req
 
 
 @dataclass
@@ -28,7 +29,7 @@ class PublicBeliefState:
     beliefs: torch.Tensor      # [batch, 2, 1326]
 
     def __post_init__(self) -> None:
-        assert self.beliefs.shape[0] == self.env.n
+        _req(self.beliefs.shape[0] == self.env.n, "self.beliefs.shape[0] == self.env.n")
 
 
 class EnvProto:

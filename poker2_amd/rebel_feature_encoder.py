@@ -14,6 +14,7 @@ import torch
 from . import _lib
 from .card_utils import NUM_HANDS
 from .chance_node_helper import MLPFeatures
+from ._guards import require as _req
 
 
 class RebelFeatureEncoder:
@@ -63,7 +64,7 @@ class RebelFeatureEncoder:
         pre_ptr, pre_all, pre_keep = None, 0, None
         if isinstance(pre_chance_node, torch.Tensor):
             pre_keep = pre_chance_node.to(device=dev, dtype=torch.uint8).contiguous()
-            assert pre_keep.shape == (m,)
+            _req(pre_keep.shape == (m,), "pre_keep.shape == (m,)")
             pre_ptr = _lib.ptr(pre_keep)
         elif pre_chance_node is not None:
             pre_all = int(bool(pre_chance_node))

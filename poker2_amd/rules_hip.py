@@ -14,6 +14,7 @@ import torch
 
 from . import _lib
 from ._lib import hip_is_available
+from ._guards import require as _req
 
 NUM_HANDS = 1326
 
@@ -100,8 +101,8 @@ def create_comparison_vector(ab_batch: torch.Tensor) -> torch.Tensor:
 
 def compare_7(a_cards, b_cards) -> int:
     """Two lists of 7 card ids -> 1 / -1 / 0 (src/p2/env/rules.py:358-387)."""
-    assert len(a_cards) == 7, f"Expected 7 cards for hand A, got {len(a_cards)}"
-    assert len(b_cards) == 7, f"Expected 7 cards for hand B, got {len(b_cards)}"
+    _req(len(a_cards) == 7, f"Expected 7 cards for hand A, got {len(a_cards)}")
+    _req(len(b_cards) == 7, f"Expected 7 cards for hand B, got {len(b_cards)}")
     planes = torch.zeros(1, 2, 4, 13, dtype=torch.bool)
     for p, cards in enumerate((a_cards, b_cards)):
         for card in cards:
@@ -111,17 +112,17 @@ def compare_7(a_cards, b_cards) -> int:
 
 def compare_7_single_batch(ab_batch: torch.Tensor) -> torch.Tensor:
     """rules.py:390-409 on the GPU: bool planes only; the flush suit is the fullest suit."""
-    assert ab_batch.dim() == 4
-    assert tuple(ab_batch.shape[1:]) == (2, 4, 13)
-    assert ab_batch.dtype == torch.bool
+    _req(ab_batch.dim() == 4, "ab_batch.dim() == 4")
+    _req(tuple(ab_batch.shape[1:]) == (2, 4, 13), "tuple(ab_batch.shape[1:]) == (2, 4, 13)")
+    _req(ab_batch.dtype == torch.bool, "ab_batch.dtype == torch.bool")
     return _compare_planes(ab_batch, 0)
 
 
 def compare_7_batches(a_batch: torch.Tensor, b_batch: torch.Tensor) -> torch.Tensor:
     """rules.py:412-426 on the GPU."""
-    assert a_batch.shape == b_batch.shape
-    assert a_batch.dim() == 3
-    assert tuple(a_batch.shape[1:]) == (4, 13)
+    _req(a_batch.shape == b_batch.shape, "a_batch.shape == b_batch.shape")
+    _req(a_batch.dim() == 3, "a_batch.dim() == 3")
+    _req(tuple(a_batch.shape[1:]) == (4, 13), "tuple(a_batch.shape[1:]) == (4, 13)")
     return compare_7_single_batch(torch.stack([a_batch, b_batch], dim=1).bool())
 
 
@@ -229,16 +230,17 @@ def showdown_value_both(beliefs: torch.Tensor, tables: torch.Tensor, potential: 
     beliefs = beliefs.contiguous().float()
     potential = potential.to(device=beliefs.device, dtype=torch.float32).contiguous()
     scale = scale.to(device=beliefs.device, dtype=torch.float32).contiguous()
-    assert potential.shape == (m, 2) and scale.shape == (m,)
-    assert tables.is_contiguous() and tables.dtype == torch.uint8 and tables.shape[1] == showdown_table_bytes()
+    _req(potential.shape == (m, 2) and scale.shape == (m,), "potential.shape == (m, 2) and scale.shape == (m,)")
+    _req(tables.is_contiguous() and tables.dtype == torch.uint8 and tables.shape[1] == showdown_table_bytes(),
+         "tables.is_contiguous() and tables.dtype == torch.uint8 and tables.shape[1] == showdown_table_bytes()")
     if table_row is not None:
         table_row = table_row.to(torch.int64).contiguous()
-        assert table_row.shape == (m,)
+        _req(table_row.shape == (m,), "table_row.shape == (m,)")
     else:
-        assert tables.shape[0] == m
+        _req(tables.shape[0] == m, "tables.shape[0] == m")
     if out is None:
         out = torch.empty_like(beliefs)
-    assert out.is_contiguous() and out.shape == beliefs.shape
+    _req(out.is_contiguous() and out.shape == beliefs.shape, "out.is_contiguous() and out.shape == beliefs.shape")
     _lib.call("p2hip_showdown_both", _lib.ptr(beliefs), _lib.ptr(tables), _lib.ptr(table_row),
               _lib.ptr(potential), _lib.ptr(scale), m, _lib.ptr(out), _lib.stream_ptr())
     return out

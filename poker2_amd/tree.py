@@ -21,6 +21,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 
 import numpy as np
+from ._guards import require as _req
 
 H = 1326
 
@@ -53,7 +54,7 @@ class RootStates:
             self.done = np.zeros(self.street.shape[0], dtype=bool)
         if self.runout is not None:
             shown = np.arange(5)[None, :] < CARDS_ON_STREET[np.clip(self.street, 0, 4)][:, None]
-            assert np.array_equal(np.where(shown, self.runout, -1), self.board), "runout does not continue the board"
+            _req(np.array_equal(np.where(shown, self.runout, -1), self.board), "runout does not continue the board")
 
     def previous_board(self) -> np.ndarray:
         """The env's ``last_board_indices`` (src/p2/env/hunl_tensor_env.py:862): every action saves the
@@ -272,7 +273,7 @@ def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
     """Breadth-first expansion to ``depth`` plies.  Below the root level a node whose betting
     round has just closed (``actions_this_round == 0``, which includes showdowns) is not
     expanded (sparse_cfr_evaluator.py:167-197)."""
-    assert roots.n > 0, "must supply at least one root state"
+    _req(roots.n > 0, "must supply at least one root state")
     bins = [float(b) for b in bet_bins]
     nb = len(bins) + 3
     n = roots.n
@@ -312,8 +313,9 @@ def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
     leaf[offsets[-2]:] = True
     child_mask = legal & ~leaf[:, None]
     child_count = child_mask.sum(axis=1).astype(np.int64)
-    assert total == n + int(child_count.sum())
-    assert (child_count[~leaf] > 0).all() and not leaf[:n].any()
+    _req(total == n + int(child_count.sum()), "total == n + int(child_count.sum())")
+    _req((child_count[~leaf] > 0).all() and not leaf[:n].any(),
+         "(child_count[~leaf] > 0).all() and not leaf[:n].any()")
     child_offsets = (offsets[1] + np.cumsum(child_count) - child_count).astype(np.int64)
     prev_actor = np.full(total, -1, dtype=np.int64)
     prev_actor[n:] = state["to_act"][parent_index[n:]]
@@ -350,7 +352,7 @@ def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: in
     from . import _lib
     if not _lib.hip_is_available():
         raise RuntimeError("build_sparse_tree_device needs libp2hip.so and a GPU; use build_sparse_tree on the host.")
-    assert roots.n > 0, "must supply at least one root state"
+    _req(roots.n > 0, "must supply at least one root state")
     bins = [float(b) for b in bet_bins]
     if len(bins) > 5:
         raise ValueError("at most 5 bet fractions (8 action bins) are supported")
@@ -358,7 +360,7 @@ def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: in
     n = roots.n
     dev = torch.device(device)
     cols = int(_lib.load().p2hip_tree_node_columns())
-    assert cols == len(_DEVICE_COLS)
+    _req(cols == len(_DEVICE_COLS), "cols == len(_DEVICE_COLS)")
     host = np.zeros((n, cols), dtype=np.int64)
     col = {name: i for i, name in enumerate(_DEVICE_COLS)}
     for name in ("street", "to_act", "button", "pot", "min_raise", "actions_this_round", "done"):
@@ -429,7 +431,7 @@ def build_sparse_tree_device(roots: RootStates, bet_bins: list[float], depth: in
     leaf = state["done"] | new_street
     leaf[offsets[-2]:] = True
     cc = child_count.cpu().numpy()
-    assert total == n + int(cc.sum())
+    _req(total == n + int(cc.sum()), "total == n + int(cc.sum())")
     prev_actor = np.full(total, -1, dtype=np.int64)
     prev_actor[n:] = state["to_act"][parent_index[n:]]
     tree = SparseTree(depth_offsets=list(offsets), n_roots=n, total=total, num_actions=nb, bet_bins=bins,

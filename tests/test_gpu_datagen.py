@@ -211,7 +211,7 @@ def test_training_data_matches_oracle_everywhere(golden_dir, name):
     """Against the oracle following the one-kernel evaluator's conventions: every entry, blocked
     hands included."""
     from tests.test_gpu_evaluator import tree_as_dict
-    case, cols = load_case(golden_dir, name)
+    case, _ = load_case(golden_dir, name)
     ev, r = golden_evaluator(case, True)
     tree = tree_as_dict(ev.tree)
     tree.update({k: v for k, v in ev.tree.state.items() if k not in tree})
@@ -388,7 +388,6 @@ def test_leaf_model_does_not_reuse_features_of_the_previous_subgame():
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.leaf_models import ChanceLeafModel, NetworkLeafModel, RangeBoardMLP
     from poker2_amd.tree import RootStates
-    rng = np.random.default_rng(60)
     n = 8
     beliefs = torch.full((n, 2, H), 1.0 / H)
 

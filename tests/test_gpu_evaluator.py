@@ -267,7 +267,7 @@ def test_sample_leaves_walks_the_sampled_policy():
     assert torch.equal(out.beliefs, ev.beliefs[out.nodes])
     np.testing.assert_array_equal(out.roots.pot, tree.state["pot"][rows])
     # deterministic sampled policy: always the LAST non-terminal action, no exploration
-    top, bottom = ev.depth_offsets[-2], ev.depth_offsets[1]
+    top = ev.depth_offsets[-2]
     ev.policy_probs_sample.zero_()
     target = np.zeros(ev.total_nodes, dtype=bool)
     for p in range(top):

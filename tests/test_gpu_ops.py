@@ -323,3 +323,41 @@ def test_unblocked_mass_grid_stride_ragged_and_empty(F):
     empty = torch.zeros(0, H, device="cuda")
     assert F.unblocked_mass_triton(empty).shape == (0, H)
     assert F.unblocked_mass_ratio_triton(empty, empty).shape == (0, H)
+
+
+def test_wrappers_refuse_arguments_that_would_index_out_of_bounds(F):
+    """Sizes, dtypes and row bounds the kernels index with are checked on the host (and stay
+    checked under ``python -O``): none of these calls may reach the GPU."""
+    rng = np.random.default_rng(77)
+    tr = random_tree(rng, 3, 2)
+    total, top, bottom = tr["total"], tr["top"], tr["bottom"]
+    reach = torch.ones(total, 2, H, device="cuda")
+    policy = torch.rand(total, H, device="cuda")
+    allowed = torch.ones(total, H, dtype=torch.bool, device="cuda")
+    pidx, pa, to_act = dev(tr["parent_index"]), dev(tr["prev_actor"]), dev(tr["to_act"])
+    co, cc = dev(tr["child_offsets"][:top].copy()), dev(tr["child_count"][:top].copy())
+    one = torch.ones((), device="cuda")
+    bad = [
+        lambda: F.fused_reach_weights_depth_(reach, policy, allowed, pidx.int(), pa, bottom, total),     # int32 indices
+        lambda: F.fused_reach_weights_depth_(reach, policy, allowed, pidx, pa, bottom, total + 5),       # rows past the end
+        lambda: F.fused_reach_weights_depth_(reach.double(), policy, allowed, pidx, pa, bottom, total),  # not fp32
+        lambda: F.fused_regret_tail_(torch.zeros(total, H, device="cuda"), reach, policy[:top].contiguous(),
+                                     policy[:top].contiguous(), pidx, pa, total + 1),
+        lambda: F.unblocked_mass_opp_at_parents_triton(reach, to_act, total + 1),
+        lambda: F.fused_dcfr_update_with_tensors_(policy, policy[:-1].contiguous(), policy.clone(), one, one, one, one,
+                                                  True, False),
+        lambda: F.fused_update_average_values_with_tensors_(reach, reach[:-1].contiguous(), one, one, one),
+        lambda: F.fused_update_average_values_with_tensors_(reach.half(), reach.half(), one, one, one),
+        lambda: F.fused_sibling_sum(policy, co, cc, bottom, total - bottom + 10),
+        lambda: F.fused_weighted_parent_sum(reach, pa, policy, policy, co, cc, total),
+        lambda: F.fused_average_policy_mix_with_tensors_(policy, policy.clone(), reach, reach[:-1].contiguous(), to_act,
+                                                         pidx, one, one, one, bottom),
+        lambda: F.fused_deep_beliefs_(reach, reach, reach.clone(), policy, dev(tr["root_index"]).int(), bottom),
+        lambda: F.fused_sample_snapshot_(policy, policy.clone(), to_act[:-1].contiguous(), torch.zeros((), dtype=torch.long,
+                                                                                                      device="cuda")),
+    ]
+    for i, call in enumerate(bad):
+        with pytest.raises(AssertionError):
+            call()
+            pytest.fail(f"call {i} was not refused")
+    torch.cuda.synchronize()

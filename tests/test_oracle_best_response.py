@@ -60,10 +60,10 @@ def test_best_response_values_match_exact_best_response(depth):
 
 
 def test_exploitability_of_a_solved_game_is_small_and_of_uniform_play_large():
-    board, hands0, hands1, p0, p1, t, bel = tiny_setup(2)
+    board, _, _, _, _, t, bel = tiny_setup(2)
     o = OCFR.OracleCFR(t, board[None], bel, cfr_iterations=300, use_final_policy_values=False)
     o.prepare()
-    expl0, br0 = OBR.compute_exploitability(o)          # uniform average policy
+    expl0, _ = OBR.compute_exploitability(o)          # uniform average policy
     for it in range(300):
         o.cfr_iteration(it)
     expl, br = OBR.compute_exploitability(o)
