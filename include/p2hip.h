@@ -61,6 +61,14 @@ int64_t p2hip_showdown_table_bytes(void);
 int p2hip_showdown_setup(const void* boards, int elem_size, int64_t m, int mode, int32_t* ranks_out,
                          int64_t* order_out, uint8_t* table_out, void* stream);
 
+/* The same table from hands that are already in strength order, without a board: per row and
+ * sorted position the hand's two cards c1_sorted, c2_sorted [m,H] int32 and its tie group
+ * [L_idx, R_idx) [m,H] int32 -- the inputs of showdown_ev_triton, search/fused_cfr_triton.py:2271-2314.
+ * bad [m] int32 receives 1 for a row that does not list each of the 1326 hands once with
+ * 0 <= L <= k < R <= H (its table is filled with in-range values but means nothing), else 0. */
+int p2hip_showdown_setup_sorted(const int32_t* c1_sorted, const int32_t* c2_sorted, const int32_t* L_idx,
+                                const int32_t* R_idx, int64_t m, uint8_t* table_out, int32_t* bad, void* stream);
+
 /* beliefs [m,2,H] -> out [m,2,H]: blocker-corrected showdown EV of both players per hand,
  * times potential[m,p] / scale[m].  table_row [m] (or NULL = identity) selects the board
  * table of each node.  Replaces _showdown_value_both / _showdown_value,

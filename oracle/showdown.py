@@ -20,7 +20,9 @@ is what torch's CPU cumsum does for float32 input.
 
 Pinned by: brute force over all hero x villain pairs (several boards from the
 reference's tests), all-tie board -> 0, delta villain -> +-potential,
-zero-sum identity over compatible pairs, |EV| <= potential/scale.  The formula takes
+zero-sum identity over compatible pairs, |EV| <= potential/scale; and by outputs of the
+reference's own ``showdown_ev_triton`` kernel (fused_cfr_triton.py:2162-2314) run under Triton's
+CPU interpreter (tests/golden/fused_ops_golden.npz, case ``showdown_sorted``).  The formula takes
 the villain range as normalised and zero on board-blocked hands (the constant 1 in
 ``den``), as the evaluator guarantees; it is not invariant to rescaling the range.
 """

@@ -55,6 +55,31 @@ __device__ void bitonic_sort_2048(unsigned long long* keys) {
   __syncthreads();
 }
 
+// Per-card lists: clist[c][j] = sorted position of the j-th weakest of the 51 combos holding card
+// c, found by counting how many of the other 50 lie below (positions are distinct).  Ends with a
+// barrier.
+__device__ __forceinline__ void fill_card_lists(const uint16_t* pos_of, uint16_t (*clist)[52]) {
+  for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) {
+    const int c = e / 51, j = e % 51;
+    const int x = j < c ? j : j + 1;
+    const int mine = pos_of[p2_combo_index(x < c ? x : c, x < c ? c : x)];
+    int below = 0;
+    for (int jj = 0; jj < 51; ++jj) {
+      const int y = jj < c ? jj : jj + 1;
+      below += pos_of[p2_combo_index(y < c ? y : c, y < c ? c : y)] < mine ? 1 : 0;
+    }
+    clist[c][below] = (uint16_t)mine;
+  }
+  __syncthreads();
+}
+
+// How many entries of one card's list lie strictly below sorted position `bound`.
+__device__ __forceinline__ int card_list_below(const uint16_t* list51, int bound) {
+  int lo = 0, hi = 51;
+  while (lo < hi) { const int mid = (lo + hi) >> 1; if ((int)list51[mid] < bound) lo = mid + 1; else hi = mid; }
+  return lo;
+}
+
 template <typename T>
 __device__ __forceinline__ int board_card(const void* boards, int64_t m, int j) {
   return (int)reinterpret_cast<const T*>(boards)[m * 5 + j];
@@ -158,20 +183,7 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_setup_kernel(const void* __
   uint16_t* t_perm = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_PERM);
   uint16_t* t_lr = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_LR);
 
-  // per-card lists: position of each of the 51 combos of card c, sorted ascending by
-  // counting how many of the other 50 lie below (positions are distinct)
-  for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) {
-    const int c = e / 51, j = e % 51;
-    const int x = j < c ? j : j + 1;
-    const int mine = pos_of[p2_combo_index(x < c ? x : c, x < c ? c : x)];
-    int below = 0;
-    for (int jj = 0; jj < 51; ++jj) {
-      const int y = jj < c ? jj : jj + 1;
-      below += pos_of[p2_combo_index(y < c ? y : c, y < c ? c : y)] < mine ? 1 : 0;
-    }
-    clist[c][below] = (uint16_t)mine;
-  }
-  __syncthreads();
+  fill_card_lists(pos_of, clist);
   uint16_t* t_clist = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_CLIST);
   for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) {
     const int c = e / 51, j = e % 51;
@@ -195,21 +207,72 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_setup_kernel(const void* __
     t_perm[k] = (uint16_t)(h | (blocked ? 0x8000 : 0));
     t_lr[2 * k] = (uint16_t)L;
     t_lr[2 * k + 1] = (uint16_t)R;
-    int cnt[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int c = q < 2 ? a : b;
-      const int bound = (q & 1) ? R : L;
-      int n = 0;  // entries of card c's list strictly below `bound`
-      int l2 = 0, h2 = 51;
-      while (l2 < h2) { int mid = (l2 + h2) >> 1; if ((int)clist[c][mid] < bound) l2 = mid + 1; else h2 = mid; }
-      n = l2;
-      cnt[q] = n;
+    t_cidx[4 * k + 0] = (uint8_t)card_list_below(clist[a], L);
+    t_cidx[4 * k + 1] = (uint8_t)card_list_below(clist[a], R);
+    t_cidx[4 * k + 2] = (uint8_t)card_list_below(clist[b], L);
+    t_cidx[4 * k + 3] = (uint8_t)card_list_below(clist[b], R);
+  }
+}
+
+// The same table from hands that are ALREADY in strength order: row m lists, per sorted position,
+// the two cards of the hand (any order) and its tie group [L, R).  No board is involved, so no
+// combo is flagged as blocked and no card list is masked.  The rows must list each of the 1326
+// combos once; `bad[m]` is set to 1 otherwise (a card outside 0..51, a repeated combo, or a tie
+// group outside 0 <= L <= k < R <= 1326) and the row's table must not be used.
+__global__ __launch_bounds__(SD_BLOCK) void showdown_setup_sorted_kernel(const int32_t* __restrict__ c1,
+                                                                          const int32_t* __restrict__ c2,
+                                                                          const int32_t* __restrict__ L_idx,
+                                                                          const int32_t* __restrict__ R_idx,
+                                                                          uint8_t* __restrict__ table_out,
+                                                                          int32_t* __restrict__ bad) {
+  __shared__ uint16_t pos_of[P2_H];
+  __shared__ uint16_t clist[P2_CARDS][52];
+  __shared__ int n_bad;
+  const int64_t m = blockIdx.x;
+  if (threadIdx.x == 0) n_bad = 0;
+  for (int h = threadIdx.x; h < P2_H; h += SD_BLOCK) pos_of[h] = 0xFFFFu;
+  __syncthreads();
+  uint16_t* t_perm = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_PERM);
+  uint16_t* t_lr = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_LR);
+  int wrong = 0;
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const int x = c1[m * P2_H + k], y = c2[m * P2_H + k];
+    const int L = L_idx[m * P2_H + k], R = R_idx[m * P2_H + k];
+    const bool ok = (uint32_t)x < 52u && (uint32_t)y < 52u && x != y && L >= 0 && L <= k && R > k && R <= P2_H;
+    int h = 0;
+    if (ok) {
+      h = p2_combo_index(x < y ? x : y, x < y ? y : x);
+      pos_of[h] = (uint16_t)k;      // a repeated combo leaves another one at 0xFFFF: counted below
+    } else {
+      wrong = 1;
     }
-    t_cidx[4 * k + 0] = (uint8_t)cnt[0];
-    t_cidx[4 * k + 1] = (uint8_t)cnt[1];
-    t_cidx[4 * k + 2] = (uint8_t)cnt[2];
-    t_cidx[4 * k + 3] = (uint8_t)cnt[3];
+    t_perm[k] = (uint16_t)h;
+    t_lr[2 * k] = (uint16_t)(ok ? L : k);
+    t_lr[2 * k + 1] = (uint16_t)(ok ? R : k + 1);
+  }
+  __syncthreads();
+  for (int h = threadIdx.x; h < P2_H; h += SD_BLOCK) wrong |= pos_of[h] == 0xFFFFu ? 1 : 0;
+  if (wrong) atomicOr(&n_bad, 1);
+  __syncthreads();
+  if (n_bad) {                     // uniform: leave the row unusable but every table byte defined and in range
+    if (threadIdx.x == 0) bad[m] = 1;
+    for (int h = threadIdx.x; h < P2_H; h += SD_BLOCK) pos_of[h] = (uint16_t)h;
+    __syncthreads();
+  } else if (threadIdx.x == 0) {
+    bad[m] = 0;
+  }
+  fill_card_lists(pos_of, clist);
+  uint16_t* t_clist = reinterpret_cast<uint16_t*>(table_out + m * SD_TABLE_BYTES + SD_OFF_CLIST);
+  for (int e = threadIdx.x; e < P2_CARDS * 51; e += SD_BLOCK) t_clist[e] = clist[e / 51][e % 51];
+  uint8_t* t_cidx = table_out + m * SD_TABLE_BYTES + SD_OFF_CIDX;
+  for (int k = threadIdx.x; k < P2_H; k += SD_BLOCK) {
+    const int h = t_perm[k];
+    const int a = p2_combo.a[h], b = p2_combo.b[h];
+    const int L = t_lr[2 * k], R = t_lr[2 * k + 1];
+    t_cidx[4 * k + 0] = (uint8_t)card_list_below(clist[a], L);
+    t_cidx[4 * k + 1] = (uint8_t)card_list_below(clist[a], R);
+    t_cidx[4 * k + 2] = (uint8_t)card_list_below(clist[b], L);
+    t_cidx[4 * k + 3] = (uint8_t)card_list_below(clist[b], R);
   }
 }
 
@@ -447,6 +510,20 @@ int p2hip_showdown_setup(const void* boards, int elem_size, int64_t m, int mode,
   if (table_out && !p2_aligned8(table_out)) return P2_EINVAL;
   hipLaunchKernelGGL(p2::showdown_setup_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
                      boards, elem_size, mode, ranks_out, order_out, table_out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_showdown_setup_sorted(const int32_t* c1_sorted, const int32_t* c2_sorted, const int32_t* L_idx,
+                                const int32_t* R_idx, int64_t m, uint8_t* table_out, int32_t* bad, void* stream) {
+  if (m < 0 || m > 0x7FFFFFFF) return P2_EINVAL;
+  if (m == 0) return 0;
+  if (!c1_sorted || !c2_sorted || !L_idx || !R_idx || !table_out || !bad) return P2_EINVAL;
+  if (!p2_aligned8(table_out) || !p2_aligned4(c1_sorted) || !p2_aligned4(c2_sorted) || !p2_aligned4(L_idx) ||
+      !p2_aligned4(R_idx) || !p2_aligned4(bad))
+    return P2_EINVAL;
+  hipLaunchKernelGGL(p2::showdown_setup_sorted_kernel, dim3((unsigned)m), dim3(p2::SD_BLOCK), 0, (hipStream_t)stream,
+                     c1_sorted, c2_sorted, L_idx, R_idx, table_out, bad);
   P2_LAUNCH_CHECK();
   return 0;
 }

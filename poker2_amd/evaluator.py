@@ -941,6 +941,36 @@ class HipSparseCFREvaluator:
         return {n: getattr(self, n) for n in STATE_NAMES}
 
 
+class _EvaluatorStateSnapshot:
+    """Copies of the 11 tensors an iteration mutates, to rewind an evaluator or to compare two
+    runs (the helper the reference keeps beside its graph runner, fused_cfr_triton.py:2322-2356:
+    ``from_evaluator``, ``restore_to``, ``max_abs_diff``, fields ``names`` and ``tensors``)."""
+
+    def __init__(self, saved: dict) -> None:
+        self._saved = dict(saved)
+
+    @property
+    def names(self) -> tuple:
+        return tuple(self._saved)
+
+    @property
+    def tensors(self) -> tuple:
+        return tuple(self._saved.values())
+
+    @classmethod
+    def from_evaluator(cls, evaluator) -> "_EvaluatorStateSnapshot":
+        return cls({name: getattr(evaluator, name).detach().clone() for name in STATE_NAMES})
+
+    def restore_to(self, evaluator) -> None:
+        for name, kept in self._saved.items():
+            getattr(evaluator, name).copy_(kept)
+
+    def max_abs_diff(self, other: "_EvaluatorStateSnapshot") -> dict:
+        _req(self.names == other.names, "snapshots hold different tensors")
+        return {name: (mine - theirs).abs().max().item()
+                for (name, mine), theirs in zip(self._saved.items(), other.tensors)}
+
+
 class GraphedCFRIteration:
     """Captures ``evaluator.cfr_iteration`` into a HIP graph and replays it for any ``t``
     (src/p2/search/fused_cfr_triton.py:2359-2451).  The iteration-dependent scalars live in

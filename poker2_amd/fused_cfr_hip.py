@@ -560,6 +560,45 @@ def fused_deep_beliefs_(out, root_beliefs, reach_weights, allowed_prob, root_ind
               int(n), total, float(eps), _S())
 
 
+def showdown_ev_triton(b_opp_sorted, c1_sorted, c2_sorted, L_idx, R_idx, eps: float = 1e-8, block_k: int = 32,
+                       block_j: int = 128) -> torch.Tensor:
+    """Showdown EV per hand, in strength order, from strength-sorted inputs: the villain range
+    ``b_opp_sorted`` [M, 1326], the two cards of each sorted hand and its tie group [L, R)
+    (fused_cfr_triton.py:2271-2314; un-sorting, the board mask and potential / scale stay with the
+    caller, as there).  Each row must list every one of the 1326 hands once.  Runs the same kernels
+    as the evaluator's showdown: a table is built from the sorted hands, then both prefix passes."""
+    _need()
+    from . import rules_hip
+    _req(b_opp_sorted.is_contiguous() and b_opp_sorted.dim() == 2, "b_opp_sorted must be contiguous [M, H]")
+    m, h = b_opp_sorted.shape
+    _req(h == _H, "b_opp_sorted.shape[1] == 1326")
+    _req(c1_sorted.shape == (m, h) and c2_sorted.shape == (m, h), "c1_sorted / c2_sorted must be [M, H]")
+    _req(L_idx.shape == (m, h) and R_idx.shape == (m, h), "L_idx / R_idx must be [M, H]")
+    _f32(b_opp_sorted=b_opp_sorted)
+    if float(eps) != 1e-8:
+        raise NotImplementedError("the showdown kernels are built for eps = 1e-8, the evaluator's value")
+    dev = b_opp_sorted.device
+    if m == 0:
+        return torch.empty(0, h, device=dev, dtype=torch.float32)
+    c1 = c1_sorted.to(device=dev, dtype=torch.int32).contiguous()
+    c2 = c2_sorted.to(device=dev, dtype=torch.int32).contiguous()
+    lo_idx = L_idx.to(device=dev, dtype=torch.int32).contiguous()
+    hi_idx = R_idx.to(device=dev, dtype=torch.int32).contiguous()
+    tables = torch.empty(m, rules_hip.showdown_table_bytes(), dtype=torch.uint8, device=dev)
+    bad = torch.empty(m, dtype=torch.int32, device=dev)
+    _lib.call("p2hip_showdown_setup_sorted", _p(c1), _p(c2), _p(lo_idx), _p(hi_idx), m, _p(tables), _p(bad), _S())
+    if bool(bad.any()):
+        rows = torch.nonzero(bad).flatten().tolist()[:8]
+        raise ValueError(f"rows {rows} do not list each of the 1326 hands once with a tie group 0 <= L <= k < R <= 1326")
+    lo, hi = torch.minimum(c1, c2).long(), torch.maximum(c1, c2).long()
+    combo = lo * (103 - lo) // 2 + (hi - lo - 1)                       # index of (lo, hi) among the 1326 hands
+    beliefs = torch.zeros(m, 2, h, device=dev, dtype=torch.float32)
+    beliefs[:, 1].scatter_(1, combo, b_opp_sorted)                      # hero 0 faces this range
+    ones = torch.ones(m, 2, device=dev, dtype=torch.float32)
+    ev = rules_hip.showdown_value_both(beliefs, tables, ones, ones[:, 0].contiguous())
+    return ev[:, 0].gather(1, combo)
+
+
 def fused_sample_snapshot_(policy_probs_sample, policy_probs, t_sample, t_tensor) -> None:
     """policy_probs_sample <- where(t_sample == t, policy_probs, policy_probs_sample)
     (fused_sparse_cfr_evaluator.py:494-499); ``t_tensor`` is a 0-D int64 device tensor."""
@@ -638,9 +677,9 @@ class ParentBeliefUnblockedStats:
 
 
 def __getattr__(name):
-    # GraphedCFRIteration lives with the evaluator (which imports this module); the reference
-    # exports it from fused_cfr_triton.py:2359-2451
-    if name == "GraphedCFRIteration":
-        from .evaluator import GraphedCFRIteration
-        return GraphedCFRIteration
+    # The graph runner and the state snapshot live with the evaluator (which imports this module);
+    # the reference exports both from fused_cfr_triton.py:2322-2451
+    if name in ("GraphedCFRIteration", "_EvaluatorStateSnapshot"):
+        from . import evaluator
+        return getattr(evaluator, name)
     raise AttributeError(name)

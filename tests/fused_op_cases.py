@@ -90,6 +90,22 @@ def inputs(name: str) -> dict:
         pidx = rng.integers(0, top, nchild).astype(np.int64)
         return dict(beliefs=r(total, 2, H), to_act=rng.integers(0, 2, total).astype(np.int64), top=top, actor=actor,
                     pidx=pidx, numer=(actor[pidx] * r(nchild, H)).astype(F32))
+    if name == "showdown_sorted":
+        # the boards of the reference's showdown scenarios (tests/test_rebel_cfr_evaluator.py:1220-1537:
+        # "Ac Qh 9d 7s 4h", the royal board where every hand ties, a paired board) and two drawn ones
+        from oracle import cards as OC
+        from oracle import showdown as OS
+        card = lambda txt: "23456789TJQKA".index(txt[0]) + 13 * "cdhs".index(txt[1])    # noqa: E731
+        boards = [[card(c) for c in b.split()] for b in ("Ac Qh 9d 7s 4h", "Ah Kh Qh Jh Th", "Tc Th Ts 7d 7h")]
+        boards += [rng.permutation(52)[:5].tolist() for _ in range(2)]
+        boards = np.asarray(boards, dtype=np.int64)
+        allowed = OC.allowed_hands_for_boards(boards)[0]
+        hrd = OS.init_hand_rank_data(boards, allowed)
+        bel = rng.gamma(0.5, size=(len(boards), 2, H)).astype(F32) * allowed[:, None, :]
+        bel[4, 1, :] = 0.0
+        bel[4, 1, np.nonzero(allowed[4])[0][:3]] = 1.0          # a villain range of three hands
+        bel = _norm(bel)
+        return dict(boards=boards, allowed=allowed, beliefs=bel, hrd=hrd)
     raise KeyError(name)
 
 
@@ -97,7 +113,7 @@ NAMES = ("dcfr_update_t0", "dcfr_update_t7", "dcfr_update_t50_plus", "dcfr_updat
          "block_normalize_2d", "regret_matching_divide", "weight_child_values", "update_average_values",
          "avg_values_zero_sum", "avg_values_zero_sum_ignore", "avg_values_zero_sum_off", "regret_tail",
          "average_policy_mix", "parent_sibling_divide", "model_values_mix", "weighted_parent_sum",
-         "reach_and_deep_beliefs", "unblocked_mass", "unblocked_opp_and_ratio")
+         "reach_and_deep_beliefs", "unblocked_mass", "unblocked_opp_and_ratio", "showdown_sorted")
 
 
 def hash_name(name: str) -> int:
@@ -172,6 +188,11 @@ def oracle_ops(name: str, x: dict) -> dict:
         opp = OU.calculate_unblocked_mass(x["beliefs"][np.arange(top), 1 - x["to_act"][:top]])
         ratio = OU.unblocked_mass_ratio(x["numer"], x["actor"], 1e-5, x["pidx"])
         return dict(opp_at_parents=opp, ratio_indirect=ratio, ratio=ratio)
+    if name == "showdown_sorted":
+        from oracle import showdown as OS
+        m = len(x["boards"])
+        ones = np.ones((m, 2), F32)
+        return {f"ev_hero{p}": OS.showdown_value(x["beliefs"], p, x["hrd"], ones, ones[:, 0]) for p in (0, 1)}
     raise KeyError(name)
 
 
@@ -287,4 +308,16 @@ def torch_ops(name: str, x: dict, F, device, raw=None) -> dict:
         numer, actor, pidx = T(x["numer"]), T(x["actor"]), T(x["pidx"])
         return dict(opp_at_parents=opp, ratio_indirect=F.unblocked_mass_ratio_indirect_triton(numer, actor, pidx),
                     ratio=F.unblocked_mass_ratio_triton(numer, actor[pidx].contiguous()))
+    if name == "showdown_sorted":
+        # EV per hand in combo order with potential = scale = 1: the reference's kernel works on the
+        # strength-sorted villain range and leaves un-sorting and the board mask to its caller
+        hrd, out = x["hrd"], {}
+        order, inv = T(hrd.sorted_indices), T(hrd.inv_sorted)
+        c1, c2 = T(hrd.hands_c1c2_sorted[..., 0].copy()), T(hrd.hands_c1c2_sorted[..., 1].copy())
+        ok = T(x["allowed"]).float()
+        for p in (0, 1):
+            b_sorted = torch.gather(T(x["beliefs"][:, 1 - p]), 1, order).contiguous()
+            ev_sorted = F.showdown_ev_triton(b_sorted, c1, c2, T(hrd.L_idx), T(hrd.R_idx))
+            out[f"ev_hero{p}"] = torch.gather(ev_sorted, 1, inv) * ok
+        return out
     raise KeyError(name)

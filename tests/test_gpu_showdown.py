@@ -132,3 +132,45 @@ def test_empty(K):
     out = K.showdown_value_both(torch.zeros(0, 2, H, device="cuda"), tables, torch.zeros(0, 2, device="cuda"),
                                 torch.zeros(0, device="cuda"))
     assert out.shape == (0, 2, H)
+
+
+def test_ev_from_strength_sorted_inputs_matches_oracle_and_refuses_bad_rows():
+    """``showdown_ev_triton`` (fused_cfr_triton.py:2271-2314): the same EV from inputs that are
+    already in strength order; un-sorting, board mask and chips are the caller's."""
+    from poker2_amd import fused_cfr_hip as F
+    rng = np.random.default_rng(9)
+    boards = np.concatenate([NAMED_BOARDS, random_boards(rng, 9)])
+    m = boards.shape[0]
+    bel = random_ranges(rng, boards)
+    allowed, _ = OC.allowed_hands_for_boards(boards)
+    hrd = OS.init_hand_rank_data(boards, allowed)
+    ones = np.ones((m, 2), np.float32)
+    exp = OS.showdown_value(bel, 0, hrd, ones, ones[:, 0])                   # hero 0, potential = scale = 1
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()       # noqa: E731
+    order, inv = dev(hrd.sorted_indices), dev(hrd.inv_sorted)
+    c1, c2 = dev(hrd.hands_c1c2_sorted[..., 0]), dev(hrd.hands_c1c2_sorted[..., 1])          # int64, as the reference keeps them
+    b_sorted = torch.gather(dev(bel[:, 1]), 1, order).contiguous()
+    ev_sorted = F.showdown_ev_triton(b_sorted, c1, c2, dev(hrd.L_idx), dev(hrd.R_idx))
+    got = (torch.gather(ev_sorted, 1, inv) * dev(allowed).float()).cpu().numpy()
+    np.testing.assert_allclose(got, exp, rtol=RTOL, atol=ATOL)
+    # the two cards of a hand may come in either order
+    ev_swapped = F.showdown_ev_triton(b_sorted, c2, c1, dev(hrd.L_idx), dev(hrd.R_idx))
+    assert torch.equal(ev_swapped, ev_sorted)
+    assert F.showdown_ev_triton(b_sorted[:0].contiguous(), c1[:0], c2[:0], dev(hrd.L_idx)[:0], dev(hrd.R_idx)[:0]).shape == (0, H)
+    # rows that are no permutation of the 1326 hands, or whose tie groups do not hold their position
+    twice = c1.clone()
+    twice[3, 10], c2_twice = c1[3, 11], c2.clone()
+    c2_twice[3, 10] = c2[3, 11]
+    with pytest.raises(ValueError):
+        F.showdown_ev_triton(b_sorted, twice, c2_twice, dev(hrd.L_idx), dev(hrd.R_idx))
+    off = c1.clone()
+    off[0, 0] = 52
+    with pytest.raises(ValueError):
+        F.showdown_ev_triton(b_sorted, off, c2, dev(hrd.L_idx), dev(hrd.R_idx))
+    late = dev(hrd.L_idx).clone()
+    late[2, 100] = 101
+    with pytest.raises(ValueError):
+        F.showdown_ev_triton(b_sorted, c1, c2, late, dev(hrd.R_idx))
+    with pytest.raises(NotImplementedError):
+        F.showdown_ev_triton(b_sorted, c1, c2, dev(hrd.L_idx), dev(hrd.R_idx), eps=1e-6)
+    torch.cuda.synchronize()

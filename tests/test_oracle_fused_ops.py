@@ -3,7 +3,8 @@ oracle/unblocked.py) against outputs of the reference's own Triton kernels, run 
 CPU interpreter by tests/golden/gen_fused_ops_golden.py.  Inputs are rebuilt from the same seeds.
 
 Tolerance: 1e-5 relative (+1e-6 absolute) per element, the bound the path states for fp32; row
-sums (float64 sums of fp32 outputs) to 1e-5 of the row's absolute mass.
+sums (float64 sums of fp32 outputs) to 1e-5 of the row's absolute mass plus a fifth of the
+per-element absolute tolerance times the row length.
 """
 import os
 
@@ -31,8 +32,10 @@ def check_against_golden(golden, name, got):
         np.testing.assert_allclose(a[..., cols], want, rtol=RTOL, atol=ATOL, equal_nan=True, err_msg=f"{name}/{key}")
         mass = np.abs(a.astype(np.float64)).sum(-1)
         rs, want_rs = a.astype(np.float64).sum(-1), golden[f"{name}/{key}_rowsum"]
-        ok = np.isclose(rs, want_rs, rtol=0, atol=0) | (np.abs(rs - want_rs) <= 1e-5 * mass + 1e-6) | \
-            (np.isnan(rs) & np.isnan(want_rs))
+        # a sum of n entries that each agree to ATOL may differ by a fraction of n * ATOL (all-tie board: the
+        # reference's tiled sums leave ~1e-7 per hand where prefix sums give exact zeros)
+        slack = 1e-5 * mass + 1e-6 + 0.2 * ATOL * a.shape[-1]
+        ok = (np.abs(rs - want_rs) <= slack) | (np.isnan(rs) & np.isnan(want_rs))
         assert ok.all(), (name, key, np.abs(rs - want_rs).max())
 
 
