@@ -181,6 +181,23 @@ def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tens
     return out
 
 
+def _avg_over_perms(hand_values: torch.Tensor, perms: torch.Tensor) -> torch.Tensor:
+    """Mean over the rows of ``perms`` [P, 1326] of ``hand_values[..., perms[q]]`` for values of
+    any leading shape (chance_node_helper.py:17-27).  Runs ``perm_mean`` with a single flop of
+    weight 1; the rows are taken in pairs, which is only a launch shape here."""
+    _req(hand_values.shape[-1] == NUM_HANDS, "hand_values.shape[-1] == 1326")
+    lead = hand_values.shape[:-1]
+    rows = hand_values.reshape(-1, NUM_HANDS).float()
+    n = rows.shape[0]
+    if n == 0:
+        return rows.reshape(*lead, NUM_HANDS)
+    if n % 2:
+        rows = torch.cat([rows, rows.new_zeros(1, NUM_HANDS)])
+    one = torch.ones(1, dtype=torch.float32, device=rows.device)
+    mean = perm_mean(rows.view(-1, 1, 2, NUM_HANDS), perms, one)
+    return mean.view(-1, NUM_HANDS)[:n].reshape(*lead, NUM_HANDS)
+
+
 def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """``perm_mean`` over ALL 24 suit permutations: the orbit of a hand is its class of starting
     hands (pair / suited / offsuit of the same ranks), so the mean is taken per class."""

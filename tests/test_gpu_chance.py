@@ -256,6 +256,19 @@ def test_flop_expand_matches_oracle(K):
                          torch.zeros(0, 3, dtype=torch.long).cuda()).shape == (5, 0, 2, H)
 
 
+@pytest.mark.parametrize("lead", [(5,), (3, 2), (2, 3, 2), (0, 2)])
+def test_avg_over_perms_any_leading_shape(K, lead):
+    """The reference's ``_avg_over_perms`` (chance_node_helper.py:17-27) on values of any leading
+    shape, an odd number of rows included."""
+    rng = np.random.default_rng(31)
+    perms = OCH.combo_suit_perms()[rng.permutation(24)[:6]]
+    hv = rng.standard_normal(lead + (H,)).astype(np.float32)
+    exp = np.mean([hv[..., q] for q in perms], axis=0, dtype=np.float64) if hv.size else hv
+    got = K._avg_over_perms(torch.from_numpy(hv).cuda(), torch.from_numpy(perms).cuda())
+    assert got.shape == hv.shape
+    np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=2e-6)
+
+
 @pytest.mark.parametrize("n_perms", [1, 6, 24])
 def test_perm_mean_matches_numpy(K, n_perms):
     rng = np.random.default_rng(22 + n_perms)
