@@ -127,6 +127,11 @@ def side_metrics() -> dict:
     out["showdown_states_per_s"] = 4096 / (ms * 1e-3)
     out["showdown_ms_per_call_B4096"] = ms
     out["showdown_algorithmic_GBps"] = 4096 * 4 * H * 4 / (ms * 1e-3) / 1e9
+    # the per-board strength table is static input that every call re-reads; it is not algorithmic
+    # traffic and is stated apart
+    table = rules_hip.showdown_table_bytes()
+    out["showdown_table_bytes_per_state"] = table
+    out["showdown_GBps_with_tables"] = 4096 * (4 * H * 4 + table) / (ms * 1e-3) / 1e9
     rng = np.random.default_rng(7)
     cards = torch.from_numpy(np.argsort(rng.random((1 << 20, 52)), axis=1)[:, :7].astype(np.int8)).cuda()
     for _ in range(5):
