@@ -83,9 +83,10 @@ def cpu_baseline(tree: str, seed: int, budget_s: float = 20.0) -> dict:
     d["showdown_potential"] = t.showdown_potential
     orc = ocfr.OracleCFR(d, boards, beliefs, cfr_iterations=200)
     orc.prepare()
-    orc.cfr_iteration(0)  # warm-up
+    orc.cfr_iteration(0)  # two warm-up iterations
+    orc.cfr_iteration(1)
     times = []
-    t_it = 1
+    t_it = 2
     start = time.perf_counter()
     while time.perf_counter() - start < budget_s and len(times) < 40:
         t0 = time.perf_counter()
