@@ -76,3 +76,34 @@ def test_wrappers_fail_loudly_without_gpu():
     helper = CH.ChanceNodeHelper(torch.device("cpu"), torch.float32, 2, model=None, autocast_dtype=None)
     with pytest.raises((RuntimeError, ValueError)):
         helper.flop_chance_values(torch.zeros(1, dtype=torch.long), None, z)
+
+
+def test_argument_guards_hold_under_python_O():
+    """The wrappers' argument checks are what keeps a wrong shape from becoming a GPU memory fault;
+    they must not be compiled out by ``python -O`` the way ``assert`` is."""
+    import subprocess
+    import sys
+    code = ("import numpy as np\n"
+            "from poker2_amd._guards import require\n"
+            "from poker2_amd.tree import RootStates, build_sparse_tree\n"
+            "assert False, 'asserts are off under -O, so this line must not raise'\n"
+            "try:\n"
+            "    require(1 + 1 == 3, 'refused')\n"
+            "except AssertionError as e:\n"
+            "    assert str(e) == 'refused'\n"
+            "else:\n"
+            "    raise SystemExit(3)\n"
+            "try:\n"
+            "    build_sparse_tree(RootStates.at_round_start(3, np.zeros(0), np.zeros((0, 2)), np.zeros((0, 5))), [0.5], 2)\n"
+            "except AssertionError:\n"
+            "    raise SystemExit(0)\n"
+            "raise SystemExit(4)\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-O", "-c", code], cwd=root, capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr[-2000:]
+    # no plain assert is left in the package's modules
+    import glob
+    import re
+    left = [p for p in glob.glob(os.path.join(root, "poker2_amd", "*.py"))
+            if re.search(r"^\s*assert\b", open(p).read(), re.M)]
+    assert left == [], left
