@@ -111,6 +111,9 @@ class HipSparseCFREvaluator:
             raise ValueError("HipSparseCFREvaluator requires a GPU device.")
         if not F.triton_is_available():
             raise RuntimeError("libp2hip.so or a GPU is not available; HipSparseCFREvaluator has no other backend.")
+        if getattr(cfg.env, "flop_showdown", False):
+            raise NotImplementedError("the env's flop_showdown game variant (showdown right after the preflop round, "
+                                      "hunl_tensor_env.py:900) is not built; the tree builders follow the full game")
         s = cfg.search
         self.float_dtype = torch.float32
         self.num_players = 2

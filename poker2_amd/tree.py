@@ -127,6 +127,9 @@ class RootStates:
         """Copy rows of an object exposing the reference env's attribute names
         (``HUNLTensorEnv``: button, street, to_act, pot, stacks, committed, min_raise,
         actions_this_round, is_allin, starting_stacks, scale, board_indices, done, bb)."""
+        if getattr(env, "flop_showdown", False):
+            raise NotImplementedError("roots of the env's flop_showdown game variant (hunl_tensor_env.py:900) are not "
+                                      "supported: the tree builders follow the full game")
         def g(name):
             x = getattr(env, name)
             x = x.detach().cpu().numpy() if hasattr(x, "detach") else np.asarray(x)

@@ -105,3 +105,10 @@ def test_roots_from_an_env_like_object_with_torch_tensors():
         assert np.array_equal(a, b) if isinstance(a, np.ndarray) else a == b, name
     t1, t2 = build_sparse_tree(roots, [0.5, 1.0], 2), build_sparse_tree(ref, [0.5, 1.0], 2)
     assert t1.total == t2.total and np.array_equal(t1.child_count, t2.child_count)
+
+
+def test_roots_of_the_flop_showdown_variant_are_refused():
+    import types
+    env = types.SimpleNamespace(flop_showdown=True)
+    with pytest.raises(NotImplementedError):
+        RootStates.from_env(env, np.arange(1))
