@@ -126,7 +126,8 @@ class RootStates:
     def from_env(cls, env, indices) -> "RootStates":
         """Copy rows of an object exposing the reference env's attribute names
         (``HUNLTensorEnv``: button, street, to_act, pot, stacks, committed, min_raise,
-        actions_this_round, is_allin, starting_stacks, scale, board_indices, done, bb)."""
+        actions_this_round, is_allin, starting_stacks, scale, board_indices, done, bb; optional
+        last_board_indices and deck)."""
         if getattr(env, "flop_showdown", False):
             raise NotImplementedError("roots of the env's flop_showdown game variant (hunl_tensor_env.py:900) are not "
                                       "supported: the tree builders follow the full game")
@@ -144,7 +145,10 @@ class RootStates:
                    is_allin=g("is_allin").astype(bool), starting_stacks=g("starting_stacks").astype(np.int64),
                    scale=g("scale").astype(np.float32), board=g("board_indices").astype(np.int64),
                    done=g("done").astype(bool), bb=int(getattr(env, "bb", 100)),
-                   last_board=g("last_board_indices").astype(np.int64) if hasattr(env, "last_board_indices") else None)
+                   last_board=g("last_board_indices").astype(np.int64) if hasattr(env, "last_board_indices") else None,
+                   # the env deals streets from the deck it was reset with: four hole cards, then the five
+                   # board cards (hunl_tensor_env.py:280-285, 900-975)
+                   runout=g("deck")[:, 4:9].astype(np.int64) if hasattr(env, "deck") else None)
 
 
 _STATE_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",

@@ -12,7 +12,9 @@ reset state is dropped from the value batch).  The leaf network is a closed-form
 encoded features (written out in ``ValueNet`` below; tests restate it), so the search, the
 encoder and the chance nodes all feed the stored targets.  The flop chance node runs in its
 exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
-A last section holds what the env's ``reset`` deals from a seeded CPU generator.
+Each case also holds one whole ``evaluate_cfr`` (sampling schedule, search, leaf sampling with
+exploration and dealing) run from a CPU generator seeded 77: the iterations it snapshots and the
+leaves it returns.  A last section holds what the env's ``reset`` deals from a seeded CPU generator.
 
 With ``--fused`` the same searches run through the reference's ``FusedSparseCFREvaluator``, its
 Triton kernels executing under Triton's CPU interpreter, and go to
@@ -175,6 +177,25 @@ def main(fused: bool = False) -> None:
                 out[f"{p}/policy_targets_sum"] = pt.astype(np.float64).sum(axis=1)
             for k, v in batch.statistics.items():
                 out[f"{p}/stat/{k}"] = v.numpy()
+        # the whole search with its random parts (cfr_evaluator.py:1497-1528: sampling schedule, search, leaf
+        # sampling with exploration, sparse_cfr_evaluator.py:325-426) from a seeded CPU generator
+        gen = torch.Generator(device="cpu")
+        gen.manual_seed(77)
+        ev2 = SparseCFREvaluator(model=ValueNet(len(bins) + 3), device=dev, cfg=cfg, generator=gen)
+        if fused:
+            ev2.__class__ = FusedSparseCFREvaluator
+            ev2._ensure_fused_attrs()
+        ev2.initialize_subgame(env, torch.arange(n), initial_beliefs=torch.from_numpy(bel.copy()))
+        pbs = ev2.evaluate_cfr(training_mode=True)
+        out[f"{name}/search/seed"] = np.int64(77)
+        out[f"{name}/search/root_deck"] = env.deck.clone().numpy()
+        out[f"{name}/search/t_sample"] = ev2.t_sample.numpy()
+        for f in ENV_FIELDS + ("deck",):
+            out[f"{name}/search/leaf/{f}"] = getattr(pbs.env, f).clone().numpy()
+        lb = pbs.beliefs.numpy()
+        out[f"{name}/search/leaf_beliefs"] = np.ascontiguousarray(lb[..., cols]).astype(np.float32)
+        out[f"{name}/search/leaf_beliefs_rowsum"] = lb.astype(np.float64).sum(-1)
+        print(name, "sampled leaves", lb.shape[0], "streets", getattr(pbs.env, "street").tolist(), flush=True)
         out[f"{name}/beliefs"] = bel
         out[f"{name}/depth_offsets"] = np.array(ev.depth_offsets, dtype=np.int64)
         out[f"{name}/settings"] = np.array([str(depth), str(iters)])

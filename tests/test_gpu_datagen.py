@@ -411,3 +411,42 @@ def test_leaf_model_does_not_reuse_features_of_the_previous_subgame():
         assert torch.equal(ev.model_indices, fresh.model_indices)
         assert torch.equal(ev.latest_values, fresh.latest_values)
         assert ev.latest_values[ev.model_indices].abs().max() > 0
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fixture", ["base", "fused"])
+@pytest.mark.parametrize("name", ["streets_mixed", "preflop"])
+def test_whole_search_from_a_seeded_generator_samples_the_reference_leaves(golden_dir, name, fused, fixture):
+    """``evaluate_cfr`` with its random parts — the sampling schedule, the hand and exploration
+    draws of the leaf walk (cfr_evaluator.py:1497-1528, :382-404, sparse_cfr_evaluator.py:325-426)
+    — from a CPU generator with the seed the reference run used: the same iterations are
+    snapshotted, the same leaves come out, and leaves that closed a betting round stand on the
+    next street with the cards the env's deck deals."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel
+    from poker2_amd.tree import RootStates
+    case, cols = load_case(golden_dir, name, fixture)
+    r = {k[5:]: v for k, v in case.items() if k.startswith("root/")}
+    n = len(r["street"])
+    roots = RootStates.from_env(SimpleNamespace(bb=100, deck=case["search/root_deck"], **r), np.arange(n))
+    assert np.array_equal(roots.runout, case["search/root_deck"][:, 4:9])
+    depth, iters = int(case["settings"][0]), int(case["settings"][1])
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(int(case["search/seed"]))
+    ev = HipSparseCFREvaluator(NetworkLeafModel(ValueNet(), DEV), torch.device(DEV),
+                               river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0), generator=gen,
+                               fused_iteration=fused)
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(case["beliefs"]))
+    leaves = ev.evaluate_cfr(training_mode=True)
+    assert np.array_equal(ev.t_sample.cpu().numpy(), case["search/t_sample"])
+    got = leaves.roots
+    names = {"board": "board_indices", "last_board": "last_board_indices"}
+    for field in ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",
+                  "is_allin", "starting_stacks", "scale", "board", "last_board", "done"):
+        want = case[f"search/leaf/{names.get(field, field)}"]
+        assert np.array_equal(np.asarray(getattr(got, field)), want.astype(np.asarray(getattr(got, field)).dtype)), field
+    assert np.array_equal(got.runout, case["search/leaf/deck"][:, 4:9])          # the deck travels with the state
+    lb = leaves.beliefs.cpu().numpy()
+    np.testing.assert_allclose(lb[..., cols], case["search/leaf_beliefs"], rtol=3e-4, atol=3e-6)
+    np.testing.assert_allclose(lb.sum(-1, dtype=np.float64), case["search/leaf_beliefs_rowsum"], rtol=1e-4)
