@@ -450,3 +450,85 @@ def test_whole_search_from_a_seeded_generator_samples_the_reference_leaves(golde
     lb = leaves.beliefs.cpu().numpy()
     np.testing.assert_allclose(lb[..., cols], case["search/leaf_beliefs"], rtol=3e-4, atol=3e-6)
     np.testing.assert_allclose(lb.sum(-1, dtype=np.float64), case["search/leaf_beliefs_rowsum"], rtol=1e-4)
+
+
+def compare_generator_batch(g, prefix, batch, cols, every_entry):
+    """One batch the loop stored or returned against the fixture's.  ``every_entry``: the fixture
+    comes from the reference's fused class, whose conventions on board-blocked hands the product
+    shares; otherwise hands that the batch's own board blocks are left out of the float checks."""
+    n = int(g[f"{prefix}/len"])
+    assert len(batch) == n, prefix
+    if n == 0:
+        return
+    f = batch.features
+    np.testing.assert_allclose(f.context.cpu().numpy(), g[f"{prefix}/context"], rtol=1e-6, atol=0, err_msg=prefix)
+    board = f.board.cpu().numpy()
+    assert np.array_equal(board, g[f"{prefix}/board"]), prefix
+    assert np.array_equal(f.to_act.cpu().numpy(), g[f"{prefix}/to_act"]), prefix
+    assert np.array_equal(f.street.cpu().numpy(), g[f"{prefix}/street"]), prefix
+    assert np.array_equal(batch.legal_masks.cpu().numpy(), g[f"{prefix}/legal_masks"]), prefix
+    ok = np.ones((n, H), bool) if every_entry else OC.allowed_hands_for_boards(board)[0]
+    rtol, atol = 3e-4, 3e-6
+    fb = f.beliefs.cpu().numpy().reshape(n, 2, H)
+    close(fb[..., cols], g[f"{prefix}/beliefs"], ok[:, None, cols], rtol, atol, f"{prefix} beliefs")
+    if batch.value_targets is not None:
+        vt = batch.value_targets.cpu().numpy()
+        close(vt[..., cols], g[f"{prefix}/value_targets"], ok[:, None, cols], rtol, atol, f"{prefix} value targets")
+    if batch.policy_targets is not None:
+        pt = batch.policy_targets.cpu().numpy()
+        close(pt[:, cols, :], g[f"{prefix}/policy_targets"], ok[:, cols, None], rtol, atol, f"{prefix} policy targets")
+
+
+@pytest.mark.parametrize("fixture", ["base", "fused"])
+def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
+    """The whole self-play loop (rebel_data_generator.py:52-95) against a run of the reference's own
+    generator, evaluator and env from the same two seeds: the same hands are dealt, the same
+    batches reach the buffers pass by pass, the call returns the same samples and leaves the same
+    public states behind — decks included, so the next call would deal the same cards."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel
+    from poker2_amd.rebel_data_generator import EnvProto, RebelDataGenerator
+    g = np.load(str(golden_dir) + ("/fused_generator_golden.npz" if fixture == "fused" else "/generator_golden.npz"))
+    n, depth, iters, asked, env_seed, search_seed = (int(x) for x in g["settings"])
+    cols = g["columns"]
+    env_gen, search_gen = torch.Generator(device="cpu"), torch.Generator(device="cpu")
+    env_gen.manual_seed(env_seed)
+    search_gen.manual_seed(search_seed)
+    proto = EnvProto(mean_stack=1000, sb=50, bb=100, randomize_stacks=True, rng=env_gen)
+    ev = HipSparseCFREvaluator(NetworkLeafModel(ValueNet(), DEV), torch.device(DEV),
+                               river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0), generator=search_gen)
+
+    class Recorder:
+        def __init__(self):
+            self.batches = []
+
+        def add_batch(self, batch):
+            self.batches.append(batch)
+    value_buffer, policy_buffer = Recorder(), Recorder()
+    dg = RebelDataGenerator(proto, ev, value_buffer, policy_buffer)
+
+    def same_states(tag, roots):
+        names = {"board": "board_indices", "last_board": "last_board_indices"}
+        for field in ("street", "to_act", "button", "pot", "stacks", "committed", "min_raise", "actions_this_round",
+                      "is_allin", "starting_stacks", "scale", "board", "done"):
+            got = np.asarray(getattr(roots, field))
+            assert np.array_equal(got, g[f"{tag}/{names.get(field, field)}"].astype(got.dtype)), (tag, field)
+        assert np.array_equal(roots.runout, g[f"{tag}/deck"][:, 4:9]), tag
+        assert np.array_equal(roots.previous_board(), g[f"{tag}/last_board_indices"]), tag
+    same_states("first_deal", dg.current_pbs.env)
+    value_batch, policy_batch = dg.generate_data(asked)
+    every = fixture == "fused"
+    assert len(policy_buffer.batches) == int(g["passes"]) and len(value_buffer.batches) == 2 * int(g["passes"])
+    for i, b in enumerate(value_buffer.batches):
+        compare_generator_batch(g, f"value_buffer/{i}", b, cols, every or i % 2 == 1)   # odd adds: ranges before the deal
+    for i, b in enumerate(policy_buffer.batches):
+        compare_generator_batch(g, f"policy_buffer/{i}", b, cols, every)
+    assert len(value_batch) == int(g["returned/value/len"]) and len(policy_batch) == int(g["returned/policy/len"])
+    assert np.array_equal(value_batch.features.board.cpu().numpy(), g["returned/value/board"])
+    assert np.array_equal(policy_batch.features.board.cpu().numpy(), g["returned/policy/board"])
+    assert dg.last_extra == int(g["last_extra"])
+    same_states("left", dg.current_pbs.env)
+    lb = dg.current_pbs.beliefs.cpu().numpy()
+    ok = np.ones(lb.shape[::2], bool) if every else OC.allowed_hands_for_boards(g["left/board_indices"])[0]
+    close(lb[..., cols], g["left/beliefs"], ok[:, None, cols], 3e-4, 3e-6, "beliefs left behind")
