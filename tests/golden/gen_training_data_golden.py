@@ -10,7 +10,8 @@ and river and flop roots at the start of a betting round (these get pre-chance v
 through the single-card / flop chance node), roots in the middle of a round, preflop roots (the
 reset state is dropped from the value batch).  The leaf network is a closed-form function of the
 encoded features (written out in ``ValueNet`` below; tests restate it), so the search, the
-encoder and the chance nodes all feed the stored targets.  The flop chance node runs in its
+encoder and the chance nodes all feed the stored targets.  Two more cases use the reference's default algorithm (linear CFR with
+CFR+, cfr_avg, zero-sum network; with and without the warm start).  The flop chance node runs in its
 exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
 Each case also holds one whole ``evaluate_cfr`` (sampling schedule, search, leaf sampling with
 exploration and dealing) run from a CPU generator seeded 77: the iterations it snapshots and the
@@ -36,11 +37,20 @@ ENV_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_r
               "is_allin", "starting_stacks", "scale", "board_indices", "last_board_indices", "done")
 STATE = ("policy_probs_avg", "beliefs", "beliefs_avg", "values_avg")
 
-# name, depth, iterations, per root: (button, bins played from the reset state)
+# name, depth, last iteration + 1, per root: (button, bins played from the reset state), search settings
+DISCOUNTED = {"cfr_type": "discounted", "cfr_plus": False, "cfr_avg": False, "warm": 0, "enforce_zero_sum": False}
 CASES = [
     ("streets_mixed", 3, 4, [(0, [1, 1, 1, 1]), (1, [3, 1, 1, 1]), (0, [1, 1, 1, 1, 1, 1]),
-                             (1, [1, 1, 1, 1, 1, 1, 2]), (0, [2, 1]), (1, [1, 1, 1, 1, 1])]),
-    ("preflop", 2, 3, [(0, []), (1, [1]), (1, [])]),
+                             (1, [1, 1, 1, 1, 1, 1, 2]), (0, [2, 1]), (1, [1, 1, 1, 1, 1])], DISCOUNTED),
+    ("preflop", 2, 3, [(0, []), (1, [1]), (1, [])], DISCOUNTED),
+    # the reference's default algorithm (structured_config.py:236-265: linear CFR with CFR+, leaf values
+    # de-averaged for cfr_avg, a model_br warm start) with a network that asks for zero-sum values
+    ("linear_avg_zero_sum", 3, 5, [(0, [1, 1, 1, 1]), (1, [1, 1, 1, 1, 1, 1]), (0, [1, 1, 1, 1, 2]), (1, [2, 1])],
+     {"cfr_type": "linear", "cfr_plus": True, "cfr_avg": True, "warm": 0, "enforce_zero_sum": True}),
+    # the same with the warm start; base class only: the fused class runs its warm start with device scalars that
+    # no iteration has filled yet (see gen_cfr_golden.py), which under linear CFR also feeds the leaf de-averaging
+    ("linear_avg_zero_sum_warm", 3, 6, [(0, [1, 1, 1, 1]), (1, [1, 1, 1, 1, 1, 1]), (0, [1, 1, 1, 1, 2]), (1, [2, 1])],
+     {"cfr_type": "linear", "cfr_plus": True, "cfr_avg": True, "warm": 2, "enforce_zero_sum": True, "base_only": True}),
 ]
 
 
@@ -71,9 +81,9 @@ def main(fused: bool = False) -> None:
              w = 0.2 + 0.1 * context[2] + 0.05 * context[1] - 0.03 * context[3]
                  + 0.01 / 13 * sum over dealt board cards of (rank + 1)."""
 
-        def __init__(self, num_actions):
+        def __init__(self, num_actions, enforce_zero_sum=False):
             self.num_actions = num_actions
-            self.enforce_zero_sum = False
+            self.enforce_zero_sum = enforce_zero_sum
             self.hidden_dim = 1
 
         def create_feature_encoder(self, env, device=None, dtype=None):
@@ -96,10 +106,11 @@ def main(fused: bool = False) -> None:
 
     rng = np.random.default_rng(515)
     cols = np.sort(rng.choice(NUM_HANDS, 64, replace=False))
-    out = {"columns": cols, "case_names": np.array([c[0] for c in CASES])}
+    cases = [c for c in CASES if not (fused and c[4].get("base_only"))]
+    out = {"columns": cols, "case_names": np.array([c[0] for c in cases])}
     dev = torch.device("cpu")
     bins = [0.5, 1.0]
-    for name, depth, iters, scripts in CASES:
+    for name, depth, iters, scripts, algo in cases:
         n = len(scripts)
         env = HUNLTensorEnv(num_envs=n, starting_stack=1000, sb=50, bb=100, default_bet_bins=list(bins), device=dev)
         deck = torch.stack([torch.from_numpy(rng.permutation(52)[:9].copy()) for _ in range(n)])
@@ -118,14 +129,14 @@ def main(fused: bool = False) -> None:
         cfg.env.stack, cfg.env.sb, cfg.env.bb, cfg.env.bet_bins, cfg.env.flop_showdown = 1000, 50, 100, bins, False
         cfg.search = SearchConfig()
         cfg.search.iterations = iters
-        cfg.search.warm_start_iterations = 0
+        cfg.search.warm_start_iterations = algo["warm"]
         cfg.search.depth = depth
         cfg.search.dcfr_alpha, cfg.search.dcfr_beta, cfg.search.dcfr_gamma = 1.5, 0.0, 2.0
         cfg.search.dcfr_plus_delay = 0
-        cfg.search.cfr_type = CFRType["discounted"]
-        cfg.search.cfr_plus = False
-        cfg.search.cfr_avg = False
-        ev = SparseCFREvaluator(model=ValueNet(len(bins) + 3), device=dev, cfg=cfg)
+        cfg.search.cfr_type = CFRType[algo["cfr_type"]]
+        cfg.search.cfr_plus = algo["cfr_plus"]
+        cfg.search.cfr_avg = algo["cfr_avg"]
+        ev = SparseCFREvaluator(model=ValueNet(len(bins) + 3, algo["enforce_zero_sum"]), device=dev, cfg=cfg)
         if fused:
             ev.__class__ = FusedSparseCFREvaluator
             ev._ensure_fused_attrs()
@@ -137,12 +148,14 @@ def main(fused: bool = False) -> None:
         for f in ENV_FIELDS:
             out[f"{name}/root/{f}"] = getattr(env, f).clone().numpy()
         ev.initialize_subgame(env, torch.arange(n), initial_beliefs=torch.from_numpy(bel.copy()))
-        ev.initialize_policy_and_beliefs()
+        ev.initialize_policy_and_beliefs()               # evaluate_cfr (cfr_evaluator.py:1497-1518) without its draws
+        if algo["warm"] > 0:
+            ev.warm_start()
         ev.set_leaf_values(0)
         ev.compute_expected_values()
         ev.values_avg[:] = ev.latest_values
         ev.t_sample = torch.full((ev.total_nodes,), -1, dtype=torch.long)
-        for t in range(iters):
+        for t in range(algo["warm"], iters):
             ev.cfr_iteration(t)
         for s in STATE:
             x = getattr(ev, s).detach().numpy()
@@ -181,7 +194,8 @@ def main(fused: bool = False) -> None:
         # sampling with exploration, sparse_cfr_evaluator.py:325-426) from a seeded CPU generator
         gen = torch.Generator(device="cpu")
         gen.manual_seed(77)
-        ev2 = SparseCFREvaluator(model=ValueNet(len(bins) + 3), device=dev, cfg=cfg, generator=gen)
+        ev2 = SparseCFREvaluator(model=ValueNet(len(bins) + 3, algo["enforce_zero_sum"]), device=dev, cfg=cfg,
+                                 generator=gen)
         if fused:
             ev2.__class__ = FusedSparseCFREvaluator
             ev2._ensure_fused_attrs()
@@ -198,7 +212,8 @@ def main(fused: bool = False) -> None:
         print(name, "sampled leaves", lb.shape[0], "streets", getattr(pbs.env, "street").tolist(), flush=True)
         out[f"{name}/beliefs"] = bel
         out[f"{name}/depth_offsets"] = np.array(ev.depth_offsets, dtype=np.int64)
-        out[f"{name}/settings"] = np.array([str(depth), str(iters)])
+        out[f"{name}/settings"] = np.array([str(depth), str(iters), algo["cfr_type"], str(algo["cfr_plus"]),
+                                            str(algo["cfr_avg"]), str(algo["warm"]), str(algo["enforce_zero_sum"])])
         print(name, "nodes", ev.total_nodes, "depth offsets", ev.depth_offsets,
               {k: len(b) for k, b in batches.items()}, flush=True)
     # the env's own reset (hunl_tensor_env.py:219-346) from a seeded CPU generator: button, deck, stacks

@@ -34,6 +34,18 @@ def load_case(golden_dir, name, fixture="base"):
     return {k[len(name) + 1:]: g[k] for k in g.files if k.startswith(name + "/")}, g["columns"]
 
 
+CASE_NAMES = ["streets_mixed", "preflop", "linear_avg_zero_sum", "linear_avg_zero_sum_warm"]
+BASE_ONLY = {"linear_avg_zero_sum_warm"}      # the reference's fused class runs its warm start on unfilled scalars
+
+
+def case_settings(case):
+    """(depth, last iteration + 1, search settings) of a fixture case."""
+    st = [str(x) for x in case["settings"]]
+    algo = {"cfr_type": st[2], "cfr_plus": st[3] == "True", "cfr_avg": st[4] == "True", "warm": int(st[5]),
+            "enforce_zero_sum": st[6] == "True"}
+    return int(st[0]), int(st[1]), algo
+
+
 def oracle_roots(case):
     r = {k[5:]: v for k, v in case.items() if k.startswith("root/")}
     return [OT.Node(to_act=int(r["to_act"][i]), button=int(r["button"][i]), street=int(r["street"][i]),
@@ -45,7 +57,7 @@ def oracle_roots(case):
 
 def run_oracle(case, fused_variant=False):
     roots, r = oracle_roots(case)
-    depth, iters = int(case["settings"][0]), int(case["settings"][1])
+    depth, iters, algo = case_settings(case)
     tree = OT.build_tree(roots, BINS, depth)
     env = ODG.tree_env(tree, r["board_indices"])
     assert np.array_equal(env["last_board_indices"][:len(roots)], r["last_board_indices"])   # the derived rule
@@ -54,9 +66,11 @@ def run_oracle(case, fused_variant=False):
         f = ODG.encode(env, beliefs, pre_chance_node=tree["new_street_mask"], indices=rows)
         return value_net_numpy(f["context"], f["street"], f["to_act"], f["board"], f["beliefs"])
     o = OCFR.OracleCFR(tree, r["board_indices"], case["beliefs"], cfr_iterations=iters, leaf_value_fn=leaf_fn,
-                       t_sample_roots=np.full(len(roots), -1, dtype=np.int64), fused_variant=fused_variant)
-    o.prepare()
-    for t in range(iters):
+                       t_sample_roots=np.full(len(roots), -1, dtype=np.int64), fused_variant=fused_variant,
+                       cfr_type=algo["cfr_type"], cfr_plus=algo["cfr_plus"], cfr_avg=algo["cfr_avg"],
+                       warm_start_iterations=algo["warm"], enforce_zero_sum=algo["enforce_zero_sum"])
+    o.prepare()                                   # includes the warm start
+    for t in range(algo["warm"], iters):
         o.cfr_iteration(t)
     return o, tree, env
 
@@ -101,8 +115,10 @@ def check_batch(got, case, tag, cols, rtol, atol):
 
 
 @pytest.mark.parametrize("fixture", ["base", "fused"])
-@pytest.mark.parametrize("name", ["streets_mixed", "preflop"])
+@pytest.mark.parametrize("name", CASE_NAMES)
 def test_oracle_training_data_matches_vectors_from_the_reference(golden_dir, name, fixture):
+    if fixture == "fused" and name in BASE_ONLY:
+        pytest.skip("no fused-class fixture for this case")
     case, cols = load_case(golden_dir, name, fixture)
     o, tree, env = run_oracle(case, fused_variant=fixture == "fused")
     assert o.depth_offsets == case["depth_offsets"].tolist()
