@@ -506,11 +506,16 @@ class OracleCFR:
         for t in range(self.warm_start_iterations, self.cfr_iterations):
             self.cfr_iteration(t)
         if self.use_final_policy_values:
-            self.set_leaf_values(0, beliefs=self.beliefs_avg)
-            self.compute_expected_values(self.policy_probs_avg, self.beliefs_avg,
-                                         self.latest_values, self.values_avg)
-            self.values_avg[:] = self.maybe_enforce_zero_sum(self.values_avg, self.beliefs_avg,
-                                                             ignore_mask=self.done)
+            self.update_average_values_final()
+
+    def update_average_values_final(self) -> None:
+        """cfr_evaluator.py:1276-1292: values of the final average strategy, leaves re-evaluated
+        on the average ranges."""
+        self.set_leaf_values(0, beliefs=self.beliefs_avg)
+        self.compute_expected_values(self.policy_probs_avg, self.beliefs_avg,
+                                     self.latest_values, self.values_avg)
+        self.values_avg[:] = self.maybe_enforce_zero_sum(self.values_avg, self.beliefs_avg,
+                                                         ignore_mask=self.done)
 
     STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
                    "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",

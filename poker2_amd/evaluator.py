@@ -379,10 +379,10 @@ class HipSparseCFREvaluator:
         self._t_scalars.update(t=t, dcfr_alpha=self.dcfr_alpha, dcfr_beta=self.dcfr_beta,
                                mix_old=float(mix_old), mix_new=float(mix_new))
         apply_dcfr = self.cfr_type in (CFRType.discounted, CFRType.discounted_plus)
-        a, b = float(t ** self.dcfr_alpha), float(t ** self.dcfr_beta)
+        (a, a_den), (b, b_den) = F.discount_pair(t, self.dcfr_alpha), F.discount_pair(t, self.dcfr_beta)
         total = float(mix_old) + float(mix_new)
         f = self._fscal_host
-        f[0], f[1], f[2], f[3] = a, b, a + 1.0, b + 1.0
+        f[0], f[1], f[2], f[3] = a, b, a_den, b_den
         f[4], f[5], f[6] = float(mix_old), float(mix_new), total
         f[7] = 1.0 / total if total != 0.0 else 1.0
         i = self._iscal_host

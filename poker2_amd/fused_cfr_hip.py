@@ -51,6 +51,17 @@ def _scalars(values, like: torch.Tensor):
     return [buf[k] for k in range(n)]
 
 
+def discount_pair(t: int, exponent: float) -> tuple[float, float]:
+    """(t**e, t**e + 1): numerator and denominator of the DCFR discount t**e / (t**e + 1)
+    (cfr_evaluator.py:1346-1362).  At t = 0 with a negative exponent — beta = -1 in the reference's
+    own settings — t**e does not exist; the factor's limit is 1, returned as (1, 1).  (The reference
+    evaluates ``0 ** e`` there and raises; its runs start after a warm start, so t >= 1.)"""
+    if t == 0 and exponent < 0:
+        return 1.0, 1.0
+    num = float(t ** exponent)
+    return num, num + 1.0
+
+
 def _scalar(value: float, like: torch.Tensor) -> torch.Tensor:
     return _scalars([value], like)[0]
 
@@ -97,9 +108,8 @@ def fused_dcfr_update_(cumulative_regrets, regret_weight_sums, regrets, t: int, 
          "cumulative_regrets.shape == regret_weight_sums.shape == regrets.shape")
     apply_dcfr = getattr(cfr_type, "name", cfr_type) in ("discounted", "discounted_plus")
     if apply_dcfr:
-        a = float(t ** dcfr_alpha)
-        b = float(t ** dcfr_beta)
-        vals = (a, b, a + 1.0, b + 1.0)
+        (a, a_den), (b, b_den) = discount_pair(t, dcfr_alpha), discount_pair(t, dcfr_beta)
+        vals = (a, b, a_den, b_den)
     else:
         vals = (1.0, 1.0, 1.0, 1.0)
     an, bn, ad, bd = _scalars(vals, cumulative_regrets)
@@ -640,12 +650,11 @@ class TScalars:
         self.t_tensor = torch.zeros((), dtype=torch.long, device=device)
 
     def update(self, t: int, dcfr_alpha: float, dcfr_beta: float, mix_old: float, mix_new: float) -> None:
-        t_alpha_num = float(t ** dcfr_alpha)
-        t_beta_num = float(t ** dcfr_beta)
+        (t_alpha_num, t_alpha_den), (t_beta_num, t_beta_den) = discount_pair(t, dcfr_alpha), discount_pair(t, dcfr_beta)
         self.t_alpha_num.fill_(t_alpha_num)
         self.t_beta_num.fill_(t_beta_num)
-        self.t_alpha_den.fill_(t_alpha_num + 1.0)
-        self.t_beta_den.fill_(t_beta_num + 1.0)
+        self.t_alpha_den.fill_(t_alpha_den)
+        self.t_beta_den.fill_(t_beta_den)
         total = float(mix_old) + float(mix_new)
         self.mix_old.fill_(float(mix_old))
         self.mix_new.fill_(float(mix_new))

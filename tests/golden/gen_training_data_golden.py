@@ -11,7 +11,9 @@ through the single-card / flop chance node), roots in the middle of a round, pre
 reset state is dropped from the value batch).  The leaf network is a closed-form function of the
 encoded features (written out in ``ValueNet`` below; tests restate it), so the search, the
 encoder and the chance nodes all feed the stored targets.  Two more cases use the reference's default algorithm (linear CFR with
-CFR+, cfr_avg, zero-sum network; with and without the warm start).  The flop chance node runs in its
+CFR+, cfr_avg, zero-sum network; with and without the warm start).  A last case has the shape of
+the reference's production settings (discounted_plus with delay, model warm start, alpha / beta /
+gamma schedules, value targets from the final average strategy).  The flop chance node runs in its
 exhaustive mode (all classes, all 24 permutations): nothing is drawn at random.
 Each case also holds one whole ``evaluate_cfr`` (sampling schedule, search, leaf sampling with
 exploration and dealing) run from a CPU generator seeded 77: the iterations it snapshots and the
@@ -24,6 +26,7 @@ Triton kernels executing under Triton's CPU interpreter, and go to
 """
 from __future__ import annotations
 
+import json
 import os
 import sys
 
@@ -38,7 +41,11 @@ ENV_FIELDS = ("street", "to_act", "button", "pot", "stacks", "committed", "min_r
 STATE = ("policy_probs_avg", "beliefs", "beliefs_avg", "values_avg")
 
 # name, depth, last iteration + 1, per root: (button, bins played from the reset state), search settings
-DISCOUNTED = {"cfr_type": "discounted", "cfr_plus": False, "cfr_avg": False, "warm": 0, "enforce_zero_sum": False}
+DEFAULTS = {"cfr_type": "discounted", "cfr_plus": False, "cfr_avg": False, "warm": 0, "enforce_zero_sum": False,
+            "delay": 0, "alpha": 1.5, "beta": 0.0, "gamma": 2.0, "alpha_final": None, "beta_final": None,
+            "gamma_final": None, "warm_type": "model_br", "warm_mult": 1.0, "final_policy_values": False,
+            "base_only": False}
+DISCOUNTED = {}
 CASES = [
     ("streets_mixed", 3, 4, [(0, [1, 1, 1, 1]), (1, [3, 1, 1, 1]), (0, [1, 1, 1, 1, 1, 1]),
                              (1, [1, 1, 1, 1, 1, 1, 2]), (0, [2, 1]), (1, [1, 1, 1, 1, 1])], DISCOUNTED),
@@ -51,6 +58,13 @@ CASES = [
     # no iteration has filled yet (see gen_cfr_golden.py), which under linear CFR also feeds the leaf de-averaging
     ("linear_avg_zero_sum_warm", 3, 6, [(0, [1, 1, 1, 1]), (1, [1, 1, 1, 1, 1, 1]), (0, [1, 1, 1, 1, 2]), (1, [2, 1])],
      {"cfr_type": "linear", "cfr_plus": True, "cfr_avg": True, "warm": 2, "enforce_zero_sum": True, "base_only": True}),
+    # the shape of the reference's own search settings (conf/config_rebel_cfr.yaml:70-92), scaled down: discounted_plus
+    # with a delay that outlasts the warm start, `model` warm start x 10, alpha / beta / gamma schedules towards their
+    # `_final` values, value targets taken from the final average strategy
+    ("production_like", 3, 9, [(1, [1, 1, 1, 1]), (0, [1, 1, 1, 1, 1, 1]), (1, [1, 1, 1, 1, 2]), (0, [1, 1, 3, 1])],
+     {"cfr_type": "discounted_plus", "delay": 4, "warm": 3, "warm_type": "model", "warm_mult": 10.0, "alpha": 2.0,
+      "alpha_final": 4.0, "beta": -1.0, "beta_final": -2.0, "gamma": 5.0, "gamma_final": 0.0,
+      "final_policy_values": True}),
 ]
 
 
@@ -64,7 +78,8 @@ def main(fused: bool = False) -> None:
     sys.path.insert(0, REF_SRC)
     import warnings
     import torch
-    from p2.core.structured_config import CFRType, Config, EnvConfig, ModelConfig, SearchConfig, TrainingConfig
+    from p2.core.structured_config import (CFRType, Config, EnvConfig, ModelConfig, SearchConfig, TrainingConfig,
+                                           WarmStartType)
     from p2.env.card_utils import NUM_HANDS
     from p2.env.hunl_tensor_env import HUNLTensorEnv
     from p2.models.model_output import ModelOutput
@@ -106,11 +121,12 @@ def main(fused: bool = False) -> None:
 
     rng = np.random.default_rng(515)
     cols = np.sort(rng.choice(NUM_HANDS, 64, replace=False))
-    cases = [c for c in CASES if not (fused and c[4].get("base_only"))]
+    cases = [c for c in CASES if not (fused and c[4].get("base_only", False))]
     out = {"columns": cols, "case_names": np.array([c[0] for c in cases])}
     dev = torch.device("cpu")
     bins = [0.5, 1.0]
-    for name, depth, iters, scripts, algo in cases:
+    for name, depth, iters, scripts, overrides in cases:
+        algo = {**DEFAULTS, **overrides}
         n = len(scripts)
         env = HUNLTensorEnv(num_envs=n, starting_stack=1000, sb=50, bb=100, default_bet_bins=list(bins), device=dev)
         deck = torch.stack([torch.from_numpy(rng.permutation(52)[:9].copy()) for _ in range(n)])
@@ -131,8 +147,13 @@ def main(fused: bool = False) -> None:
         cfg.search.iterations = iters
         cfg.search.warm_start_iterations = algo["warm"]
         cfg.search.depth = depth
-        cfg.search.dcfr_alpha, cfg.search.dcfr_beta, cfg.search.dcfr_gamma = 1.5, 0.0, 2.0
-        cfg.search.dcfr_plus_delay = 0
+        cfg.search.dcfr_alpha, cfg.search.dcfr_beta, cfg.search.dcfr_gamma = algo["alpha"], algo["beta"], algo["gamma"]
+        cfg.search.dcfr_alpha_final, cfg.search.dcfr_beta_final = algo["alpha_final"], algo["beta_final"]
+        cfg.search.dcfr_gamma_final = algo["gamma_final"]
+        cfg.search.dcfr_plus_delay = algo["delay"]
+        cfg.search.warm_start_type = WarmStartType[algo["warm_type"]]
+        cfg.search.warm_start_multiplier = algo["warm_mult"]
+        cfg.search.value_targets_from_final_policy = algo["final_policy_values"]
         cfg.search.cfr_type = CFRType[algo["cfr_type"]]
         cfg.search.cfr_plus = algo["cfr_plus"]
         cfg.search.cfr_avg = algo["cfr_avg"]
@@ -157,6 +178,8 @@ def main(fused: bool = False) -> None:
         ev.t_sample = torch.full((ev.total_nodes,), -1, dtype=torch.long)
         for t in range(algo["warm"], iters):
             ev.cfr_iteration(t)
+        if ev.use_final_policy_values:
+            ev.update_average_values_final()
         for s in STATE:
             x = getattr(ev, s).detach().numpy()
             out[f"{name}/state/{s}"] = np.ascontiguousarray(x[..., cols]).astype(np.float32)
@@ -212,8 +235,7 @@ def main(fused: bool = False) -> None:
         print(name, "sampled leaves", lb.shape[0], "streets", getattr(pbs.env, "street").tolist(), flush=True)
         out[f"{name}/beliefs"] = bel
         out[f"{name}/depth_offsets"] = np.array(ev.depth_offsets, dtype=np.int64)
-        out[f"{name}/settings"] = np.array([str(depth), str(iters), algo["cfr_type"], str(algo["cfr_plus"]),
-                                            str(algo["cfr_avg"]), str(algo["warm"]), str(algo["enforce_zero_sum"])])
+        out[f"{name}/settings"] = np.array([str(depth), str(iters), json.dumps(algo)])
         print(name, "nodes", ev.total_nodes, "depth offsets", ev.depth_offsets,
               {k: len(b) for k, b in batches.items()}, flush=True)
     # the env's own reset (hunl_tensor_env.py:219-346) from a seeded CPU generator: button, deck, stacks

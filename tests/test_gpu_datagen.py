@@ -12,7 +12,7 @@ from oracle import cards as OC
 from oracle import cfr as OCFR
 from oracle import chance as OCH
 from oracle import datagen as ODG
-from tests.test_oracle_datagen import BINS, case_settings, load_case, value_net_numpy
+from tests.test_oracle_datagen import BINS, case_settings, load_case, oracle_search_arguments, value_net_numpy
 
 pytestmark = pytest.mark.gpu
 H = 1326
@@ -97,10 +97,14 @@ def test_bet_amounts_match_oracle():
 def search_config(n, depth, iters, algo):
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.fused_cfr_hip import CFRType
-    cfg = river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0)
-    cfg.search.cfr_type = CFRType[algo["cfr_type"]]
-    cfg.search.cfr_plus, cfg.search.cfr_avg = algo["cfr_plus"], algo["cfr_avg"]
-    cfg.search.warm_start_iterations = algo["warm"]
+    cfg = river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=algo["delay"])
+    z = cfg.search
+    z.cfr_type = CFRType[algo["cfr_type"]]
+    z.cfr_plus, z.cfr_avg = algo["cfr_plus"], algo["cfr_avg"]
+    z.warm_start_iterations, z.warm_start_type, z.warm_start_multiplier = algo["warm"], algo["warm_type"], algo["warm_mult"]
+    z.dcfr_alpha, z.dcfr_beta, z.dcfr_gamma = algo["alpha"], algo["beta"], algo["gamma"]
+    z.dcfr_alpha_final, z.dcfr_beta_final, z.dcfr_gamma_final = algo["alpha_final"], algo["beta_final"], algo["gamma_final"]
+    z.value_targets_from_final_policy = algo["final_policy_values"]
     return cfg
 
 
@@ -128,6 +132,8 @@ def golden_evaluator(case, fused):
     ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))     # includes the warm start
     for t in range(algo["warm"], iters):
         ev.cfr_iteration(t)
+    if ev.use_final_policy_values:
+        ev.update_average_values_final()
     ev.chance_helper.FLOP_SAMPLE_SIZE, ev.chance_helper.NUM_PERM_SAMPLES = 0, 0
     return ev, r
 
@@ -149,18 +155,19 @@ def batch_as_dict(b):
 def close(got, exp, mask, rtol, atol, what):
     """Agreement on the entries of ``mask``; elsewhere (hands the board blocks, where the
     one-kernel evaluator and the base class legitimately differ) nothing is asserted.  At most
-    max(2, 1e-4 of the entries) may miss the tolerance — regret matching divides by small sums —
-    and none of those by more than 1e-4."""
+    max(2, 5e-4 of the entries) may miss the tolerance — regret matching divides by small sums —
+    and none of those by more than 1e-4 (the allowance the oracle itself needs against the same
+    fixtures, tests/test_oracle_datagen.py)."""
     m = np.broadcast_to(mask, got.shape)
     diff = np.abs(got - exp)[m]
     over = diff > (atol + rtol * np.abs(exp))[m]
-    assert over.sum() <= max(2, 1e-4 * diff.size) and (not over.any() or diff[over].max() < 1e-4), \
+    assert over.sum() <= max(2, 5e-4 * diff.size) and (not over.any() or diff[over].max() < 1e-4), \
         f"{what}: {int(over.sum())} of {diff.size} over tolerance, max abs diff {diff.max():.3e}"
 
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("fixture", ["base", "fused"])
-@pytest.mark.parametrize("name", ["streets_mixed", "preflop", "linear_avg_zero_sum"])
+@pytest.mark.parametrize("name", ["streets_mixed", "preflop", "linear_avg_zero_sum", "production_like"])
 def test_training_data_matches_vectors_from_the_reference(golden_dir, name, fused, fixture):
     """``fixture`` "base": written by the reference's SparseCFREvaluator, compared on the hands the
     board allows (the product follows the fused class, which differs from the base class on
@@ -226,7 +233,7 @@ def test_training_data_matches_vectors_from_the_reference(golden_dir, name, fuse
             assert not pt.transpose(0, 2, 1)[illegal].any()                          # no child, no probability
 
 
-@pytest.mark.parametrize("name", ["streets_mixed", "linear_avg_zero_sum_warm"])
+@pytest.mark.parametrize("name", ["streets_mixed", "linear_avg_zero_sum_warm", "production_like"])
 def test_training_data_matches_oracle_everywhere(golden_dir, name):
     """Against the oracle following the one-kernel evaluator's conventions: every entry, blocked
     hands included.  The second case (linear CFR with CFR+, cfr_avg, zero-sum network, warm start)
@@ -245,11 +252,12 @@ def test_training_data_matches_oracle_everywhere(golden_dir, name):
     _, iters, algo = case_settings(case)
     o = OCFR.OracleCFR(tree, r["board_indices"], case["beliefs"], cfr_iterations=iters, leaf_value_fn=leaf_fn,
                        t_sample_roots=np.full(ev.root_nodes, -1, dtype=np.int64), fused_variant=True,
-                       cfr_type=algo["cfr_type"], cfr_plus=algo["cfr_plus"], cfr_avg=algo["cfr_avg"],
-                       warm_start_iterations=algo["warm"], enforce_zero_sum=algo["enforce_zero_sum"])
+                       **oracle_search_arguments(algo))
     o.prepare()
     for t in range(algo["warm"], iters):
         o.cfr_iteration(t)
+    if o.use_final_policy_values:
+        o.update_average_values_final()
     canonical, count, _ = OCH.canonical_flops()
     exp = ODG.training_data(o, env, BINS, value_net_numpy, flop_tables=(canonical, count, OCH.combo_suit_perms()))
     got = [batch_as_dict(b) for b in ev.training_data()]
@@ -439,7 +447,7 @@ def test_leaf_model_does_not_reuse_features_of_the_previous_subgame():
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("fixture", ["base", "fused"])
-@pytest.mark.parametrize("name", ["streets_mixed", "preflop", "linear_avg_zero_sum"])
+@pytest.mark.parametrize("name", ["streets_mixed", "preflop", "linear_avg_zero_sum", "production_like"])
 def test_whole_search_from_a_seeded_generator_samples_the_reference_leaves(golden_dir, name, fused, fixture):
     """``evaluate_cfr`` with its random parts — the sampling schedule, the hand and exploration
     draws of the leaf walk (cfr_evaluator.py:1497-1528, :382-404, sparse_cfr_evaluator.py:325-426)

@@ -500,3 +500,45 @@ def test_b1024_three_raise_tree_200_iterations_invariants():
     # and the search did its job on every root: far less exploitable than the uniform start
     after = ev._compute_exploitability().local_exploitability
     assert (after < 0.5 * before).all() and after.max() < 0.15 and (after > -1e-4).all()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_negative_beta_from_iteration_zero(fused):
+    """beta = -1 is the reference's own setting.  At t = 0 the discount t**beta / (t**beta + 1) has
+    no value of its own (the reference raises on ``0 ** -1`` and only ever starts after a warm
+    start); the product uses its limit, 1.  Nothing has been accumulated at t = 0, so the first
+    iteration must not depend on beta at all, and later ones follow the oracle."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import discount_pair
+    from poker2_amd.tree import RootStates
+    assert discount_pair(0, -1.0) == (1.0, 1.0) and discount_pair(4, -1.0) == (0.25, 1.25)
+    assert discount_pair(0, 1.5) == (0.0, 1.0) and discount_pair(0, 0.0) == (1.0, 2.0)
+    rng = np.random.default_rng(8)
+    boards = random_boards(rng, 3)
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(3, np.full(3, 200), np.tile([[800, 800]], (3, 1)), boards, button=np.arange(3) % 2)
+
+    def run(beta, iters):
+        cfg = river_dcfr_config(3, iterations=8, depth=2, dcfr_delay=0)
+        cfg.search.dcfr_beta = beta
+        ev = HipSparseCFREvaluator(None, torch.device("cuda"), cfg, fused_iteration=fused)
+        ev.initialize_subgame(roots, np.arange(3), torch.from_numpy(beliefs))
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+        for t in range(iters):
+            ev.cfr_iteration(t)
+        return ev
+    first_neg, first_zero = run(-1.0, 1), run(0.0, 1)
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        assert torch.equal(getattr(first_neg, name), getattr(first_zero, name)), name
+    ev = run(-1.0, 5)
+    # the oracle, like the reference, cannot take t = 0 with a negative beta: give it beta = 0 for that iteration
+    orc = OCFR.OracleCFR(tree_as_dict(ev.tree), boards, beliefs, cfr_type="discounted", dcfr_alpha=1.5, dcfr_beta=0.0,
+                         dcfr_gamma=2.0, cfr_iterations=8, t_sample_roots=np.full(3, -1, dtype=np.int64),
+                         fused_variant=True)
+    orc.prepare()
+    orc.cfr_iteration(0)
+    orc.dcfr_beta = orc.dcfr_beta_initial = -1.0
+    for t in range(1, 5):
+        orc.cfr_iteration(t)
+    compare(ev, orc, rtol=2e-4, atol=2e-5)
