@@ -30,6 +30,10 @@ CASES = [
     ("flop_b1_d2", 1, [1.0], 2, [(200, 900, 900, 1)]),
     # street 0: the roots are the env's reset state (blinds posted); the row holds (pot, starting stacks, button)
     ("preflop_b2_d4", 0, [0.5, 1.0], 4, [(150, 1000, 1000, 0), (150, 1000, 1000, 1)]),
+    # the reference's own table (conf/config_rebel_cfr.yaml:66-70,72: blinds 5 / 10, 100 big blinds deep, depth 5);
+    # a last element gives (small blind, big blind), 50 / 100 where absent
+    ("preflop_deep_d5", 0, [0.5, 1.0], 5, [(15, 1000, 1000, 0), (15, 1000, 1000, 1), (15, 1700, 300, 0)], (5, 10)),
+    ("flop_deep_d5", 1, [0.5, 1.0], 5, [(20, 990, 990, 1), (60, 970, 970, 0), (400, 800, 800, 1)], (5, 10)),
 ]
 
 
@@ -39,15 +43,22 @@ def main() -> None:
     from p2.env.hunl_tensor_env import HUNLTensorEnv
 
     out = {}
-    for name, street, bins, depth, rows in CASES:
+    for name, street, bins, depth, rows, *rest in CASES:
         n = len(rows)
-        env = HUNLTensorEnv(num_envs=n, starting_stack=1000, sb=50, bb=100,
+        sb, bb = rest[0] if rest else (50, 100)
+        env = HUNLTensorEnv(num_envs=n, starting_stack=1000, sb=sb, bb=bb,
                             default_bet_bins=list(bins), device=torch.device("cpu"))
         deck = torch.arange(9).repeat(n, 1)
         env.reset(force_button=torch.tensor([r[3] for r in rows]), force_deck=deck)
         for _ in range(2 * street):
             env.step_bins(torch.ones(n, dtype=torch.long))
         assert (env.street == street).all() and (env.actions_this_round == 0).all()
+        if street == 0 and any(r[1] != 1000 or r[2] != 1000 for r in rows):
+            # unequal starting stacks at the reset state: what reset leaves, with other stacks behind the blinds
+            start = torch.tensor([[r[1], r[2]] for r in rows])
+            env.stacks[:] = start - env.committed
+            env.starting_stacks[:] = start
+            env.scale[:] = start[:, 0].float()
         if street > 0:
             pot = torch.tensor([r[0] for r in rows])
             stacks = torch.tensor([[r[1], r[2]] for r in rows])
@@ -91,6 +102,7 @@ def main() -> None:
             full.copy_state_from(e, torch.arange(e.N), torch.arange(cur, cur + e.N))
             cur += e.N
         out[f"{name}/bins"] = np.asarray(bins, dtype=np.float64)
+        out[f"{name}/blinds"] = np.asarray([sb, bb], dtype=np.int64)
         out[f"{name}/depth"] = np.asarray(depth)
         out[f"{name}/roots"] = np.asarray(rows, dtype=np.int64)
         out[f"{name}/root_street"] = np.asarray(street)

@@ -81,3 +81,24 @@ def test_device_builder_from_preflop_roots():
     roots = RootStates.preflop(n, starting_stacks=rng.integers(150, 20000, (n, 2)), button=rng.integers(0, 2, n))
     same_tree(build_sparse_tree(roots, [0.5, 1.0], 5, max_raises=3),
               build_sparse_tree_device(roots, [0.5, 1.0], 5, max_raises=3))
+
+
+def test_device_builder_on_the_reference_env_fixture(golden_dir):
+    """Every case of tests/golden/tree_golden.npz (written by the reference's HUNLTensorEnv: river,
+    turn, flop and reset-state roots, three bin sets, depths 2-12, the 50 / 100 and the 5 / 10
+    blinds) straight through the device builder."""
+    from poker2_amd.tree import build_sparse_tree_device
+    from tests.test_tree import STATE_KEYS, cases, roots_of
+    seen = 0
+    for name, case in cases(golden_dir):
+        roots, _, _ = roots_of(case)
+        t = build_sparse_tree_device(roots, [float(x) for x in case["bins"]], int(case["depth"]))
+        assert t.depth_offsets == list(case["depth_offsets"]), name
+        assert np.array_equal(t.parent_index, case["parent_index"]), name
+        assert np.array_equal(t.action_from_parent, case["action_from_parent"]), name
+        assert np.array_equal(t.legal_mask, case["legal_mask"]), name
+        for k in STATE_KEYS:
+            assert np.array_equal(t.state[k], case[k].astype(t.state[k].dtype)), (name, k)
+        assert np.array_equal(t.reward[t.fold_mask], case["reward"][t.fold_mask]), name
+        seen += 1
+    assert seen >= 9

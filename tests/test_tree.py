@@ -22,12 +22,14 @@ def roots_of(case):
     r = case["roots"]
     pot, stacks, button = r[:, 0], r[:, 1:3], r[:, 3]
     street = int(case["root_street"])
+    sb, bb = (int(x) for x in case["blinds"]) if "blinds" in case else (50, 100)
     if street == 0:      # reset state: the row holds the starting stacks
-        return (RootStates.preflop(len(r), starting_stacks=stacks, button=button),
-                [OT.make_preflop_root(int(s[0]), int(s[1]), button=int(b)) for s, b in zip(stacks, button)])
-    prod = RootStates.at_round_start(street, pot, stacks, np.full((len(r), 5), -1), button=button)
-    orac = [OT.make_root(street, int(p), int(s[0]), int(s[1]), button=int(b)) for p, s, b in zip(pot, stacks, button)]
-    return prod, orac
+        return (RootStates.preflop(len(r), starting_stacks=stacks, button=button, sb=sb, bb=bb),
+                [OT.make_preflop_root(int(s[0]), int(s[1]), button=int(b), sb=sb, bb=bb) for s, b in zip(stacks, button)],
+                bb)
+    prod = RootStates.at_round_start(street, pot, stacks, np.full((len(r), 5), -1), button=button, bb=bb)
+    orac = [OT.make_root(street, int(p), int(s[0]), int(s[1]), button=int(b), bb=bb) for p, s, b in zip(pot, stacks, button)]
+    return prod, orac, bb
 
 
 def test_builders_match_reference_env_fixture(golden_dir):
@@ -35,9 +37,9 @@ def test_builders_match_reference_env_fixture(golden_dir):
     for name, case in cases(golden_dir):
         bins = [float(x) for x in case["bins"]]
         depth = int(case["depth"])
-        prod, orac = roots_of(case)
+        prod, orac, bb = roots_of(case)
         t = build_sparse_tree(prod, bins, depth)
-        o = OT.build_tree(orac, bins, depth)
+        o = OT.build_tree(orac, bins, depth, bb=bb)
         assert t.depth_offsets == list(case["depth_offsets"]) == o["depth_offsets"], name
         assert np.array_equal(t.parent_index, case["parent_index"]) and np.array_equal(o["parent_index"], case["parent_index"])
         assert np.array_equal(t.action_from_parent, case["action_from_parent"])
@@ -53,7 +55,7 @@ def test_builders_match_reference_env_fixture(golden_dir):
             assert np.array_equal(getattr(t, k), o[k]), (name, k)
         assert np.array_equal(t.showdown_potential, o["showdown_potential"])
         n += 1
-    assert n >= 7
+    assert n >= 9
 
 
 def test_hand_derived_river_tree():
