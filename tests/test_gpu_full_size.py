@@ -150,3 +150,67 @@ def test_data_generation_step_B16384():
     rows = torch.from_numpy(rows).to(DEV)
     for name in ("policy_probs_avg", "beliefs_avg", "values_avg"):
         same_but_few(getattr(big, name)[rows], getattr(ref, name), name)
+
+
+def test_generator_with_the_reference_production_settings():
+    """The self-play loop with every search setting of the reference's own configuration
+    (conf/config_rebel_cfr.yaml: 192 hands, blinds 5 / 10 at 100 big blinds, bins 0.5 / 1 pot,
+    depth 5, discounted_plus with delay, `model` warm start x 10, alpha 2->4 / beta -1->-2 /
+    gamma 5->0 schedules, value targets from the final average strategy, a zero-sum network),
+    iterations scaled down from 200 / 15 / 80 to 16 / 3 / 6.  Properties only: the loop runs for
+    several passes, hands advance and are replaced, every batch is finite and in range."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType
+    from poker2_amd.leaf_models import NetworkLeafModel, RangeBoardMLP
+    from poker2_amd.rebel_data_generator import EnvProto, RebelDataGenerator
+    n = 192
+    dev = torch.device(DEV)
+    cfg = river_dcfr_config(n, iterations=16, depth=5, dcfr_delay=6)
+    z = cfg.search
+    z.cfr_type, z.cfr_plus, z.cfr_avg = CFRType.discounted_plus, False, False
+    z.warm_start_iterations, z.warm_start_type, z.warm_start_multiplier = 3, "model", 10.0
+    z.dcfr_alpha, z.dcfr_alpha_final, z.dcfr_beta, z.dcfr_beta_final = 2.0, 4.0, -1.0, -2.0
+    z.dcfr_gamma, z.dcfr_gamma_final = 5.0, 0.0
+    z.value_targets_from_final_policy = True
+    cfg.env.bet_bins, cfg.env.bb = [0.5, 1.0], 10
+    env_gen = torch.Generator(device="cpu")
+    env_gen.manual_seed(3)
+    search_gen = torch.Generator(device=dev)
+    search_gen.manual_seed(4)
+    net = RangeBoardMLP(hidden=256, layers=2).to(dev)
+    model = NetworkLeafModel(net, dev, enforce_zero_sum=True, autocast_dtype=torch.bfloat16)
+    ev = HipSparseCFREvaluator(model, dev, cfg, generator=search_gen)
+
+    class Buffer:
+        def __init__(self):
+            self.batches = []
+
+        def add_batch(self, batch):
+            self.batches.append(batch)
+    value_buffer, policy_buffer = Buffer(), Buffer()
+    dg = RebelDataGenerator(EnvProto(mean_stack=1000, sb=5, bb=10, randomize_stacks=True, rng=env_gen), ev,
+                            value_buffer, policy_buffer)
+    assert (dg.current_pbs.env.pot == 15).all() and (dg.current_pbs.env.min_raise == 10).all()
+    streets_seen = set()
+    for _ in range(3):
+        value_batch, policy_batch = dg.generate_data(300)
+        assert len(value_batch) >= 300 - n and len(policy_batch) > 0
+        streets_seen |= set(np.asarray(dg.current_pbs.env.street).tolist())
+    passes = len(policy_buffer.batches)
+    assert passes >= 4 and len(value_buffer.batches) == 2 * passes
+    assert len(streets_seen) >= 2                                        # hands moved on to later streets
+    for i, b in enumerate(value_buffer.batches):
+        if len(b) == 0:
+            continue
+        vt = b.value_targets
+        assert torch.isfinite(vt).all() and torch.isfinite(b.features.beliefs).all()
+        if i % 2 == 0:
+            assert float(vt.abs().max()) <= 1.0                          # the clamped batch
+        s = b.features.beliefs.view(len(b), 2, H).sum(-1)
+        torch.testing.assert_close(s, torch.ones_like(s), rtol=0, atol=1e-4)
+    for b in policy_buffer.batches:
+        pt = b.policy_targets
+        assert torch.isfinite(pt).all() and not pt.permute(0, 2, 1)[~b.legal_masks].any()
+        mass = pt.sum(-1)
+        assert ((mass - 1).abs() < 1e-4).logical_or(mass.abs() < 1e-6).all()
