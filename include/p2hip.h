@@ -329,15 +329,28 @@ typedef struct P2HipIterArgs {
   float* scratch;
   const float* fscal;
   const int64_t* iscal;
+  /* Optional work items (both NULL: one item per root, item w = root w, n_items = roots).
+   * root_parent_offsets / root_showdown_offsets then have n_items + 1 entries and delimit, per item,
+   * the families and showdown rows one workgroup walks; item_root [n_items] names the root an item
+   * belongs to.  With few roots a root's tree may be cut at a level into a top item (item_top = 1: the
+   * families and showdown rows above the cut) and one subtree item per node of the cut level that has
+   * children (item_top = 0); every family and showdown row belongs to exactly one item.  An iteration
+   * is then four launches: all items with phases 4, top items with 8, subtree items with 8|2, top items
+   * with 2 (the regret part of a family reads rows that the reach / belief part of the family above
+   * rewrites, so it runs everywhere first). */
+  const int64_t* item_root;
+  const uint8_t* item_top;
 } P2HipIterArgs;
 
 /* One workgroup per root runs the whole iteration of FusedSparseCFREvaluator.cfr_iteration
  * (search/fused_sparse_cfr_evaluator.py:478-533; base search/cfr_evaluator.py:1330-1381) with
  * cfr_avg = False: sample snapshot, instantaneous regrets, DCFR update, regret matching, reach,
- * beliefs, average policy, reach_avg, beliefs_avg (phases bit 0); showdown leaf values, value
- * backup, average values (phases bit 1).  host_args is a HOST pointer to a struct of device
- * pointers; max_children = largest child count in the tree (<= 8). */
-int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max_children, int phases,
+ * beliefs, average policy, reach_avg, beliefs_avg (phases bit 0; bit 2 = the regret part alone, bit 3 = the
+ * reach / belief / average-policy part alone); showdown leaf values, value backup, average values
+ * (phases bit 1).  host_args is a HOST pointer to a struct of device
+ * pointers; n_items = workgroups to launch (= roots unless the work-item lists are given);
+ * max_children = largest child count in the tree (<= 8). */
+int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max_children, int phases,
                         void* stream);
 
 /* Copy 8 floats and 8 int64 from HOST arrays into the device arrays fscal[8] / iscal[8] read by

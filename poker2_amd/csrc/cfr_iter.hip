@@ -69,8 +69,23 @@ struct IterArgs {
   // iteration-dependent scalars in device memory
   const float* fscal;    // t_alpha_num, t_beta_num, t_alpha_den, t_beta_den, mix_old, mix_new, mix_total, mix_inv_total
   const int64_t* iscal;  // t, apply_dcfr, cfr_plus, avg_policy_copy, enforce_zero_sum, update_avg_values, cfr_avg, linear
-  int phases;            // bit 0: sweeps 1+2, bit 1: sweep 3
+  // Work items (optional; null = one item per root, item w is root w).  An item is a run of the
+  // root_parents / root_showdown_nodes lists that one workgroup walks: a whole root, or — to fill
+  // the chip when there are few roots — the top of a root's tree above a cut level (item_top = 1)
+  // or the subtree under one node of the cut level (item_top = 0).  Every family and every
+  // showdown row belongs to exactly one item; item_root[w] is the root the item belongs to.
+  const int64_t* item_root;
+  const uint8_t* item_top;
+  int phases;            // PHASE_* bits
 };
+
+// Which sweeps a launch runs.  Sweep 1 of a family reads its parent's beliefs, values and reach_avg
+// as the PREVIOUS iteration left them; sweep 2 needs sweep 1 of its family and sweep 2 of its
+// ancestors (it rewrites the rows sweep 1 of the families below reads); sweep 3 needs sweep 2 of its
+// subtree and sweep 3 of its descendants.  Inside one workgroup that walks a whole root the three
+// simply follow each other (PHASE_12 | PHASE_3).  With a root split into work items it takes four
+// launches: every item sweep 1, tree tops sweep 2, subtrees sweeps 2 + 3, tree tops sweep 3.
+constexpr int PHASE_12 = 1, PHASE_3 = 2, PHASE_1 = 4, PHASE_2 = 8;
 
 constexpr int IT_VSTRIDE = P2_H + 2;  // floats between vectors staged in LDS
 constexpr int IT_RED = 20;            // block-reduction slots: 2 + 2 * 8 children, rounded up
@@ -179,8 +194,10 @@ template <int MAXC>
 __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(IterArgs A) {
   constexpr int IT_CHUNK = ItChunk<MAXC>::value;
   __shared__ IterLds<IT_CHUNK> L;
-  const int64_t r = blockIdx.x;
-  const int64_t pp0 = A.root_parent_offsets[r], pp1 = A.root_parent_offsets[r + 1];
+  const int64_t w = blockIdx.x;                               // work item: indexes the per-item lists
+  const int64_t r = A.item_root ? A.item_root[w] : w;         // its root: root-level inputs (ranges, board, table)
+  const bool top = A.item_top ? A.item_top[w] != 0 : true;    // the item's first family is the root's own
+  const int64_t pp0 = A.root_parent_offsets[w], pp1 = A.root_parent_offsets[w + 1];
 
   Lane ln;
   IT_FOR(j) {
@@ -204,11 +221,11 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
   const bool cfr_avg = A.iscal[6] != 0, linear = A.iscal[7] != 0;
   const float* leaf_beliefs = cfr_avg ? A.beliefs_avg : A.beliefs;
 
-  if (A.phases & 1) {
+  if (A.phases & (PHASE_12 | PHASE_1)) {
     // ---------------- sweep 1: regrets -> DCFR -> regret matching ----------------
     PROF_BEGIN(t_s1);
     const bool take_sample = A.t_sample[r] == t_now;
-    {
+    if (top) {
       // The root row takes part in the flat DCFR update like every other row: its regret is
       // zero (never positive), so only its weight sum moves.
       float2 ws[IT_PPT];
@@ -236,10 +253,11 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
         if (u < nch) {
           const int64_t p = A.root_parents[i0 + u];
           const int actor = (int)A.to_act[p];
-          float2 bo[IT_PPT], tmp[IT_PPT];
+          float2 bo[IT_PPT];
           ld(bo, leaf_beliefs, p * 2 + (1 - actor), ln);
-          ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
           to_lds(L.u.vecs[u], bo, ln);
+          float2 tmp[IT_PPT];
+          ld(tmp, A.reach_avg, p * 2 + actor, ln);  // the mix in sweep 2 needs the pre-update value
           st(A.scratch, p, tmp, ln);
         }
       }
@@ -321,8 +339,10 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
       p2_sync_lds();  // the staged vectors and L.cs are rewritten by the next chunk
     }
     PROF_END(0, t_s1);
-    PROF_BEGIN(t_s2);
+  }
 
+  if (A.phases & (PHASE_12 | PHASE_2)) {
+    PROF_BEGIN(t_s2);
     // ---------------- sweep 2: reach, beliefs, average policy ----------------
     // (re-reads policy / reach rows that the same lane wrote: no cross-lane hand-off)
     float2 rb[2][IT_PPT], rba[2][IT_PPT], ap[IT_PPT];
@@ -510,10 +530,10 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
     PROF_END(1, t_s2);
   }
 
-  if (A.phases & 2) {
+  if (A.phases & PHASE_3) {
     // ---------------- sweep 3a: showdown leaves ----------------
     PROF_BEGIN(t_s3);
-    const int64_t sd0 = A.root_showdown_offsets[r], sd1 = A.root_showdown_offsets[r + 1];
+    const int64_t sd0 = A.root_showdown_offsets[w], sd1 = A.root_showdown_offsets[w + 1];
     if (sd1 > sd0 && A.tables) {
       PROF_BEGIN(t_sd);
       ShowdownRegs sdr;
@@ -636,7 +656,7 @@ __global__ __launch_bounds__(IT_BLOCK, IT_MIN_WAVES) void cfr_iteration_kernel(I
       }
       st(A.latest, p * 2, vp[0], ln);
       st(A.latest, p * 2 + 1, vp[1], ln);
-      if (i == pp0 && update_avg) {
+      if (i == pp0 && update_avg && top) {
         // the root is nobody's child: update its average values here
         float2 nv[2][IT_PPT];
         float s4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -730,12 +750,14 @@ int p2hip_upload_floats(float* dst, const float* host_values, int n, void* strea
 
 // P2HipIterArgs (include/p2hip.h) mirrors p2::IterArgs field by field.
 
-int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max_children, int phases,
+int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max_children, int phases,
                         void* stream) {
-  if (!host_args || n_roots < 0 || max_children < 1 || max_children > 8 || (phases & ~3) || phases == 0)
+  if (!host_args || n_items < 0 || n_items > 0x7FFFFFFF || max_children < 1 || max_children > 8 || (phases & ~15) ||
+      phases == 0)
     return P2_EINVAL;
-  if (n_roots == 0) return 0;
+  if (n_items == 0) return 0;
   const P2HipIterArgs& h = *host_args;
+  if ((h.item_root == nullptr) != (h.item_top == nullptr)) return P2_EINVAL;
   const void* required[] = {h.child_offsets, h.child_count, h.to_act, h.node_flags, h.root_parent_offsets, h.root_parents,
                             h.root_showdown_offsets,  // root_showdown_nodes is empty (null) without showdown rows
                             h.t_sample, h.allowed, h.allowed_prob, h.potential, h.scale, h.policy, h.policy_avg,
@@ -756,8 +778,9 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_roots, int max
   a.policy_sample = h.policy_sample; a.cum = h.cum; a.wsum = h.wsum; a.beliefs = h.beliefs;
   a.beliefs_avg = h.beliefs_avg; a.reach = h.reach; a.reach_avg = h.reach_avg; a.latest = h.latest;
   a.values_avg = h.values_avg; a.scratch = h.scratch; a.fscal = h.fscal; a.iscal = h.iscal;
+  a.item_root = h.item_root; a.item_top = h.item_top;
   a.phases = phases;
-  const dim3 grid((unsigned)n_roots), block(p2::IT_BLOCK);
+  const dim3 grid((unsigned)n_items), block(p2::IT_BLOCK);
   if (max_children <= 5)
     hipLaunchKernelGGL((p2::cfr_iteration_kernel<5>), grid, block, 0, (hipStream_t)stream, a);
   else

@@ -56,7 +56,22 @@ class _IterArgs(ctypes.Structure):
         "child_offsets", "child_count", "to_act", "node_flags", "root_parent_offsets", "root_parents",
         "root_showdown_offsets", "root_showdown_nodes", "t_sample",
         "allowed", "allowed_prob", "tables", "potential", "scale", "policy", "policy_avg", "policy_sample", "cum",
-        "wsum", "beliefs", "beliefs_avg", "reach", "reach_avg", "latest", "values_avg", "scratch", "fscal", "iscal")]
+        "wsum", "beliefs", "beliefs_avg", "reach", "reach_avg", "latest", "values_avg", "scratch", "fscal", "iscal",
+        "item_root", "item_top")]
+
+
+# Sweeps a launch of the iteration kernel runs (include/p2hip.h): 1 = regrets + reach/beliefs, 2 = values,
+# 4 = regrets alone, 8 = reach/beliefs alone.
+_PHASE_12, _PHASE_3, _PHASE_1, _PHASE_2 = 1, 2, 4, 8
+# One workgroup per root fills the chip (256 CUs x 3 resident workgroups) from 768 roots on.  Below
+# SPLIT_ROOTS_BELOW roots each root's tree is cut at level SPLIT_CUT_LEVEL into work items (the top of
+# the tree, and one subtree per node of that level) that get a workgroup each.  Measured on the
+# three-raise river tree (105 nodes per root), ms per iteration unsplit -> split: 96 roots 1.28 -> 0.71,
+# 192 roots 1.40 -> 1.01, 384 roots 1.82 -> 1.66, 767 roots 2.90 -> 2.63 (and slower than unsplit on
+# another tree); a cut right under the root leaves subtrees whose chain of families is as long as
+# half the tree, deeper cuts put more of the tree into the few top items.
+SPLIT_ROOTS_BELOW = 512
+SPLIT_CUT_LEVEL = 2
 
 
 def _cfr_type_name(x) -> str:
@@ -103,7 +118,8 @@ class _TreeEnv(SimpleNamespace):
 class HipSparseCFREvaluator:
     def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
                  compile_model: bool = True, fused_iteration: bool = True,
-                 max_raises: int | None = None, tree_builder: str = "device") -> None:
+                 max_raises: int | None = None, tree_builder: str = "device",
+                 split_small_batches: bool | None = None) -> None:
         self.model = model
         self.device = torch.device(device)
         self.cfg = cfg
@@ -146,6 +162,8 @@ class HipSparseCFREvaluator:
         if tree_builder not in ("device", "host"):
             raise ValueError("tree_builder must be 'device' or 'host'")
         self.tree_builder = tree_builder     # both give identical trees; 'host' is the numpy builder
+        # None: split each root into several workgroups when there are too few roots to fill the chip
+        self.split_small_batches = split_small_batches
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -161,6 +179,7 @@ class HipSparseCFREvaluator:
         self._fscal_host = (ctypes.c_float * 8)()
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
+        self._iter_args_sub = None
         self._chance_helper = None
         self.subgame_serial = 0
 
@@ -291,6 +310,63 @@ class HipSparseCFREvaluator:
         self._max_children = int(tree.child_count.max()) if T else 1
         self._has_model_leaves = bool(model_mask.any())
         self._iter_args = None
+        self._iter_args_sub = None
+        split = self.split_small_batches
+        if split is None:
+            split = N < SPLIT_ROOTS_BELOW
+        self._items = self._split_items(tree) if split else None
+
+    def _split_items(self, tree: SparseTree):
+        """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h):
+        items 0..N-1 are the tops of the roots' trees above the cut level, items N.. the subtrees under
+        the cut level's nodes that have children.  Returns device arrays (family rows + offsets, showdown
+        rows + offsets, item_root, item_top) and the number of subtree items; None if the tree is too
+        shallow to cut."""
+        N, T = self.root_nodes, tree.total
+        offs = tree.depth_offsets
+        n_levels = len(offs) - 1
+        has_children = tree.child_count > 0
+        cut = min(SPLIT_CUT_LEVEL, n_levels - 2)
+        while cut >= 1 and not has_children[offs[cut]:offs[cut + 1]].any():
+            cut -= 1                                            # the deepest level that still has families below it
+        if cut < 1:
+            return None
+        anchor = np.full(T, -1, dtype=np.int64)                 # the cut-level node a deeper row sits under (itself there)
+        anchor[offs[cut]:offs[cut + 1]] = np.arange(offs[cut], offs[cut + 1])
+        for d in range(cut + 1, n_levels):
+            rows = np.arange(offs[d], offs[d + 1])
+            anchor[rows] = anchor[tree.parent_index[rows]]
+        subs = np.nonzero(has_children[offs[cut]:offs[cut + 1]])[0] + offs[cut]        # ascending rows
+        M = len(subs)
+
+        def grouped(rows, keys, groups):
+            """rows ordered by group (ascending inside a group) and offsets [len(groups) + 1]."""
+            slot = np.searchsorted(groups, keys)
+            order = np.argsort(slot, kind="stable")
+            counts = np.bincount(slot, minlength=len(groups))
+            return rows[order], np.concatenate([[0], np.cumsum(counts)])
+        roots = np.arange(N)
+        upper = np.nonzero(has_children[:offs[cut]])[0]
+        top_parents, top_po = grouped(upper, tree.root_index[upper], roots)
+        upper_sd = np.nonzero(tree.showdown_mask[:offs[cut + 1]])[0]
+        top_sd, top_so = grouped(upper_sd, tree.root_index[upper_sd], roots)
+        deep = np.arange(offs[cut], T)
+        sub_parent_rows = deep[has_children[deep]]
+        sub_parents, sub_po = grouped(sub_parent_rows, anchor[sub_parent_rows], subs)
+        deep_sd = np.arange(offs[cut + 1], T)
+        deep_sd = deep_sd[tree.showdown_mask[deep_sd]]
+        sub_sd, sub_so = grouped(deep_sd, anchor[deep_sd], subs)
+        parents = np.concatenate([top_parents, sub_parents]).astype(np.int64)
+        parent_offsets = np.concatenate([top_po, top_po[-1] + sub_po[1:]]).astype(np.int64)
+        showdown = np.concatenate([top_sd, sub_sd]).astype(np.int64)
+        showdown_offsets = np.concatenate([top_so, top_so[-1] + sub_so[1:]]).astype(np.int64)
+        item_root = np.concatenate([roots, tree.root_index[subs]]).astype(np.int64)
+        item_top = np.concatenate([np.ones(N, np.uint8), np.zeros(M, np.uint8)])
+        _req(len(parents) == int(has_children.sum()) and len(showdown) == int(tree.showdown_mask.sum()),
+             "every family and every showdown row must belong to exactly one work item")
+        return SimpleNamespace(parents=self._t(parents), parent_offsets=self._t(parent_offsets),
+                               showdown=self._t(showdown), showdown_offsets=self._t(showdown_offsets),
+                               item_root=self._t(item_root), item_top=self._t(item_top), n_sub=M, cut=cut)
 
     def initialize_subgame(self, src_env, src_indices, initial_beliefs: torch.Tensor | None = None) -> None:
         """cfr_evaluator.py:770-828."""
@@ -571,14 +647,42 @@ class HipSparseCFREvaluator:
         a.reach, a.reach_avg = p(self.self_reach), p(self.self_reach_avg)
         a.latest, a.values_avg, a.scratch = p(self.latest_values), p(self.values_avg), p(self._scratch)
         a.fscal, a.iscal = p(self._fscal), p(self._iscal)
+        it = self._items
+        if it is not None:
+            a.root_parent_offsets, a.root_parents = p(it.parent_offsets), p(it.parents)
+            a.root_showdown_offsets, a.root_showdown_nodes = p(it.showdown_offsets), p(it.showdown)
+            a.item_root, a.item_top = p(it.item_root), p(it.item_top)
         return a
 
+    def _launch_items(self, args: _IterArgs, n_items: int, phases: int) -> None:
+        if n_items == 0:
+            return
+        code = _lib.load().p2hip_cfr_iteration(ctypes.byref(args), n_items, self._max_children, phases,
+                                               _lib.stream_ptr())
+        _lib.check(code, "p2hip_cfr_iteration")
+
     def _launch_iteration(self, phases: int) -> None:
+        """``phases``: 1 = regrets, policy, reach, beliefs; 2 = leaf values and backup; 3 = both."""
         if self._iter_args is None:
             self._iter_args = self._build_iter_args()
-        code = _lib.load().p2hip_cfr_iteration(ctypes.byref(self._iter_args), self.root_nodes, self._max_children,
-                                               phases, _lib.stream_ptr())
-        _lib.check(code, "p2hip_cfr_iteration")
+            if self._items is not None:
+                # the subtree items alone: the same lists entered behind the N root items
+                sub, N = self._build_iter_args(), self.root_nodes
+                sub.root_parent_offsets += 8 * N
+                sub.root_showdown_offsets += 8 * N
+                sub.item_root += 8 * N
+                sub.item_top += N
+                self._iter_args_sub = sub
+        if self._items is None:
+            self._launch_items(self._iter_args, self.root_nodes, phases)
+            return
+        N, M = self.root_nodes, self._items.n_sub
+        if phases & _PHASE_12:
+            self._launch_items(self._iter_args, N + M, _PHASE_1)          # regrets of every family, all items at once
+            self._launch_items(self._iter_args, N, _PHASE_2)              # tree tops, top-down
+        self._launch_items(self._iter_args_sub, M, (_PHASE_2 if phases & _PHASE_12 else 0) | (phases & _PHASE_3))
+        if phases & _PHASE_3:
+            self._launch_items(self._iter_args, N, _PHASE_3)              # the tops' backup comes last
 
     def cfr_iteration(self, t: int) -> None:
         """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533)."""

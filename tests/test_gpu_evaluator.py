@@ -542,3 +542,59 @@ def test_negative_beta_from_iteration_zero(fused):
     for t in range(1, 5):
         orc.cfr_iteration(t)
     compare(ev, orc, rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("cut", [1, 2, 9])
+@pytest.mark.parametrize("seed", range(10))
+def test_split_work_items_give_bit_identical_results(seed, cut, monkeypatch):
+    """With few roots the iteration kernel gives every root several workgroups: the tree is cut at a
+    level (1: right under the root; 2: the default; 9: as deep as families go), the top of each tree
+    is one work item, every subtree under the cut another, and an iteration takes four launches
+    instead of one.  Every family still goes through the same arithmetic, so all eleven state
+    tensors must be bit-identical to the one-workgroup-per-root launch — over random trees, CFR variants, mid-round roots, a sampling
+    iteration, river and (odd seeds) turn roots; depth-limit and street-end leaves get their values
+    from a leaf model between the two halves of an iteration."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType
+    from poker2_amd.tree import RootStates
+    import poker2_amd.evaluator as evaluator_module
+    monkeypatch.setattr(evaluator_module, "SPLIT_CUT_LEVEL", cut)
+    rng = np.random.default_rng(7000 + seed)
+    n = int(rng.integers(1, 7))
+    bins = sorted(rng.choice([0.25, 0.5, 0.75, 1.0, 2.0], size=int(rng.integers(1, 5)), replace=False).tolist())
+    depth = int(rng.integers(2, 6))
+    max_raises = [None, 2, 3][int(rng.integers(0, 3))]
+    cfr_type = ["discounted", "discounted_plus", "standard", "linear"][seed % 4]
+    street = 2 if seed % 2 else 3
+    boards = random_boards(rng, n)
+    if street == 2:
+        boards[:, 4] = -1
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(street, rng.integers(40, 900, n), rng.integers(30, 2500, (n, 2)), boards,
+                                      button=rng.integers(0, 2, n), bb=int(rng.choice([10, 100])))
+
+    class LeafModel:                       # a deterministic stand-in for the value network
+        enforce_zero_sum = bool(seed % 3 == 0)
+
+        def leaf_values(self, bel, rows, ev):
+            return 0.3 * torch.flip(bel, dims=[1]) * 50.0 - 0.01
+
+    def run(split):
+        cfg = river_dcfr_config(n, iterations=12, depth=depth, dcfr_delay=int(seed % 3))
+        cfg.search.cfr_type = CFRType[cfr_type]
+        cfg.search.cfr_plus, cfg.search.cfr_avg = bool(seed % 2), bool((seed // 2) % 2)
+        cfg.env.bet_bins = bins
+        ev = HipSparseCFREvaluator(LeafModel(), torch.device("cuda"), cfg, max_raises=max_raises,
+                                   split_small_batches=split)
+        ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+        assert (ev._items is not None) == split
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), 2, dtype=torch.long))
+        for t in range(5):
+            ev.cfr_iteration(t)
+        return ev
+    a, b = run(True), run(False)
+    assert a._items.n_sub > 0 and 1 <= a._items.cut <= cut
+    for name in OCFR.OracleCFR.STATE_NAMES:
+        assert torch.equal(getattr(a, name), getattr(b, name)), \
+            f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type} street {street}: {name}"
