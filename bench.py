@@ -11,7 +11,8 @@ resident in HBM before the timed region.  Prints ONE JSON line:
                on the launch stream) against the 8 TB/s HBM peak
   cpu_baseline the numpy oracle (a CPU restatement of the reference's torch path) timed on
                this box's host cores on a small sample of the same workload
-  extra        showdown evaluations/s (B=4096 boards) and 7-card hands ranked/s (2^20 hands)
+  extra        showdown evaluations/s (B=4096 boards), 7-card hands ranked/s (2^20 hands), and the
+               iteration at the reference's own batch of 192 roots
 """
 from __future__ import annotations
 
@@ -145,6 +146,20 @@ def side_metrics() -> dict:
     ms = ev0.elapsed_time(ev1) / reps
     out["rank7_hands_per_s"] = (1 << 20) / (ms * 1e-3)
     out["rank7_ms_per_call_2e20"] = ms
+    # the batch the reference's own settings search at a time (num_envs: 192), on the three-raise tree: few roots
+    # are cut into work items that get a workgroup each
+    small, _, _ = make_evaluator(192, "raise3", 42, iterations=64)
+    for t in range(1, 6):
+        small.cfr_iteration(t)
+    ev0.record()
+    for t in range(6, 6 + reps):
+        small.cfr_iteration(t)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / reps
+    out["iteration_ms_B192_three_raise_tree"] = ms
+    out["subgame_iterations_per_s_B192"] = 192 / (ms * 1e-3)
+    out["algorithmic_GBps_B192"] = BYTES_PER_NODE_ITER * small.total_nodes / (ms * 1e-3) / 1e9
     return out
 
 
@@ -192,7 +207,7 @@ def main() -> None:
     for k in range(args.steps):
         ev.prepare_replay(t)          # tiny scalar-upload kernel, outside the kernel timing
         starts[k].record()
-        ev.cfr_iteration(t)           # ONE launch of the iteration kernel
+        ev.cfr_iteration(t)           # ONE launch of the iteration kernel (four with fewer than 512 roots)
         ends[k].record()
         t += 1
     torch.cuda.synchronize()
