@@ -207,7 +207,7 @@ def main() -> None:
     for k in range(args.steps):
         ev.prepare_replay(t)          # tiny scalar-upload kernel, outside the kernel timing
         starts[k].record()
-        ev.cfr_iteration(t)           # ONE launch of the iteration kernel (four with fewer than 512 roots)
+        ev.cfr_iteration(t)           # ONE launch of the iteration kernel (four with fewer than 400 roots)
         ends[k].record()
         t += 1
     torch.cuda.synchronize()

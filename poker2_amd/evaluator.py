@@ -68,9 +68,10 @@ _PHASE_12, _PHASE_3, _PHASE_1, _PHASE_2 = 1, 2, 4, 8
 # the tree, and one subtree per node of that level) that get a workgroup each.  Measured on the
 # three-raise river tree (105 nodes per root), ms per iteration unsplit -> split: 96 roots 1.28 -> 0.71,
 # 192 roots 1.40 -> 1.01, 384 roots 1.82 -> 1.66, 767 roots 2.90 -> 2.63 (and slower than unsplit on
-# another tree); a cut right under the root leaves subtrees whose chain of families is as long as
+# another tree); depth-2 tree (21 nodes per root): 96 roots 0.21 -> 0.13, 384 roots 0.36 -> 0.34, 500 roots
+# 0.38 -> 0.42; a cut right under the root leaves subtrees whose chain of families is as long as
 # half the tree, deeper cuts put more of the tree into the few top items.
-SPLIT_ROOTS_BELOW = 512
+SPLIT_ROOTS_BELOW = 400
 SPLIT_CUT_LEVEL = 2
 
 
