@@ -107,3 +107,17 @@ def test_argument_guards_hold_under_python_O():
     left = [p for p in glob.glob(os.path.join(root, "poker2_amd", "*.py"))
             if re.search(r"^\s*assert\b", open(p).read(), re.M)]
     assert left == [], left
+
+
+def test_bench_refuses_more_than_one_gpu_and_has_the_contract_flags():
+    """bench.py measures one GPU; asked for more it says so and exits without touching a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "bench.py", "--gpus", "2", "--steps", "1", "--warmup", "0"], cwd=root,
+                         capture_output=True, text=True, timeout=300)
+    assert res.returncode == 2 and "ONE GPU" in res.stderr and res.stdout.strip() == ""
+    helptext = subprocess.run([sys.executable, "bench.py", "--help"], cwd=root, capture_output=True, text=True,
+                              timeout=300).stdout
+    for flag in ("--gpus", "--steps", "--warmup"):
+        assert flag in helptext
