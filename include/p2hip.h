@@ -83,12 +83,15 @@ int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64
  * board, in (i, c) ascending order: post_beliefs[s] = the ranges with the hands that hold c or
  * a board card removed, renormalised per player (uniform over the allowed hands when the sum
  * is <= 1e-12); board_samples[s] = the board with c in its first empty slot; root_lookup[s] = i.
- * sample_offsets [n+1] int64 (device) = prefix sums of 52 - cards on board.  Replaces the
+ * sample_offsets [n+1] int64 (device) = prefix sums of 52 - cards on board.  source_rows = rows of
+ * pre_beliefs / board, total_samples = rows the three outputs hold: a state whose row index lies
+ * outside 0..source_rows-1 is skipped and no sample at or beyond total_samples is written, so
+ * offsets that disagree with the boards cannot make the kernel leave its buffers.  Replaces the
  * expansion half of ChanceNodeHelper.single_card_chance_values,
  * search/chance_node_helper.py:394-443. */
 int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
-                        const int64_t* sample_offsets, float* post_beliefs, int64_t* board_samples,
-                        int64_t* root_lookup, void* stream);
+                        const int64_t* sample_offsets, int64_t source_rows, int64_t total_samples,
+                        float* post_beliefs, int64_t* board_samples, int64_t* root_lookup, void* stream);
 
 /* expected[i] = mean of hand_values [S,2,H] over samples sample_offsets[i] .. sample_offsets[i+1]
  * (index_add_ + divide of search/chance_node_helper.py:467-477). */

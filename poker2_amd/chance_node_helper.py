@@ -88,6 +88,9 @@ def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, 
     board = board_pre.to(device=dev, dtype=torch.int64).contiguous()
     roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
     b = roots.numel()
+    source_rows = min(pre.shape[0], board.shape[0])
+    if b and (int(roots.min()) < 0 or int(roots.max()) >= source_rows):
+        raise IndexError("root_indices out of range")
     on_board = ((board[roots] >= 0) & (board[roots] < 52)).sum(dim=1)
     offsets = torch.zeros(b + 1, dtype=torch.int64, device=dev)
     torch.cumsum(52 - on_board, dim=0, out=offsets[1:])
@@ -102,8 +105,11 @@ def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, 
     post = torch.empty(total, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     board_samples = torch.empty(total, 5, dtype=torch.int64, device=dev)
     root_lookup = torch.empty(total, dtype=torch.int64, device=dev)
+    # With ``cards_on_board`` given the sample count is taken on trust; the kernel gets the buffers'
+    # size and writes nothing beyond it if a board holds fewer cards than claimed.
     _lib.call("p2hip_chance_expand", _lib.ptr(pre), _lib.ptr(roots), _lib.ptr(board), b, _lib.ptr(offsets),
-              _lib.ptr(post), _lib.ptr(board_samples), _lib.ptr(root_lookup), _lib.stream_ptr())
+              source_rows, total, _lib.ptr(post), _lib.ptr(board_samples), _lib.ptr(root_lookup),
+              _lib.stream_ptr())
     return post, board_samples, root_lookup, offsets
 
 

@@ -44,6 +44,7 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
                                                                   const int64_t* __restrict__ root_indices,
                                                                   const int64_t* __restrict__ board,
                                                                   const int64_t* __restrict__ sample_offsets,
+                                                                  int64_t source_rows, int64_t total_samples,
                                                                   float* __restrict__ post_beliefs,
                                                                   int64_t* __restrict__ board_samples,
                                                                   int64_t* __restrict__ root_lookup) {
@@ -51,6 +52,7 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
   __shared__ double cs[2 * P2_CARDS];
   const int64_t i = blockIdx.x;
   const int64_t root = root_indices ? root_indices[i] : i;
+  if (root < 0 || root >= source_rows) return;   // uniform per workgroup: nothing to read, nothing written
   int bcards[5];
   uint64_t bits;
   const int ncards = chance_board(board + root * 5, bcards, bits);
@@ -102,6 +104,9 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
   int64_t s = sample_offsets[i] + c_begin - __popcll(bits & ((1ull << c_begin) - 1ull));
   for (int c = c_begin; c < c_end; ++c) {
     if ((bits >> c) & 1ull) continue;
+    // the caller sized the outputs for `total_samples`; a state with fewer cards on its board than
+    // the caller assumed would run past them
+    if (s < 0 || s >= total_samples || ncards >= 5) break;
     const float sum0 = (float)(total0 - cs[c]);
     const float sum1 = (float)(total1 - cs[P2_CARDS + c]);
     const bool ok0 = sum0 > 1e-12f, ok1 = sum1 > 1e-12f;
@@ -449,15 +454,16 @@ __global__ __launch_bounds__(CH_BLOCK) void orbit_mean_kernel(const float* __res
 extern "C" {
 
 int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
-                        const int64_t* sample_offsets, float* post_beliefs, int64_t* board_samples,
-                        int64_t* root_lookup, void* stream) {
-  if (n < 0) return P2_EINVAL;
+                        const int64_t* sample_offsets, int64_t source_rows, int64_t total_samples,
+                        float* post_beliefs, int64_t* board_samples, int64_t* root_lookup, void* stream) {
+  if (n < 0 || source_rows < 0 || total_samples < 0) return P2_EINVAL;
   if (n == 0) return 0;
   if (!pre_beliefs || !board || !sample_offsets || !post_beliefs || !board_samples || !root_lookup) return P2_EINVAL;
   if (!p2_aligned8(pre_beliefs) || !p2_aligned8(post_beliefs)) return P2_EINVAL;
   if (n > 0x7FFFFFFF) return P2_EINVAL;
   hipLaunchKernelGGL(p2::chance_expand_kernel, dim3((unsigned)n, p2::CH_SPLIT), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
-                     pre_beliefs, root_indices, board, sample_offsets, post_beliefs, board_samples, root_lookup);
+                     pre_beliefs, root_indices, board, sample_offsets, source_rows, total_samples, post_beliefs,
+                     board_samples, root_lookup);
   P2_LAUNCH_CHECK();
   return 0;
 }

@@ -13,7 +13,7 @@
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.
-int p2hip_abi_version(void) { return 1; }
+int p2hip_abi_version(void) { return 2; }
 // Number of visible HIP devices (0 when there is none); never throws.
 int p2hip_device_count(void) {
   int n = 0;

@@ -21,8 +21,9 @@ Leaf model protocol (the value network itself stays ordinary PyTorch): ``model``
     leaf_values(beliefs[K,2,1326], node_rows[K], evaluator) -> [K,2,1326]
     policy_logits(beliefs[T,2,1326], node_rows[K], evaluator) -> [K,1326,A]   (optional)
 
-Out of scope here (host-side, post-search): leaf sampling, training-data assembly,
-exploitability statistics, warm start.
+Also here, either side of the iterations: warm start (``warm_start``), leaf sampling
+(``sample_leaves``), training-data assembly (``training_data``) and the local best response /
+exploitability statistics (``_compute_exploitability``).
 """
 from __future__ import annotations
 
@@ -171,6 +172,7 @@ class HipSparseCFREvaluator:
         self.tree_depth = 0
         self.depth_offsets = [0]
         self.last_model_values = None
+        self._last_model_values_buf = None
         self._t_scalars = F.TScalars(self.device, dtype=self.float_dtype)
         self._skip_t_scalars_update = False
         self._skip_record_stats = True
@@ -619,7 +621,14 @@ class HipSparseCFREvaluator:
                                               beliefs[self.model_indices].contiguous(), self._t_scalars.mix_onon,
                                               self._t_scalars.mix_oon, unmixed, self.enforce_zero_sum)
             self.latest_values.index_copy_(0, self.model_indices, unmixed)
-        self.last_model_values = hv
+        # The previous network output lives in a buffer of its own (the reference pins it the same
+        # way, fused_sparse_cfr_evaluator.py:464-469): a captured graph keeps reading this address on
+        # every replay, and a network that reuses its output tensor cannot alias "last" and "current".
+        buf = self._last_model_values_buf
+        if buf is None or buf.shape != hv.shape or buf.dtype != hv.dtype:
+            buf = self._last_model_values_buf = torch.empty_like(hv)
+        buf.copy_(hv)
+        self.last_model_values = buf
 
     @torch.no_grad()
     def set_leaf_values(self, t: int, beliefs: torch.Tensor | None = None, *, showdown: bool = True) -> None:

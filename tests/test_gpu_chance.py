@@ -134,6 +134,19 @@ def test_helper_edge_cases(K):
                         cards_on_board=4)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+    # a state index outside the ranges is refused on the host ...
+    with pytest.raises(IndexError):
+        K.chance_expand(torch.from_numpy(pre).cuda(), torch.tensor([3]).cuda(), torch.from_numpy(boards).cuda())
+    # ... and a claimed card count above a board's real one (3 cards dealt, 4 claimed: 49 samples
+    # where 48 were sized) cannot make the kernel write past the buffers: it stops at their end
+    boards3 = boards.copy()
+    boards3[1, 3] = -1
+    c = K.chance_expand(torch.from_numpy(pre).cuda(), torch.arange(3).cuda(), torch.from_numpy(boards3).cuda(),
+                        cards_on_board=4)
+    torch.cuda.synchronize()
+    assert c[0].shape[0] == 3 * 48 and int(c[3][-1]) == 3 * 48 + 1      # offsets say 145, the buffers hold 144
+    assert torch.equal(c[0][:48], a[0][:48]) and torch.equal(c[2][:48], a[2][:48])
+    assert int(c[2].max()) <= 2 and int(c[2].min()) >= 0
 
 
 # ---- turn subgame: street-end leaves valued through the chance node + a small network --------

@@ -153,6 +153,69 @@ def test_fused_and_per_op_paths_agree_and_graph_replay():
         assert torch.equal(a, g), f"graph replay differs on {name}"
 
 
+@pytest.mark.parametrize("cfr_type", ["linear", "discounted"])
+def test_graph_replay_with_a_leaf_network_and_cfr_avg(cfr_type):
+    """cfr_avg de-averages the network's answer against its answer of the PREVIOUS iteration
+    (fused_sparse_cfr_evaluator.py:420-472).  A captured iteration reads that previous answer
+    from a fixed address on every replay, so it must sit in a buffer the evaluator owns; the
+    network here also returns the same output tensor every call, which would make "previous" and
+    "current" one tensor if the evaluator merely kept a reference.  Replays must equal eager
+    iterations bit for bit."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.fused_cfr_hip import CFRType, GraphedCFRIteration, _EvaluatorStateSnapshot
+    from poker2_amd.tree import RootStates
+    n, iters = 5, 9
+    rng = np.random.default_rng(91)
+    boards = random_boards(rng, n)
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(3, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards, button=np.arange(n) % 2)
+
+    class ReusingNetwork:                  # depends on the ranges, keeps ONE output tensor
+        enforce_zero_sum = True
+
+        def __init__(self):
+            self.out = None
+
+        def leaf_values(self, bel, rows, ev):
+            if self.out is None or self.out.shape != bel.shape:
+                self.out = torch.empty_like(bel)
+            torch.mul(torch.flip(bel, dims=[1]), 40.0, out=self.out)
+            self.out.sub_(0.02)
+            return self.out
+
+    def make():
+        cfg = river_dcfr_config(n, iterations=iters, depth=2, dcfr_delay=0)
+        cfg.search.cfr_type = CFRType[cfr_type]
+        cfg.search.cfr_avg = True
+        ev = HipSparseCFREvaluator(ReusingNetwork(), torch.device("cuda"), cfg, fused_iteration=True)
+        ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+        return ev
+    eager, graphed = make(), make()
+    assert eager._has_model_leaves
+    for t in range(3):
+        graphed.cfr_iteration(t)
+    assert graphed.last_model_values is not graphed.model.out
+    snap = _EvaluatorStateSnapshot.from_evaluator(graphed)
+    last = graphed.last_model_values.clone()
+    runner = GraphedCFRIteration(graphed)
+    runner.capture(t_capture=3, num_warmup=0)
+    snap.restore_to(graphed)               # rewind to the state after t = 2, previous answer included
+    graphed.last_model_values.copy_(last)
+    for t in range(iters):
+        eager.cfr_iteration(t)
+        if t >= 3:
+            runner.replay(t)
+            torch.cuda.synchronize()
+            for name in OCFR.OracleCFR.STATE_NAMES:
+                assert torch.equal(getattr(eager, name), getattr(graphed, name)), f"t={t}: replay differs on {name}"
+    assert torch.equal(eager.last_model_values, graphed.last_model_values)
+    # the de-averaging did run: the leaf rows are not the network's plain answer
+    leaf = eager.latest_values[eager.model_indices]
+    assert not torch.equal(leaf, eager.model.leaf_values(eager.beliefs_avg[eager.model_indices], None, eager))
+
+
 def test_structural_invariants_after_many_iterations():
     iters = 60
     ev, _ = make_pair(8, 16, 1, seed=3, fused=True, iters=iters)
