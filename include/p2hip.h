@@ -122,6 +122,18 @@ int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const 
 int p2hip_orbit_mean(const float* hand_values, int64_t n, int64_t n_flops, const float* weight, int accumulate,
                      float* out, float* workspace, int shares, void* stream);
 
+/* p2hip_orbit_mean without the workspace argument.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The partial sums of shares > 1 go to an array inside the
+ * library (P2HIP_ORBIT_SCRATCH_FLOATS float32 = 16 MiB per GPU, held until the process ends); the
+ * call allocates and frees nothing.  shares * n * 2 * 1326 floats must fit it: a larger request
+ * returns 2 (hipErrorOutOfMemory) before anything is launched.  Same results, bit for bit, as
+ * p2hip_orbit_mean with the same `shares`.  Every call on one GPU uses that GPU's array: calls
+ * that overlap on one GPU (different streams, threads) race; calls on one stream do not. */
+#define P2HIP_ORBIT_SCRATCH_FLOATS (4 * 1024 * 1024)
+int p2hip_orbit_mean_static(const float* hand_values, int64_t n, int64_t n_flops, const float* weight,
+                            int accumulate, float* out, int shares, void* stream);
+
 /* ---- either side of the search in data generation ------------------------------------------ */
 
 /* Context features and board of RebelFeatureEncoder.encode (models/mlp/rebel_feature_encoder.py:55-127)

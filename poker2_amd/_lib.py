@@ -43,6 +43,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_perm_mean": [_P, _L, _L, _P, _I, _P, _I, _P, _P, _I, _P],
     "p2hip_chance_mean": [_P, _P, _L, _P, _P],
     "p2hip_orbit_mean": [_P, _L, _L, _P, _I, _P, _P, _I, _P],
+    "p2hip_orbit_mean_static": [_P, _L, _L, _P, _I, _P, _I, _P],
     "p2hip_encode_context": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _L, _P, _P, _P],
     "p2hip_bet_amounts": [_P, _P, _P, _P, _L, _P, _I, _P, _P],
     "p2hip_policy_targets": [_P, _P, _L, _P, _P, _P, _I, _P, _P],

@@ -204,9 +204,18 @@ def _avg_over_perms(hand_values: torch.Tensor, perms: torch.Tensor) -> torch.Ten
     return mean.view(-1, NUM_HANDS)[:n].reshape(*lead, NUM_HANDS)
 
 
-def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+ORBIT_SCRATCH_FLOATS = 4 * 1024 * 1024     # P2HIP_ORBIT_SCRATCH_FLOATS of include/p2hip.h
+
+
+def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None, *,
+               static_scratch: bool = False) -> torch.Tensor:
     """``perm_mean`` over ALL 24 suit permutations: the orbit of a hand is its class of starting
-    hands (pair / suited / offsuit of the same ranks), so the mean is taken per class."""
+    hands (pair / suited / offsuit of the same ranks), so the mean is taken per class.
+
+    ``static_scratch=True`` (needs ``out``) takes the entry point that allocates nothing
+    (``p2hip_orbit_mean_static``): partial sums go to a 16 MiB array inside the library, so the
+    call can sit under graph capture; it refuses inputs whose partial sums do not fit and must
+    not overlap with another such call on the same GPU."""
     if not _lib.hip_is_available():
         raise RuntimeError("orbit_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(hand_values, "orbit_mean")
@@ -224,6 +233,18 @@ def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tenso
         _req(out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous(),
              "out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()")
     shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
+    if static_scratch:
+        if not accumulate:
+            raise ValueError("static_scratch=True allocates nothing: pass the output tensor as `out`")
+        if hv is not hand_values or w is not weight:
+            raise ValueError("static_scratch=True allocates nothing: hand_values and weight must already be "
+                             "contiguous float32 tensors on the GPU")
+        if shares > 1 and shares * b * 2 * NUM_HANDS > ORBIT_SCRATCH_FLOATS:
+            raise ValueError(f"{shares} shares x {b} states need {shares * b * 2 * NUM_HANDS} floats of partial sums; "
+                             f"the library's static array holds {ORBIT_SCRATCH_FLOATS}")
+        _lib.call("p2hip_orbit_mean_static", _lib.ptr(hv), b, k, _lib.ptr(w), 1, _lib.ptr(out), shares,
+                  _lib.stream_ptr())
+        return out
     workspace = torch.empty(shares, b, 2, NUM_HANDS, dtype=torch.float32, device=dev) if shares > 1 else None
     _lib.call("p2hip_orbit_mean", _lib.ptr(hv), b, k, _lib.ptr(w), int(accumulate), _lib.ptr(out),
               _lib.ptr(workspace), shares, _lib.stream_ptr())

@@ -14,6 +14,7 @@
 // range, cs[c] = its mass on hands holding c), so one card-sum pass per state serves all of
 // its 46-49 samples.  The expansion is a pure write stream (about 48 x 10.6 KB per state).
 #pragma once
+#include <mutex>
 #include "common.h"
 #include "unblocked.hip"
 
@@ -551,6 +552,69 @@ int p2hip_orbit_mean(const float* hand_values, int64_t n, int64_t n_flops, const
   const int64_t grid = (npairs + p2::CH_BLOCK - 1) / p2::CH_BLOCK;
   hipLaunchKernelGGL(p2::perm_reduce_kernel, dim3((unsigned)grid), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
                      (const float2*)workspace, shares, npairs, accumulate, (float2*)out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- the suit-orbit mean for callers that cannot allocate ---------------------------------------
+// Partial sums of p2hip_orbit_mean_static live in this file-scope array instead of a workspace the
+// caller allocates.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends.  In host code the array's NAME is only a handle for hipGetSymbolAddress: kernels and
+// copies take the per-device address resolved below.
+#define P2_ORBIT_SCRATCH_FLOATS (4 * 1024 * 1024)   /* 16 MiB; equals P2HIP_ORBIT_SCRATCH_FLOATS of include/p2hip.h */
+static __device__ __align__(256) float p2_orbit_scratch[P2_ORBIT_SCRATCH_FLOATS];
+
+namespace p2 {
+constexpr int SCRATCH_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+
+// Device address of the scratch array on the CURRENT device, resolved once per device.
+static int orbit_scratch_address(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= SCRATCH_MAX_DEVICES) return P2_EINVAL;
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(p2_orbit_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace p2
+
+int p2hip_orbit_mean_static(const float* hand_values, int64_t n, int64_t n_flops, const float* weight,
+                            int accumulate, float* out, int shares, void* stream) {
+  if (n < 0 || n_flops < 0 || shares < 1) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!hand_values || !weight || !out || !p2_aligned8(hand_values) || !p2_aligned8(out)) return P2_EINVAL;
+  if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
+  const int64_t per_share = (n_flops + shares - 1) / shares;
+  const int64_t npairs = n * 2 * P2_HPAIRS;
+  if (shares == 1) {   // no partial sums: the kernel writes the output itself
+    hipLaunchKernelGGL(p2::orbit_mean_kernel, dim3((unsigned)(2 * n), 1), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                       hand_values, weight, n_flops, per_share, accumulate, out, (int64_t)0);
+    P2_LAUNCH_CHECK();
+    return 0;
+  }
+  // [shares, n, 2, H] partial sums must fit the array; refused before anything is launched
+  if ((int64_t)shares * npairs * 2 > (int64_t)P2_ORBIT_SCRATCH_FLOATS) return (int)hipErrorOutOfMemory;
+  float* scratch = nullptr;
+  const int rc = p2::orbit_scratch_address(&scratch);
+  if (rc != 0) return rc;
+  // Nothing in the array has to start at zero: every (share, state, player) row the reduction reads is
+  // written in full by the first kernel, also by a share that holds no flop.
+  hipLaunchKernelGGL(p2::orbit_mean_kernel, dim3((unsigned)(2 * n), (unsigned)shares), dim3(p2::CH_BLOCK), 0,
+                     (hipStream_t)stream, hand_values, weight, n_flops, per_share, 0, scratch, npairs * 2);
+  P2_LAUNCH_CHECK();
+  const int64_t grid = (npairs + p2::CH_BLOCK - 1) / p2::CH_BLOCK;
+  hipLaunchKernelGGL(p2::perm_reduce_kernel, dim3((unsigned)grid), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+                     (const float2*)scratch, shares, npairs, accumulate, (float2*)out);
   P2_LAUNCH_CHECK();
   return 0;
 }
