@@ -64,3 +64,13 @@ def random_tree(rng: np.random.Generator, n_roots: int, depth: int, max_children
     return dict(depth_offsets=offsets, parent_index=parent, child_count=child_count, child_offsets=child_offsets,
                 to_act=to_act, prev_actor=prev_actor, root_index=root_index.astype(np.int64), total=total,
                 top=top, bottom=n_roots)
+
+
+def tree_as_dict(t):
+    """The arrays of a SparseTree that oracle.cfr.OracleCFR takes."""
+    d = {k: getattr(t, k) for k in ("depth_offsets", "parent_index", "action_from_parent", "child_count",
+                                    "child_offsets", "prev_actor", "legal_mask", "leaf_mask", "new_street_mask",
+                                    "fold_mask", "showdown_mask", "reward")}
+    d.update({k: t.state[k] for k in ("to_act", "done", "scale")})
+    d["showdown_potential"] = t.showdown_potential
+    return d

@@ -5,18 +5,9 @@ import pytest
 import torch
 
 from oracle import cfr as OCFR
-from tests.helpers import random_boards, random_ranges
+from tests.helpers import random_boards, random_ranges, tree_as_dict
 
 pytestmark = pytest.mark.gpu
-
-
-def tree_as_dict(t):
-    d = {k: getattr(t, k) for k in ("depth_offsets", "parent_index", "action_from_parent", "child_count",
-                                    "child_offsets", "prev_actor", "legal_mask", "leaf_mask", "new_street_mask",
-                                    "fold_mask", "showdown_mask", "reward")}
-    d.update({k: t.state[k] for k in ("to_act", "done", "scale")})
-    d["showdown_potential"] = t.showdown_potential
-    return d
 
 
 def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discounted", delay=0, cfr_plus=False,
@@ -267,30 +258,46 @@ def test_best_response_and_exploitability_match_oracle(depth, max_raises):
 def test_200_iterations_average_strategy_quality_and_root_values():
     """River subgames on the three-raise tree (105 nodes per root), 200 discounted-CFR iterations.
     Element-wise agreement cannot survive that long: the algorithm's thresholds make the
-    iteration chaotic (two ORACLE runs whose initial ranges differ by 2e-7 relative on 50 hands
-    differ by 0.36 in single policy entries and by 1.2e-3 in root values after 200 iterations).
-    What must agree is what a search returns: the root values and the quality of the average
-    strategy, measured by the reference's own local exploitability."""
+    iteration chaotic (tests/test_oracle_chaos.py measures it on the oracle alone).  What must agree
+    is what a search returns — root values, best-response values and the local exploitability of the
+    average strategy — and HOW WELL is measured here, not assumed: a second oracle run whose initial
+    ranges differ by 2e-7 relative (one float32 rounding) is the yardstick, and the product may sit no
+    further from the oracle than three times that twin does (with a floor of 2e-4, for quantities the
+    twin happens to reproduce)."""
     from oracle import best_response as OBR
     iters, n = 200, 2
     ev, orc = make_pair(n, 16, 3, seed=77, fused=True, iters=iters)
+    _, twin = make_pair(n, 16, 3, seed=77, fused=True, iters=iters)
+    rng = np.random.default_rng(5)
+    for arr in (twin.beliefs, twin.beliefs_avg):
+        arr[:n] *= (1.0 + 2e-7 * rng.standard_normal(arr[:n].shape)).astype(np.float32)
+    twin.root_pre_chance_beliefs = twin.beliefs[:n].copy()
+    twin.prepare()
     assert ev.total_nodes == 105 * n
     for t in range(iters):
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
+        twin.cfr_iteration(t)
         if t == 4:
             compare(ev, orc, rtol=2e-4, atol=2e-5)          # element-wise early on ...
         if t == 9:
             compare(ev, orc, rtol=1e-3, atol=1e-4)          # ... growing about tenfold per 25 iterations
     got = ev._compute_exploitability()
     expl, br = OBR.compute_exploitability(orc)
-    np.testing.assert_allclose(got.local_exploitability.cpu().numpy(), expl, rtol=0.05)
-    np.testing.assert_allclose(got.local_best_response_values.cpu().numpy(), br, atol=2e-3)
+    expl_twin, br_twin = OBR.compute_exploitability(twin)
+
+    def within_three_twins(name, product, oracle, twin_value, floor=2e-4):
+        product, oracle, twin_value = (np.asarray(x, dtype=np.float64) for x in (product, oracle, twin_value))
+        yard = max(float(np.abs(twin_value - oracle).max()), floor)
+        dist = float(np.abs(product - oracle).max())
+        assert dist <= 3.0 * yard, f"{name}: product {dist:.3e} from the oracle, perturbed oracle {yard:.3e}"
+    within_three_twins("local exploitability", got.local_exploitability.cpu().numpy(), expl, expl_twin)
+    within_three_twins("best-response values", got.local_best_response_values.cpu().numpy(), br, br_twin)
     assert (expl < 0.12).all()                              # started at 0.47-0.48 (uniform play)
-    root_gpu, root_orc = ev.values_avg[:n].cpu().numpy(), orc.values_avg[:n]
-    assert np.abs(root_gpu - root_orc).max() < 1e-2
+    root_gpu, root_orc, root_twin = ev.values_avg[:n].cpu().numpy(), orc.values_avg[:n], twin.values_avg[:n]
+    within_three_twins("root values per hand", root_gpu, root_orc, root_twin)
     w = orc.beliefs_avg[:n]
-    np.testing.assert_allclose((root_gpu * w).sum(-1), (root_orc * w).sum(-1), atol=1e-3)
+    within_three_twins("range-weighted root values", (root_gpu * w).sum(-1), (root_orc * w).sum(-1), (root_twin * w).sum(-1))
 
 
 @pytest.mark.parametrize("ws_type,mult", [("model", 10.0), ("model_br", 1.0)])
