@@ -13,6 +13,9 @@ from tests.helpers import random_boards
 
 pytestmark = pytest.mark.gpu
 H = 1326
+# searches whose leaf values come from a network: how far product and oracle may sit apart on the
+# entries the oracle determines, in tolerances (measured on the MI355X; see tests/parity.py)
+NETWORK_FACTOR = 5.0      # largest seen: 2.4
 
 
 @pytest.fixture(scope="module")
@@ -175,7 +178,8 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused, streets):
     from poker2_amd.leaf_models import ChanceLeafModel, RangeBoardMLP
     from poker2_amd.tree import RootStates
     from tests.helpers import random_ranges
-    from tests.test_gpu_evaluator import compare, tree_as_dict
+    from tests import parity as PAR
+    from tests.helpers import tree_as_dict
     rng = np.random.default_rng(12)
     n, iters = len(streets), 5
     streets = np.array(streets)
@@ -208,14 +212,19 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused, streets):
     orc = OCFR.OracleCFR(tree_as_dict(tree), boards, beliefs, cfr_iterations=iters, leaf_value_fn=leaf_fn,
                          t_sample_roots=np.full(n, -1, dtype=np.int64), fused_variant=True)
     orc.prepare()
-    compare(ev, orc, rtol=2e-4, atol=2e-5)
+    # The network runs through hipBLASLt here and numpy there, so leaf values differ by GEMM summation
+    # order, a few roundings of the network's output.  Which entries of the state that leaves open is
+    # measured on the oracle (tests/parity.py: twins that start a few roundings away); every other
+    # entry is held to NETWORK_FACTOR x (1e-5 relative + parity.ATOL).
+    pack = PAR.OracleWithTwins(orc, seed=12, n_twins=2, amp=3e-7)
+    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what="after the preparation step: ")
     assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3     # the network's values are not trivial
-    # the network runs through hipBLASLt here and numpy there: leaf values differ by GEMM summation
-    # order (~1e-6 relative) and regret matching divides by small regret sums, hence the wider bar
     for t in range(iters):
         ev.cfr_iteration(t)
-        orc.cfr_iteration(t)
-        compare(ev, orc, rtol=1e-3, atol=3e-4)
+        pack.cfr_iteration(t)
+        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what=f"t={t}: ")
+        print(f"t={t}: worst determined entry {PAR.worst_of(rep):.2f} tolerances, largest exempt share "
+              f"{max(r['exempt'] for r in rep.values()):.1e}")
 
 
 def test_helper_matches_vectors_from_the_reference_helper(K, golden_dir):
@@ -387,7 +396,8 @@ def test_preflop_subgame_with_flop_leaves_matches_oracle(K):
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.leaf_models import ChanceLeafModel, RangeBoardMLP
     from poker2_amd.tree import RootStates
-    from tests.test_gpu_evaluator import compare, tree_as_dict
+    from tests import parity as PAR
+    from tests.helpers import tree_as_dict
     rng = np.random.default_rng(14)
     n, iters = 2, 3
     boards = np.full((n, 5), -1, dtype=np.int64)
@@ -429,12 +439,15 @@ def test_preflop_subgame_with_flop_leaves_matches_oracle(K):
     orc = OCFR.OracleCFR(tree_as_dict(tree), boards, beliefs, cfr_iterations=iters, leaf_value_fn=leaf_fn,
                          t_sample_roots=np.full(n, -1, dtype=np.int64), fused_variant=True)
     orc.prepare()
-    compare(ev, orc, rtol=2e-4, atol=2e-5)
+    pack = PAR.OracleWithTwins(orc, seed=14, n_twins=2, amp=3e-7)      # as in the turn test above
+    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what="after the preparation step: ")
     assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3
     for t in range(iters):
         ev.cfr_iteration(t)
-        orc.cfr_iteration(t)
-        compare(ev, orc, rtol=1e-3, atol=3e-4)      # network through hipBLASLt vs numpy: GEMM summation order
+        pack.cfr_iteration(t)
+        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what=f"t={t}: ")
+        print(f"t={t}: worst determined entry {PAR.worst_of(rep):.2f} tolerances, largest exempt share "
+              f"{max(r['exempt'] for r in rep.values()):.1e}")
 
 
 def test_orbit_mean_equals_the_mean_over_all_24_permutations(K):

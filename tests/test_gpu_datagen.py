@@ -135,6 +135,7 @@ def golden_evaluator(case, fused):
     if ev.use_final_policy_values:
         ev.update_average_values_final()
     ev.chance_helper.FLOP_SAMPLE_SIZE, ev.chance_helper.NUM_PERM_SAMPLES = 0, 0
+    WORST.clear()
     return ev, r
 
 
@@ -152,17 +153,78 @@ def batch_as_dict(b):
     return host(out)
 
 
-def close(got, exp, mask, rtol, atol, what):
-    """Agreement on the entries of ``mask``; elsewhere (hands the board blocks, where the
-    one-kernel evaluator and the base class legitimately differ) nothing is asserted.  At most
-    max(2, 5e-4 of the entries) may miss the tolerance — regret matching divides by small sums —
-    and none of those by more than 1e-4 (the allowance the oracle itself needs against the same
-    fixtures, tests/test_oracle_datagen.py)."""
-    m = np.broadcast_to(mask, got.shape)
-    diff = np.abs(got - exp)[m]
-    over = diff > (atol + rtol * np.abs(exp))[m]
-    assert over.sum() <= max(2, 5e-4 * diff.size) and (not over.any() or diff[over].max() < 1e-4), \
-        f"{what}: {int(over.sum())} of {diff.size} over tolerance, max abs diff {diff.max():.3e}"
+# Training targets sit behind a whole search (4-12 iterations of regret matching), so product and
+# reference differ by accumulated roundings.  Exemptions are by cause, as in tests/parity.py: the
+# oracle runs the same search, twice more from a state a few roundings away, and an entry of a target
+# is exempt if either twin moves it by more than a third of the tolerance; every other entry is held
+# to TARGET_FACTOR x (1e-5 relative + the absolute part below).  Largest seen on the MI355X: see the
+# printed reports; the exempt share of a tensor is capped.
+TARGET_ATOL = {"beliefs": 1e-7, "value_targets": 2e-6, "policy_targets": 1e-6}
+TARGET_FACTOR = 5.0
+TARGET_MAX_EXEMPT = 0.35
+LOOP_FACTOR = 30.0     # largest seen: 13.3
+
+
+def oracle_with_twins(case, ev, r, fused_variant=True, n_twins=2):
+    """The oracle's training data of the case's search and that of `n_twins` perturbed twins."""
+    from tests import parity as PAR
+    from tests.helpers import tree_as_dict
+    tree = tree_as_dict(ev.tree)
+    tree.update({k: v for k, v in ev.tree.state.items() if k not in tree})
+    env = ODG.tree_env(tree, r["board_indices"])
+
+    def leaf_fn(beliefs, rows):
+        f = ODG.encode(env, beliefs, pre_chance_node=tree["new_street_mask"], indices=rows)
+        return value_net_numpy(f["context"], f["street"], f["to_act"], f["board"], f["beliefs"])
+    _, iters, algo = case_settings(case)
+    o = OCFR.OracleCFR(tree, r["board_indices"], case["beliefs"], cfr_iterations=iters, leaf_value_fn=leaf_fn,
+                       t_sample_roots=np.full(ev.root_nodes, -1, dtype=np.int64), fused_variant=fused_variant,
+                       **oracle_search_arguments(algo))
+    o.prepare()
+    pack = PAR.OracleWithTwins(o, n_twins=n_twins, amp=3e-7, seed=21)
+    for t in range(algo["warm"], iters):
+        pack.cfr_iteration(t)
+    canonical, count, _ = OCH.canonical_flops()
+    out = []
+    for x in [pack.base] + pack.twins:
+        if x.use_final_policy_values:
+            x.update_average_values_final()
+        out.append(ODG.training_data(x, env, BINS, value_net_numpy, flop_tables=(canonical, count, OCH.combo_suit_perms())))
+    return out[0], out[1:]
+
+
+def open_entries(exp, twins, field, batch):
+    """Entries of target `field` of batch number `batch` that the twins move by more than a third of
+    the tolerance (None if the batch has no such field)."""
+    def pick(d):
+        if field == "beliefs":
+            x = d[batch]["features"]["beliefs"]
+            return x.reshape(x.shape[0], 2, H)
+        return d[batch].get(field)
+    base = pick(exp)
+    if base is None:
+        return None
+    tol = (TARGET_ATOL[field] + 1e-5 * np.abs(base)) / 3.0
+    mask = np.zeros(base.shape, dtype=bool)
+    for tw in twins:
+        mask |= np.abs(pick(tw) - base) > tol
+    return mask
+
+
+WORST = {}
+
+
+def close(got, exp, compared, open_, field, what):
+    """`got` against `exp` on the entries of `compared` that are not `open_`."""
+    m = np.broadcast_to(compared, got.shape) & ~np.broadcast_to(open_, got.shape)
+    tol = TARGET_ATOL[field] + 1e-5 * np.abs(exp)
+    ratio = np.where(m, np.abs(got - exp) / tol, 0.0)
+    exempt = float(np.broadcast_to(open_, got.shape)[np.broadcast_to(compared, got.shape)].mean()) if got.size else 0.0
+    worst = float(ratio.max()) if ratio.size else 0.0
+    WORST[what] = max(WORST.get(what, 0.0), worst)
+    assert worst <= TARGET_FACTOR, f"{what}: {int((ratio > TARGET_FACTOR).sum())} of {int(m.sum())} determined " \
+                                   f"entries beyond {TARGET_FACTOR:g} tolerances, worst {worst:.2f}; exempt share {exempt:.2e}"
+    assert exempt <= TARGET_MAX_EXEMPT, f"{what}: {exempt:.2e} of the entries are exempt"
 
 
 @pytest.mark.parametrize("fused", [True, False])
@@ -190,8 +252,8 @@ def test_training_data_matches_vectors_from_the_reference(golden_dir, name, fuse
     if fixture == "fused":
         allowed_root = np.ones_like(allowed_root)
     batches = [batch_as_dict(b) for b in ev.training_data()]
-    rtol, atol = 3e-4, 3e-6          # float32; four iterations of regret matching behind the targets
-    for got, tag in zip(batches, ("value", "pre_value", "policy")):
+    exp_o, twins_o = oracle_with_twins(case, ev, r, fused_variant=fixture == "fused")
+    for bi, (got, tag) in enumerate(zip(batches, ("value", "pre_value", "policy"))):
         k = int(case[f"{tag}/len"])
         ft = got["features"]
         assert ft["context"].shape[0] == k
@@ -221,16 +283,20 @@ def test_training_data_matches_vectors_from_the_reference(golden_dir, name, fuse
         if tag == "pre_value":      # ranges before the deal: the hands the dealt cards block still carry mass
             np.testing.assert_allclose(fb[..., cols], case[f"{tag}/beliefs"], rtol=1e-6, atol=0)
         else:
-            close(fb[..., cols], case[f"{tag}/beliefs"], ok[:, None, cols], rtol, atol, f"{tag} beliefs")
+            close(fb[..., cols], case[f"{tag}/beliefs"], ok[:, None, cols],
+                  open_entries(exp_o, twins_o, "beliefs", bi)[..., cols], "beliefs", f"{tag} beliefs")
         if "value_targets" in got:
             mask = ok[:, None, :] if tag == "value" else np.ones((k, 1, H), bool)
-            close(got["value_targets"], case[f"{tag}/value_targets"], mask, rtol, atol, f"{tag} value targets")
+            close(got["value_targets"], case[f"{tag}/value_targets"], mask,
+                  open_entries(exp_o, twins_o, "value_targets", bi), "value_targets", f"{tag} value targets")
         if "policy_targets" in got:
             pt = got["policy_targets"]
             assert pt.shape == (k, H, len(BINS) + 3)
-            close(pt[:, cols, :], case[f"{tag}/policy_targets"], ok[:, cols, None], rtol, atol, "policy targets")
+            close(pt[:, cols, :], case[f"{tag}/policy_targets"], ok[:, cols, None],
+                  open_entries(exp_o, twins_o, "policy_targets", bi)[:, cols, :], "policy_targets", "policy targets")
             illegal = ~case[f"{tag}/legal_masks"]
             assert not pt.transpose(0, 2, 1)[illegal].any()                          # no child, no probability
+    print(name, fixture, "worst determined entry, in tolerances:", {k: round(v, 2) for k, v in WORST.items()})
 
 
 @pytest.mark.parametrize("name", ["streets_mixed", "linear_avg_zero_sum_warm", "production_like"])
@@ -239,45 +305,33 @@ def test_training_data_matches_oracle_everywhere(golden_dir, name):
     hands included.  The second case (linear CFR with CFR+, cfr_avg, zero-sum network, warm start)
     has no fused-class fixture — the reference's fused class cannot run its warm start there — so
     this comparison, with the oracle's base variant pinned on the same case, is what holds it."""
-    from tests.test_gpu_evaluator import tree_as_dict
     case, _ = load_case(golden_dir, name)
     ev, r = golden_evaluator(case, True)
-    tree = tree_as_dict(ev.tree)
-    tree.update({k: v for k, v in ev.tree.state.items() if k not in tree})
-    env = ODG.tree_env(tree, r["board_indices"])
-
-    def leaf_fn(beliefs, rows):
-        f = ODG.encode(env, beliefs, pre_chance_node=tree["new_street_mask"], indices=rows)
-        return value_net_numpy(f["context"], f["street"], f["to_act"], f["board"], f["beliefs"])
-    _, iters, algo = case_settings(case)
-    o = OCFR.OracleCFR(tree, r["board_indices"], case["beliefs"], cfr_iterations=iters, leaf_value_fn=leaf_fn,
-                       t_sample_roots=np.full(ev.root_nodes, -1, dtype=np.int64), fused_variant=True,
-                       **oracle_search_arguments(algo))
-    o.prepare()
-    for t in range(algo["warm"], iters):
-        o.cfr_iteration(t)
-    if o.use_final_policy_values:
-        o.update_average_values_final()
-    canonical, count, _ = OCH.canonical_flops()
-    exp = ODG.training_data(o, env, BINS, value_net_numpy, flop_tables=(canonical, count, OCH.combo_suit_perms()))
+    exp, twins = oracle_with_twins(case, ev, r)
     got = [batch_as_dict(b) for b in ev.training_data()]
 
-    def same(a, b, path):
+    def same(a, b, tw, path):
         if isinstance(b, dict):
             assert set(a) == set(b), path
             for k in b:
-                same(a[k], b[k], f"{path}/{k}")
+                same(a[k], b[k], [t[k] for t in tw], f"{path}/{k}")
         elif np.issubdtype(np.asarray(b).dtype, np.floating):
-            # float32; regret matching divides by small regret sums, so a handful of policy entries
-            # (and what is built from them) move by more than the 3e-4 of the rest
-            tol = (3e-3, 5e-5) if "local_" in path else (3e-4, 3e-6)
-            err = np.abs(a - b) - (tol[1] + tol[0] * np.abs(b))
-            assert (err > 0).sum() <= max(2, 1e-4 * err.size) and np.abs(a - b).max() < 1e-3, \
-                f"{path}: {(err > 0).sum()} entries off, max abs diff {np.abs(a - b).max():.3e}"
+            leaf = path.rsplit("/", 1)[-1]
+            if "local_" in path:                       # scalars out of the best-response pass
+                np.testing.assert_allclose(a, b, rtol=3e-3, atol=5e-5, err_msg=path)
+            elif leaf in TARGET_ATOL:
+                tol = (TARGET_ATOL[leaf] + 1e-5 * np.abs(b)) / 3.0
+                open_ = np.zeros(np.shape(b), dtype=bool)
+                for t in tw:
+                    open_ |= np.abs(t - b) > tol
+                close(a, b, np.ones(np.shape(b), dtype=bool), open_, leaf, path)
+            else:                                      # context features: the same float32 operations
+                np.testing.assert_allclose(a, b, rtol=1e-6, atol=0, err_msg=path)
         else:
             assert np.array_equal(a, b), path
-    for a, b, tag in zip(got, exp, ("value", "pre_value", "policy")):
-        same(a, b, tag)
+    for bi, (a, b, tag) in enumerate(zip(got, exp, ("value", "pre_value", "policy"))):
+        same(a, b, [t[bi] for t in twins], tag)
+    print(name, "worst determined entry, in tolerances:", {k: round(v, 2) for k, v in WORST.items()})
 
 
 def test_policy_targets_kernel_matches_pull_back_on_a_deep_tree():
@@ -502,15 +556,23 @@ def compare_generator_batch(g, prefix, batch, cols, every_entry):
     assert np.array_equal(f.street.cpu().numpy(), g[f"{prefix}/street"]), prefix
     assert np.array_equal(batch.legal_masks.cpu().numpy(), g[f"{prefix}/legal_masks"]), prefix
     ok = np.ones((n, H), bool) if every_entry else OC.allowed_hands_for_boards(board)[0]
-    rtol, atol = 3e-4, 3e-6
+    # No oracle runs this loop, so there are no twins to say which entries are open: every compared entry
+    # is held, without exemption, to LOOP_FACTOR x (1e-5 relative + TARGET_ATOL) — three iterations of
+    # regret matching per search, nine searches feeding one another (measured; the numerics of one
+    # search are what the tests above hold tightly).
+    def all_close(got, exp, compared, field, what):
+        m = np.broadcast_to(compared, got.shape)
+        ratio = np.where(m, np.abs(got - exp) / (TARGET_ATOL[field] + 1e-5 * np.abs(exp)), 0.0)
+        WORST[what.split("/")[-1]] = max(WORST.get(what.split("/")[-1], 0.0), float(ratio.max()))
+        assert ratio.max() <= LOOP_FACTOR, f"{what}: worst entry {ratio.max():.1f} tolerances (bound {LOOP_FACTOR:g})"
     fb = f.beliefs.cpu().numpy().reshape(n, 2, H)
-    close(fb[..., cols], g[f"{prefix}/beliefs"], ok[:, None, cols], rtol, atol, f"{prefix} beliefs")
+    all_close(fb[..., cols], g[f"{prefix}/beliefs"], ok[:, None, cols], "beliefs", f"{prefix} beliefs")
     if batch.value_targets is not None:
         vt = batch.value_targets.cpu().numpy()
-        close(vt[..., cols], g[f"{prefix}/value_targets"], ok[:, None, cols], rtol, atol, f"{prefix} value targets")
+        all_close(vt[..., cols], g[f"{prefix}/value_targets"], ok[:, None, cols], "value_targets", f"{prefix} value targets")
     if batch.policy_targets is not None:
         pt = batch.policy_targets.cpu().numpy()
-        close(pt[:, cols, :], g[f"{prefix}/policy_targets"], ok[:, cols, None], rtol, atol, f"{prefix} policy targets")
+        all_close(pt[:, cols, :], g[f"{prefix}/policy_targets"], ok[:, cols, None], "policy_targets", f"{prefix} policy targets")
 
 
 @pytest.mark.parametrize("fixture", ["base", "fused"])
@@ -526,6 +588,7 @@ def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
     g = np.load(str(golden_dir) + ("/fused_generator_golden.npz" if fixture == "fused" else "/generator_golden.npz"))
     n, depth, iters, asked, env_seed, search_seed = (int(x) for x in g["settings"])
     cols = g["columns"]
+    WORST.clear()
     env_gen, search_gen = torch.Generator(device="cpu"), torch.Generator(device="cpu")
     env_gen.manual_seed(env_seed)
     search_gen.manual_seed(search_seed)
@@ -565,4 +628,8 @@ def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
     same_states("left", dg.current_pbs.env)
     lb = dg.current_pbs.beliefs.cpu().numpy()
     ok = np.ones(lb.shape[::2], bool) if every else OC.allowed_hands_for_boards(g["left/board_indices"])[0]
-    close(lb[..., cols], g["left/beliefs"], ok[:, None, cols], 3e-4, 3e-6, "beliefs left behind")
+    ratio = np.where(ok[:, None, cols], np.abs(lb[..., cols] - g["left/beliefs"]) /
+                     (TARGET_ATOL["beliefs"] + 1e-5 * np.abs(g["left/beliefs"])), 0.0)
+    assert ratio.max() <= LOOP_FACTOR, f"beliefs left behind: worst entry {ratio.max():.1f} tolerances"
+    print(fixture, "loop: worst entry, in tolerances:", {k: round(v, 1) for k, v in WORST.items()},
+          "beliefs left behind", round(float(ratio.max()), 1))

@@ -1,10 +1,13 @@
 """GPU parity of the whole CFR iteration: the one-kernel path and the per-operation path of
 HipSparseCFREvaluator against the numpy oracle on seeded river subgames."""
+import copy
+
 import numpy as np
 import pytest
 import torch
 
 from oracle import cfr as OCFR
+from tests import parity as PAR
 from tests.helpers import random_boards, random_ranges, tree_as_dict
 
 pytestmark = pytest.mark.gpu
@@ -58,24 +61,47 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
     return ev, orc
 
 
-# Hard thresholds in the algorithm (showdown denominator > 1e-8, belief / policy sums > 1e-5,
-# regret sums > 1e-8) are discontinuities: when the exact value sits on a threshold (e.g. every
-# villain combo shares a card with the hero's hand, so the compatible mass is rounding noise
-# around 0) two correct float32 implementations may take different branches.  Such elements
-# are exempt by COUNT: at most FLIP_FRACTION of a tensor may miss the tolerance.
-FLIP_FRACTION = 1e-4
+# How far product and oracle may sit apart when BOTH run on their own, as a multiple of the
+# tolerance (1e-5 relative + parity.ATOL) on the entries the oracle determines; measured over every
+# case of this file on the MI355X (largest seen: 2.4 after the first iteration, 3.8 within eight).
+# From the second iteration on the inputs of an iteration differ by roundings and regret matching
+# — a quotient of differences of nearly equal values — amplifies them; that the iteration ITSELF
+# is right to well within the tolerance is what the one-step comparison shows.
+FREE_FACTOR_FIRST, FREE_FACTOR_LATER = 3.0, 5.0
+
+
+class Lockstep:
+    """The product, an oracle that iterates on its own (with perturbed twins, tests/parity.py) and
+    an oracle that is handed the product's state before every iteration."""
+
+    def __init__(self, ev, orc, seed=1):
+        self.ev = ev
+        self.free = PAR.OracleWithTwins(orc, seed=seed)
+        self.step = copy.deepcopy(orc)
+        self.worst_step, self.worst_free = 0.0, 0.0
+
+    def iterate(self, t, first=0):
+        PAR.set_state(self.step, PAR.state_of(self.ev))
+        self.ev.cfr_iteration(t)
+        self.free.cfr_iteration(t)
+        self.step.cfr_iteration(t)
+        got = PAR.state_of(self.ev)
+        rs = PAR.compare_step(got, self.step, what=f"t={t}, one step from the same state: ")
+        rf = PAR.compare_free(got, self.free, factor=FREE_FACTOR_FIRST if t == first else FREE_FACTOR_LATER,
+                              what=f"t={t}, free running: ")
+        self.worst_step = max([self.worst_step] + [r["worst_over_tol"] for r in rs.values()])
+        self.worst_free = max([self.worst_free] + [r["worst_over_tol"] for r in rf.values()])
 
 
 def compare(ev, orc, rtol, atol, names=None):
+    """Plain comparison at a stated tolerance, no exemptions (used where product and oracle were
+    just handed the same inputs, or by tests of other modules with their own tolerance)."""
     worst = {}
     for name in names or OCFR.OracleCFR.STATE_NAMES:
         a = getattr(ev, name).cpu().numpy()
         b = getattr(orc, name)
-        err = np.abs(a - b) - (atol + rtol * np.abs(b))
         worst[name] = float(np.abs(a - b).max())
-        bad = int((err > 0).sum())
-        assert bad <= FLIP_FRACTION * err.size, \
-            f"{name}: max abs diff {np.abs(a - b).max():.3e}, {bad} of {err.size} elements out of tolerance"
+        np.testing.assert_allclose(a, b, rtol=rtol, atol=atol, err_msg=name)
     return worst
 
 
@@ -90,10 +116,10 @@ def test_iterations_match_oracle(fused, depth, max_raises):
     iters = 8
     ev, orc = make_pair(3, depth, max_raises, seed=11 + depth, fused=fused, iters=iters,
                         t_sample=np.array([2, 5, 100]))
+    both = Lockstep(ev, orc)
     for t in range(iters):
-        ev.cfr_iteration(t)
-        orc.cfr_iteration(t)
-        compare(ev, orc, rtol=2e-4, atol=2e-5)
+        both.iterate(t)
+    print(f"worst entry: {both.worst_step:.2f} x tolerance one step, {both.worst_free:.2f} x free running")
     # the snapshot of root 0 was taken at t = 2, of root 1 at t = 5, root 2 never
     assert ev.policy_probs_sample[ev._root_index == 2].abs().max().item() == 0.0
     assert ev.policy_probs_sample[ev._root_index == 0].abs().max().item() > 0.0
@@ -111,10 +137,9 @@ def test_variants_fused_vs_oracle(cfr_type, delay, cfr_plus, zs, cfr_avg):
     ev, orc = make_pair(2, 2, None, seed=5, fused=True, iters=iters, cfr_type=cfr_type, delay=delay,
                         cfr_plus=cfr_plus, enforce_zs=zs, stacks=(500, 900), pot=300, bins=(0.33, 0.75, 1.5),
                         cfr_avg=cfr_avg)
+    both = Lockstep(ev, orc)
     for t in range(iters):
-        ev.cfr_iteration(t)
-        orc.cfr_iteration(t)
-    compare(ev, orc, rtol=2e-4, atol=2e-5)
+        both.iterate(t)
 
 
 def test_fused_and_per_op_paths_agree_and_graph_replay():
@@ -239,15 +264,24 @@ def test_best_response_and_exploitability_match_oracle(depth, max_raises):
     for name in OCFR.OracleCFR.STATE_NAMES:
         getattr(orc, name)[:] = getattr(ev, name).cpu().numpy()
     rng = np.random.default_rng(0)
+    # A hand whose two best children tie within rounding may pick either, which moves the OTHER
+    # player's values; which entries that leaves open is measured on the oracle (tests/parity.py):
+    # three copies of the state, every entry a few roundings away, and an entry is exempt if any
+    # copy moves it by more than a third of the tolerance.
+    twins = PAR.OracleWithTwins(orc, seed=9).twins
     for dev_np in (np.zeros(ev.total_nodes, np.int64), np.ones(ev.total_nodes, np.int64),
                    rng.integers(0, 2, ev.total_nodes), None):
         dev_t = None if dev_np is None else torch.from_numpy(dev_np).cuda()
         got = ev._best_response_values(ev.policy_probs_avg, ev.beliefs_avg, ev.values_avg, dev_t).cpu().numpy()
         exp = OBR.best_response_values(orc, orc.policy_probs_avg, orc.beliefs_avg, orc.values_avg, dev_np)
-        err = np.abs(got - exp) - (2e-6 + 1e-5 * np.abs(exp))       # float32: 1e-5 relative
-        # exempt by count: a hand whose two best children tie within rounding may pick the other
-        # child, which moves the OTHER player's value by O(1)
-        assert (err > 0).mean() <= FLIP_FRACTION, f"max abs diff {np.abs(got - exp).max():.3e}"
+        tol = 2e-6 + 1e-5 * np.abs(exp)                             # float32: 1e-5 relative
+        open_ = np.zeros(exp.shape, dtype=bool)
+        for tw in twins:
+            moved = OBR.best_response_values(tw, tw.policy_probs_avg, tw.beliefs_avg, tw.values_avg, dev_np)
+            open_ |= np.abs(moved - exp) > tol / 3.0
+        assert open_.mean() <= 0.05, f"{open_.mean():.2e} of the best-response values are undetermined"
+        bad = (np.abs(got - exp) > tol) & ~open_
+        assert not bad.any(), f"{int(bad.sum())} determined entries out of tolerance, worst {np.abs(got - exp)[~open_].max():.3e}"
     stats = ev._compute_exploitability()
     expl, br = OBR.compute_exploitability(orc)
     np.testing.assert_allclose(stats.local_exploitability.cpu().numpy(), expl, rtol=1e-4, atol=2e-6)
@@ -278,10 +312,6 @@ def test_200_iterations_average_strategy_quality_and_root_values():
         ev.cfr_iteration(t)
         orc.cfr_iteration(t)
         twin.cfr_iteration(t)
-        if t == 4:
-            compare(ev, orc, rtol=2e-4, atol=2e-5)          # element-wise early on ...
-        if t == 9:
-            compare(ev, orc, rtol=1e-3, atol=1e-4)          # ... growing about tenfold per 25 iterations
     got = ev._compute_exploitability()
     expl, br = OBR.compute_exploitability(orc)
     expl_twin, br_twin = OBR.compute_exploitability(twin)
@@ -305,12 +335,13 @@ def test_warm_start_matches_oracle(ws_type, mult):
     iters = 8
     ev, orc = make_pair(3, 16, 1, seed=41, fused=True, iters=iters, cfr_type="discounted_plus", delay=4,
                         warm_start=3, warm_start_type=ws_type, warm_start_multiplier=mult)
-    compare(ev, orc, rtol=2e-4, atol=2e-5)                  # state right after the warm start
+    # the state right after the warm start (one best-response pass or one regret-matching inversion)
+    PAR.compare_free(PAR.state_of(ev), PAR.OracleWithTwins(orc, n_twins=0), factor=FREE_FACTOR_FIRST,
+                     what="after the warm start: ")
     assert ev.regret_weight_sums[ev.root_nodes:].abs().max().item() > 0
+    both = Lockstep(ev, orc)
     for t in range(3, iters):
-        ev.cfr_iteration(t)
-        orc.cfr_iteration(t)
-    compare(ev, orc, rtol=5e-4, atol=5e-5)
+        both.iterate(t, first=3)
 
 
 def test_sample_leaves_walks_the_sampled_policy():
@@ -412,29 +443,34 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
     ev.prepare_search(t_sample=t_sample)
     cols = g["columns"]
     allowed = OC.allowed_hands_for_boards(board)[0][ev.tree.root_index][:, cols]       # [total, 64]
-    if fixture == "fused":
-        allowed = np.ones_like(allowed)
+    # which entries float32 arithmetic determines is measured on the oracle (perturbed twins,
+    # tests/parity.py), run alongside on the same search
+    from tests.test_oracle_cfr_golden import build
+    orc, _, _ = build({**{k: g[k] for k in g.files}, "fused_variant": fixture == "fused"}, name)
+    orc.prepare()
+    pack = PAR.OracleWithTwins(orc, seed=6)
+    names = [s for s in OCFR.OracleCFR.STATE_NAMES if s not in left_out]
+    worst = {}
 
-    def check(tag, rtol, atol):
-        for s in OCFR.OracleCFR.STATE_NAMES:
-            if s in left_out:
-                continue
-            got = getattr(ev, s).cpu().numpy()[..., cols]
-            exp = g[f"{name}/{tag}/{s}"]
-            m = allowed if got.ndim == 2 else np.broadcast_to(allowed[:, None, :], got.shape)
-            err = (np.abs(got - exp) - (atol + rtol * np.abs(exp)))[m]
-            assert (err > 0).sum() <= max(2, 2e-3 * err.size), \
-                f"{name} {tag} {s}: max abs diff {np.abs(got - exp)[m].max():.3e}"
-            assert np.abs(got - exp)[m].max() < 2e-3, f"{name} {tag} {s}"
-    check("prep", 1e-5, 2e-6)
+    def check(tag, factor):
+        got = {s: getattr(ev, s).cpu().numpy()[..., cols] for s in names}
+        expected = {s: g[f"{name}/{tag}/{s}"] for s in names}
+        blocked = None if fixture == "fused" else ~allowed
+        rep = PAR.compare_free(got, pack, factor=factor, names=names, expected=expected,
+                               select=lambda s, arr: arr[..., cols],
+                               also_exempt=None if blocked is None else
+                               (lambda s: blocked if got[s].ndim == 2 else blocked[:, None, :]),
+                               max_exempt=1.0 if blocked is not None else 0.25, what=f"{name} {tag}: ")
+        worst[tag] = max(r["worst_over_tol"] for r in rep.values())
+    check("prep", FREE_FACTOR_FIRST)
     stored = set(g[f"{name}/stored"].tolist())
     for t in range(int(warm), int(iters)):
         ev.cfr_iteration(t)
+        pack.cfr_iteration(t)
         if t in stored:
-            # float32 throughout; regret matching divides by small sums, so a relative 1e-5 in the
-            # regrets shows as ~5e-5 in a policy and in the reach products built from it
-            tol = 5e-5 if t < int(warm) + 2 else 3e-4
-            check(f"t{t}", tol, tol / 5)
+            check(f"t{t}", FREE_FACTOR_FIRST if t == int(warm) else FREE_FACTOR_LATER)
+    print(name, fixture, "fused" if fused else "per-op", "worst determined entry, in tolerances:",
+          {k: round(v, 2) for k, v in worst.items()})
     if left_out:
         return
     stats = ev._compute_exploitability()
@@ -609,9 +645,10 @@ def test_negative_beta_from_iteration_zero(fused):
     orc.prepare()
     orc.cfr_iteration(0)
     orc.dcfr_beta = orc.dcfr_beta_initial = -1.0
+    twins = PAR.OracleWithTwins(orc, seed=3)
     for t in range(1, 5):
-        orc.cfr_iteration(t)
-    compare(ev, orc, rtol=2e-4, atol=2e-5)
+        twins.cfr_iteration(t)
+    PAR.compare_free(PAR.state_of(ev), twins, factor=FREE_FACTOR_LATER, what="beta = -1, after five iterations: ")
 
 
 @pytest.mark.parametrize("cut", [1, 2, 9])

@@ -12,6 +12,9 @@ import pytest
 
 from oracle import cfr as OCFR
 from oracle import tree as OT
+from tests import parity as PAR
+
+FACTOR_PREP, FACTOR_FIRST, FACTOR_LATER = 2.0, 2.0, 5.0
 
 STATE = OCFR.OracleCFR.STATE_NAMES
 
@@ -48,43 +51,51 @@ def build(golden, name):
 NAN_IN_FUSED_REFERENCE = {"warm_model_d2": ("policy_probs_avg", "self_reach_avg", "beliefs_avg", "values_avg")}
 
 
-def check(o, golden, name, tag, rtol, atol):
+def check(pack, golden, name, tag, factor):
+    """The oracle against the reference's vectors on the stored hand columns: every entry the
+    arithmetic determines (tests/parity.py: perturbed twins of the oracle mark the rest) within
+    `factor` x (1e-5 relative + parity.ATOL); row sums over all 1326 hands as a second, coarser check
+    that covers the columns the fixture does not store."""
     cols = golden["columns"]
+    o = pack.base
+    names = []
     for s in STATE:
-        got = getattr(o, s)
         exp = golden[f"{name}/{tag}/{s}"]
         if golden["fused_variant"] and s in NAN_IN_FUSED_REFERENCE.get(name, ()):
             if s == "policy_probs_avg":
                 assert np.isnan(exp).any(), "the fixture no longer shows the reference's NaN: compare this case too"
             continue
         assert not np.isnan(exp).any(), (name, tag, s)
-        err = np.abs(got[..., cols] - exp) - (atol + rtol * np.abs(exp))
-        # hands whose regret sums are tiny amplify rounding (and some sit on the algorithm's hard
-        # thresholds): up to 0.2 % of the entries may miss the tolerance, none by more than 1e-3
-        assert (err > 0).sum() <= max(2, 2e-3 * err.size), \
-            f"{name} {tag} {s}: max abs diff {np.abs(got[..., cols] - exp).max():.3e}"
-        assert np.abs(got[..., cols] - exp).max() < 1e-3, f"{name} {tag} {s}"
-        np.testing.assert_allclose(got.astype(np.float64).sum(-1), golden[f"{name}/{tag}/{s}_rowsum"],
-                                   rtol=max(rtol, 1e-4), atol=1e-3, err_msg=f"{name} {tag} {s} row sums")
+        names.append(s)
+        np.testing.assert_allclose(getattr(o, s).astype(np.float64).sum(-1), golden[f"{name}/{tag}/{s}_rowsum"],
+                                   rtol=1e-4, atol=1e-3, err_msg=f"{name} {tag} {s} row sums")
+    got = {s: getattr(o, s) for s in names}
+    expected = {s: golden[f"{name}/{tag}/{s}"] for s in names}
+    return PAR.compare_free(got, pack, factor=factor, names=names, expected=expected,
+                            select=lambda s, arr: arr[..., cols], what=f"{name} {tag}: ")
 
 
 @pytest.mark.parametrize("name", ["discounted_d2", "dplus_d3", "linear_avg_d2", "linear_noplus_d2", "standard_d2",
                                   "warm_br_d2", "warm_model_d2", "warm_model_dplus_d2"])
 def test_oracle_iterations_match_reference_vectors(golden, name):
     o, warm, iters = build(golden, name)
-    o.prepare()                                   # includes the warm start of the last two cases
-    # after a warm start the state has been through one regret-matching division already
-    check(o, golden, name, "prep", rtol=1e-5 if warm == 0 else 5e-5, atol=2e-6 if warm == 0 else 1e-5)
+    o.prepare()                                   # includes the warm start of the last three cases
+    pack = PAR.OracleWithTwins(o, seed=4)
+    # numpy and torch add in a different order, so even the oracle sits a few roundings from the
+    # reference's own numbers; measured: within the tolerance after the preparation step, within
+    # twice it after the first iteration, within five times it for the rest of these short searches
+    rep = check(pack, golden, name, "prep", FACTOR_PREP)
+    worst = {"prep": max(r["worst_over_tol"] for r in rep.values())}
+    exempt = max(r["exempt"] for r in rep.values())
     stored = set(golden[f"{name}/stored"].tolist())
     for t in range(warm, iters):
-        o.cfr_iteration(t)
+        pack.cfr_iteration(t)
         if t in stored:
-            # float32, 1e-5 relative on the first iterations; rounding differences between numpy
-            # and torch reductions grow slowly afterwards
-            # regret matching divides by small sums: 1e-5 relative in the regrets is a few 1e-6
-            # absolute in a policy and in the reach products built from it
-            tol = (2e-5 if warm == 0 else 5e-5) if t < warm + 2 else 1e-4
-            check(o, golden, name, f"t{t}", rtol=tol, atol=tol / 2)
+            rep = check(pack, golden, name, f"t{t}", FACTOR_FIRST if t == warm else FACTOR_LATER)
+            worst[t] = max(r["worst_over_tol"] for r in rep.values())
+            exempt = max([exempt] + [r["exempt"] for r in rep.values()])
+    print(name, "worst determined entry, in tolerances:", {k: round(v, 2) for k, v in worst.items()},
+          f"largest exempt share of a tensor {exempt:.1e}")
     # the reference's own local exploitability of the final average strategy (:718-764)
     from oracle import best_response as OBR
     if np.isnan(golden[f"{name}/local_exploitability"]).any():
