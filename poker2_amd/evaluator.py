@@ -318,6 +318,26 @@ class HipSparseCFREvaluator:
         if split is None:
             split = N < SPLIT_ROOTS_BELOW
         self._items = self._split_items(tree) if split else None
+        self._root_items = None
+        if self._items is None and T:
+            # Roots of unequal size (mixed streets, stacks, pots): one work item per root, largest tree
+            # first, so that the launch does not end on a long root that started last.
+            size = np.bincount(tree.root_index, minlength=N)
+            if size.min() != size.max():
+                order = np.argsort(-size, kind="stable").astype(np.int64)
+
+                def per_item(mask):
+                    rows = np.nonzero(mask)[0]
+                    slot = np.argsort(order)[tree.root_index[rows]]                 # position of the row's root in the order
+                    by_slot = np.argsort(slot, kind="stable")
+                    counts = np.bincount(slot, minlength=N)
+                    return (self._t(rows[by_slot].astype(np.int64)),
+                            self._t(np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)))
+                parents, parent_offsets = per_item(tree.child_count > 0)
+                showdown, showdown_offsets = per_item(tree.showdown_mask)
+                self._root_items = SimpleNamespace(parents=parents, parent_offsets=parent_offsets, showdown=showdown,
+                                                   showdown_offsets=showdown_offsets, item_root=self._t(order),
+                                                   item_top=self._t(np.ones(N, np.uint8)))
 
     def _split_items(self, tree: SparseTree):
         """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h):
@@ -359,6 +379,18 @@ class HipSparseCFREvaluator:
         deep_sd = np.arange(offs[cut + 1], T)
         deep_sd = deep_sd[tree.showdown_mask[deep_sd]]
         sub_sd, sub_so = grouped(deep_sd, anchor[deep_sd], subs)
+        # Largest subtrees first: a launch lasts until its last work item ends, and items are handed to
+        # the compute units in index order, so the long ones must not be the ones that start last.
+        size = np.bincount(np.searchsorted(subs, anchor[deep][np.isin(anchor[deep], subs)]), minlength=M)
+        order = np.argsort(-size, kind="stable")
+
+        def reordered(rows, offsets):
+            pieces = [rows[offsets[g]:offsets[g + 1]] for g in order]
+            lengths = np.array([len(x) for x in pieces], dtype=np.int64)
+            return (np.concatenate(pieces) if pieces else rows), np.concatenate([[0], np.cumsum(lengths)])
+        sub_parents, sub_po = reordered(sub_parents, sub_po)
+        sub_sd, sub_so = reordered(sub_sd, sub_so)
+        subs = subs[order]
         parents = np.concatenate([top_parents, sub_parents]).astype(np.int64)
         parent_offsets = np.concatenate([top_po, top_po[-1] + sub_po[1:]]).astype(np.int64)
         showdown = np.concatenate([top_sd, sub_sd]).astype(np.int64)
@@ -657,7 +689,7 @@ class HipSparseCFREvaluator:
         a.reach, a.reach_avg = p(self.self_reach), p(self.self_reach_avg)
         a.latest, a.values_avg, a.scratch = p(self.latest_values), p(self.values_avg), p(self._scratch)
         a.fscal, a.iscal = p(self._fscal), p(self._iscal)
-        it = self._items
+        it = self._items if self._items is not None else self._root_items
         if it is not None:
             a.root_parent_offsets, a.root_parents = p(it.parent_offsets), p(it.parents)
             a.root_showdown_offsets, a.root_showdown_nodes = p(it.showdown_offsets), p(it.showdown)
