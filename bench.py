@@ -11,8 +11,10 @@ resident in HBM before the timed region.  Prints ONE JSON line:
                on the launch stream) against the 8 TB/s HBM peak
   cpu_baseline the numpy oracle (a CPU restatement of the reference's torch path) timed on
                this box's host cores on a small sample of the same workload
-  extra        showdown evaluations/s (B=4096 boards), 7-card hands ranked/s (2^20 hands), and the
-               iteration at the reference's own batch of 192 roots
+  extra        showdown evaluations/s (B=4096 boards), 7-card hands ranked/s (2^20 hands), each with
+               its CPU leg; the iteration at the reference's own batch of 192 roots; and the same
+               iteration kernel on the other river workloads (three-raise tree, 1024 roots), so that
+               the headline is not read as the only case
 """
 from __future__ import annotations
 
@@ -33,9 +35,23 @@ BYTES_PER_NODE_ITER = 29 * H * 4          # 17 vectors written + 12 read per nod
 HBM_PEAK_GBS = 8000.0
 TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2), "raise3": (16, 3), "depth5": (5, None)}
 # HBM bytes per launch of the iteration kernel from two rocprofv3 --pmc passes (FETCH_SIZE, then
-# WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy): an offline
-# measurement per workload, quoted in the JSON line; None where no counter run exists.
-MEASURED_TRAFFIC_BYTES = {("depth2", 4096): 6.00e9 + 6.80e9}
+# WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy).  NOT measured by this
+# program: counters need the profiler, so these are constants taken from the summary file named
+# below, one per workload that has a counter run; None elsewhere.  (read bytes, written bytes)
+TRAFFIC_SOURCE = "profiles/cfr_iteration_kernel_river.hbm_counters.txt"
+MEASURED_TRAFFIC_BYTES = {("depth2", 4096): (5.873e9, 6.723e9), ("raise3", 4096): (32.00e9, 35.98e9),
+                          ("depth2", 1024): (1.455e9, 1.681e9)}
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def synth_roots(n: int, seed: int):
@@ -100,7 +116,8 @@ def cpu_baseline(tree: str, seed: int, budget_s: float = 20.0) -> dict:
         cores = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
     except Exception:
         cores = os.cpu_count() or 1
-    return {"value": n / med, "unit": "subgame-iterations/s", "cores": int(cores), "kind": "port",
+    return {"value": n / med, "unit": "subgame-iterations/s", "cores": int(cores), "cpu_model": cpu_model(),
+            "kind": "port",
             "sample": f"{n} river subgames ({t.total // n} nodes each), median of {len(times)} iterations "
                       f"of the numpy oracle, {med * 1e3:.1f} ms per iteration"}
 
@@ -160,6 +177,61 @@ def side_metrics() -> dict:
     out["iteration_ms_B192_three_raise_tree"] = ms
     out["subgame_iterations_per_s_B192"] = 192 / (ms * 1e-3)
     out["algorithmic_GBps_B192"] = BYTES_PER_NODE_ITER * small.total_nodes / (ms * 1e-3) / 1e9
+    del small
+    # the same iteration kernel on the other river workloads (HIP events around 20 launches each)
+    others = []
+    for roots, tree in ((4096, "raise3"), (4096, "raise1"), (1024, "depth2"), (1024, "raise3")):
+        ev, _, _ = make_evaluator(roots, tree, 42, iterations=64)
+        for t in range(5):
+            ev.cfr_iteration(t)
+        torch.cuda.synchronize()
+        ev0.record()
+        for t in range(5, 25):
+            ev.cfr_iteration(t)
+        ev1.record()
+        torch.cuda.synchronize()
+        ms = ev0.elapsed_time(ev1) / 20
+        gbs = BYTES_PER_NODE_ITER * ev.total_nodes / (ms * 1e-3) / 1e9
+        others.append({"roots": roots, "tree": tree, "nodes_per_root": ev.total_nodes // roots, "iteration_ms": ms,
+                       "algorithmic_GBps": gbs, "frac": gbs / HBM_PEAK_GBS})
+        del ev
+        torch.cuda.empty_cache()
+    out["iteration_other_workloads"] = others
+    return out
+
+
+def cpu_side_baselines(budget_s: float = 6.0) -> dict:
+    """CPU legs of the two side metrics on this box's host cores: the C restatement of the reference's
+    rules evaluator on 2^20 hands (one thread), and the numpy restatement of its showdown
+    (cfr_evaluator.py:492-601, the [M,1327,52] prefix-sum formulation) on a sample of the 4096 states."""
+    from oracle import ranker_c
+    from oracle import showdown as osd
+    from oracle import cards as ocards
+    out = {"cpu_model": cpu_model()}
+    rng = np.random.default_rng(7)
+    cards = np.argsort(rng.random((1 << 20, 52)), axis=1)[:, :7].astype(np.int8)
+    ranker_c.rank_cards(cards[:1024])
+    t0 = time.perf_counter()
+    ranker_c.rank_cards(cards)
+    dt = time.perf_counter() - t0
+    out["rank7_hands_per_s"] = (1 << 20) / dt
+    out["rank7_sample"] = f"2^20 hands, oracle/ranker.c, 1 thread, {dt * 1e3:.0f} ms"
+    m = 32
+    boards, beliefs = synth_roots(m, 42)
+    allowed, _ = ocards.allowed_hands_for_boards(boards)
+    hrd = osd.init_hand_rank_data(boards, allowed)
+    pot, scale = np.ones((m, 2), np.float32), np.ones(m, np.float32)
+    osd.showdown_value_both(beliefs, hrd, pot, scale)
+    times = []
+    start = time.perf_counter()
+    while time.perf_counter() - start < budget_s and len(times) < 9:
+        t0 = time.perf_counter()
+        osd.showdown_value_both(beliefs, hrd, pot, scale)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    out["showdown_states_per_s"] = m / med
+    out["showdown_sample"] = f"{m} of the 4096 states (tables prepared beforehand, as on the GPU), numpy oracle, " \
+                             f"median of {len(times)} calls, {med * 1e3:.0f} ms per call"
     return out
 
 
@@ -218,6 +290,11 @@ def main() -> None:
     algo_bytes = BYTES_PER_NODE_ITER * ev.total_nodes
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
     assert torch.isfinite(ev.values_avg).all()
+    rw = MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots))
+    traffic = float(sum(rw)) if rw else None
+    total_nodes = ev.total_nodes
+    del ev
+    torch.cuda.empty_cache()
 
     result = {
         "metric": "river CFR iters/sec x subgames",
@@ -234,11 +311,16 @@ def main() -> None:
         "data": "synthetic",
         "config": {"workload": f"fused DCFR iteration, river subgames, B={args.roots}, tree={args.tree} "
                                f"({nodes_per_root} nodes/root, bins 0.5/1.0, pot 200, stacks 800)",
-                   "roots": args.roots, "nodes_per_root": nodes_per_root, "total_nodes": ev.total_nodes,
+                   "roots": args.roots, "nodes_per_root": nodes_per_root, "total_nodes": total_nodes,
                    "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots)),
+                     "traffic": traffic,
+                     "traffic_note": "offline constant from " + TRAFFIC_SOURCE + " (rocprofv3 --pmc FETCH_SIZE / "
+                                     "WRITE_SIZE runs of this command), not measured by this run" if traffic else
+                                     "no counter run exists for this workload",
+                     "traffic_read_write": list(rw) if rw else None,
+                     "frac_of_peak_on_measured_traffic": (traffic / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if traffic else None,
                      "kernel": "cfr_iteration_kernel", "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes},
     }
@@ -246,6 +328,8 @@ def main() -> None:
         result["cpu_baseline"] = cpu_baseline(args.tree, args.seed)
     if not args.no_extra:
         result["extra"] = side_metrics()
+        if not args.no_cpu_baseline:
+            result["extra"]["cpu"] = cpu_side_baselines()
     print(json.dumps(result))
 
 

@@ -171,6 +171,19 @@ def cases(repeats: int):
     yield (f"encode nodes={ev.total_nodes}", ev.total_nodes * (13 * 8 + 16 + 5 * 8 + 10 * 8),
            lambda: ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask))
 
+    # --- local best response, one tree level of the same search: the 16 384 parents of level 1, four
+    # children each (per parent: the actor's range, per child its policy row and both value rows in,
+    # both value rows of the parent out)
+    from . import _lib
+    base, end = int(ev.depth_offsets[1]), int(ev.depth_offsets[2])
+    n_par, n_ch = end - base, int(ev.child_count[base:end].sum())
+    deviator = torch.zeros(ev.total_nodes, dtype=torch.int64, device=dev)
+    vals = torch.rand(ev.total_nodes, 2, H, device=dev)
+    yield (f"best_response_level parents={n_par}", (3 * n_par + 3 * n_ch) * H * 4,
+           lambda: _lib.call("p2hip_best_response_level", _lib.ptr(vals), _lib.ptr(ev.policy_probs_avg),
+                             _lib.ptr(ev.beliefs), _lib.ptr(ev.env.to_act), _lib.ptr(deviator),
+                             _lib.ptr(ev.child_offsets), _lib.ptr(ev.child_count), base, n_par, _lib.stream_ptr()))
+
 
 def main() -> None:
     ap = argparse.ArgumentParser()
