@@ -154,6 +154,21 @@ int p2hip_encode_context(const int64_t* to_act, const int64_t* button, const int
 int p2hip_bet_amounts(const int64_t* to_act, const int64_t* stacks, const int64_t* committed, const int64_t* pot,
                       int64_t m, const float* host_bins, int n_bins, int64_t* amounts, void* stream);
 
+/* The rows of the node table that go to the leaf network, and its answers coming back: the evaluator's
+ * `beliefs[model_indices]` gather and `latest_values.index_copy_(0, model_indices, values)`
+ * (search/cfr_evaluator.py:1030-1043, search/fused_sparse_cfr_evaluator.py:431-445), with the
+ * conversion to and from the network's dtype folded in (under autocast the reference casts in separate
+ * passes).  src / dst [total_rows, 2, 1326] float32; rows [k] int64 (entries outside [0, total_rows)
+ * are skipped); dtype 0 = float32, 1 = bfloat16 (round to nearest even), 2 = float16.
+ * gather : dst[i, 0:2652] = src[rows[i]] in dst_dtype; dst rows are dst_stride ELEMENTS apart, so the
+ *          target may be the network's input matrix with further feature columns behind the ranges.
+ * scatter: dst[rows[i]] = src[i, 0:2652] as float32; src rows are src_stride elements apart.
+ * Both sides 8-byte aligned; strides even (float32) or a multiple of four (16-bit types). */
+int p2hip_gather_leaf_rows(const float* src, const int64_t* rows, int64_t k, int64_t total_rows, void* dst, int dst_dtype,
+                           int64_t dst_stride, void* stream);
+int p2hip_scatter_leaf_rows(const void* src, int src_dtype, int64_t src_stride, const int64_t* rows, int64_t k, float* dst,
+                            int64_t total_rows, void* stream);
+
 /* Policy targets of CFREvaluator.training_data (search/cfr_evaluator.py:1392-1393; _pull_back,
  * search/sparse_cfr_evaluator.py:465-489): out [n_rows, H, num_actions] with
  * out[k,h,a] = policy_avg[c,h] for the child c of node rows[k] that action a leads to, 0 for

@@ -47,6 +47,8 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_encode_context": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _L, _P, _P, _P],
     "p2hip_bet_amounts": [_P, _P, _P, _P, _L, _P, _I, _P, _P],
     "p2hip_policy_targets": [_P, _P, _L, _P, _P, _P, _I, _P, _P],
+    "p2hip_gather_leaf_rows": [_P, _P, _L, _L, _P, _I, _L, _P],
+    "p2hip_scatter_leaf_rows": [_P, _I, _L, _P, _L, _P, _L, _P],
     "p2hip_unblocked_mass": [_P, _L, _P, _P],
     "p2hip_unblocked_mass_by_player": [_P, _P, _L, _I, _P, _P],
     "p2hip_unblocked_mass_ratio": [_P, _P, _P, _L, _F, _P, _P],

@@ -104,6 +104,82 @@ __global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* _
   }
 }
 
+
+// ---- leaf rows to and from the value network -------------------------------------------------
+// A leaf's two ranges are one 2 x 1326 row of the [total, 2, 1326] float32 node table.  The network
+// wants the rows of ITS leaves as one dense matrix, possibly in bf16 / fp16 and with further feature
+// columns behind the ranges; its answers go back into the node table.  One workgroup per leaf, four
+// floats per lane and step (rows are 8-byte aligned: two 8-byte loads, one 8- or 16-byte store).
+constexpr int LEAF_ROW = 2 * P2_H;            // 2652 floats
+constexpr int LEAF_CHUNKS = LEAF_ROW / 4;     // 663
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {   // round to nearest even, like torch
+  auto one = [](float x) -> uint32_t {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;          // NaN stays NaN
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  };
+  return one(a) | (one(b) << 16);
+}
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+  const _Float16 x = (_Float16)a, y = (_Float16)b;
+  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
+}
+
+// dst[i, 0:2652] = src[rows[i]] converted to DT (0 float32, 1 bfloat16, 2 float16); dst rows are
+// dst_stride elements apart (columns behind 2652 are left alone).
+template <int DT>
+__global__ __launch_bounds__(DG_BLOCK) void gather_leaf_rows_kernel(const float* __restrict__ src,
+                                                                    const int64_t* __restrict__ rows, int64_t total_rows,
+                                                                    void* __restrict__ dst, int64_t dst_stride) {
+  const int64_t i = blockIdx.x;
+  const int64_t r = rows[i];
+  if (r < 0 || r >= total_rows) return;
+  const float2* s = reinterpret_cast<const float2*>(src + r * LEAF_ROW);
+  for (int c = threadIdx.x; c < LEAF_CHUNKS; c += DG_BLOCK) {
+    const float2 a = s[2 * c], b = s[2 * c + 1];
+    if (DT == 0) {
+      float2* d = reinterpret_cast<float2*>(reinterpret_cast<float*>(dst) + i * dst_stride);
+      d[2 * c] = a;
+      d[2 * c + 1] = b;
+    } else {
+      uint2* d = reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(dst) + i * dst_stride);
+      d[c] = DT == 1 ? make_uint2(pack_bf16(a.x, a.y), pack_bf16(b.x, b.y)) : make_uint2(pack_f16(a.x, a.y), pack_f16(b.x, b.y));
+    }
+  }
+}
+
+// dst[rows[i]] = src[i, 0:2652] converted to float32; src rows are src_stride elements apart.
+template <int DT>
+__global__ __launch_bounds__(DG_BLOCK) void scatter_leaf_rows_kernel(const void* __restrict__ src, int64_t src_stride,
+                                                                     const int64_t* __restrict__ rows, int64_t total_rows,
+                                                                     float* __restrict__ dst) {
+  const int64_t i = blockIdx.x;
+  const int64_t r = rows[i];
+  if (r < 0 || r >= total_rows) return;
+  float2* d = reinterpret_cast<float2*>(dst + r * LEAF_ROW);
+  for (int c = threadIdx.x; c < LEAF_CHUNKS; c += DG_BLOCK) {
+    float2 a, b;
+    if (DT == 0) {
+      const float2* s = reinterpret_cast<const float2*>(reinterpret_cast<const float*>(src) + i * src_stride);
+      a = s[2 * c];
+      b = s[2 * c + 1];
+    } else {
+      const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(src) + i * src_stride)[c];
+      if (DT == 1) {
+        a = make_float2(__builtin_bit_cast(float, u.x << 16), __builtin_bit_cast(float, u.x & 0xFFFF0000u));
+        b = make_float2(__builtin_bit_cast(float, u.y << 16), __builtin_bit_cast(float, u.y & 0xFFFF0000u));
+      } else {
+        auto h = [](uint32_t v) -> float { return (float)__builtin_bit_cast(_Float16, (uint16_t)v); };
+        a = make_float2(h(u.x & 0xFFFFu), h(u.x >> 16));
+        b = make_float2(h(u.y & 0xFFFFu), h(u.y >> 16));
+      }
+    }
+    d[2 * c] = a;
+    d[2 * c + 1] = b;
+  }
+}
+
 }  // namespace p2
 
 extern "C" {
@@ -162,6 +238,41 @@ int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n
     default: return P2_EINVAL;
   }
 #undef P2_PT_CASE
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_gather_leaf_rows(const float* src, const int64_t* rows, int64_t k, int64_t total_rows, void* dst, int dst_dtype,
+                           int64_t dst_stride, void* stream) {
+  if (k < 0 || total_rows < 0 || dst_dtype < 0 || dst_dtype > 2 || dst_stride < p2::LEAF_ROW) return P2_EINVAL;
+  if (k == 0) return 0;
+  if (!src || !rows || !dst || k > 0x7FFFFFFF) return P2_EINVAL;
+  // 8-byte accesses on both sides: float32 rows need an even stride, 16-bit rows a multiple of four
+  if (!p2_aligned8(src) || !p2_aligned8(dst) || (dst_stride % (dst_dtype == 0 ? 2 : 4)) != 0) return P2_EINVAL;
+  const dim3 grid((unsigned)k), block(p2::DG_BLOCK);
+  if (dst_dtype == 0)
+    hipLaunchKernelGGL(p2::gather_leaf_rows_kernel<0>, grid, block, 0, (hipStream_t)stream, src, rows, total_rows, dst, dst_stride);
+  else if (dst_dtype == 1)
+    hipLaunchKernelGGL(p2::gather_leaf_rows_kernel<1>, grid, block, 0, (hipStream_t)stream, src, rows, total_rows, dst, dst_stride);
+  else
+    hipLaunchKernelGGL(p2::gather_leaf_rows_kernel<2>, grid, block, 0, (hipStream_t)stream, src, rows, total_rows, dst, dst_stride);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_scatter_leaf_rows(const void* src, int src_dtype, int64_t src_stride, const int64_t* rows, int64_t k, float* dst,
+                            int64_t total_rows, void* stream) {
+  if (k < 0 || total_rows < 0 || src_dtype < 0 || src_dtype > 2 || src_stride < p2::LEAF_ROW) return P2_EINVAL;
+  if (k == 0) return 0;
+  if (!src || !rows || !dst || k > 0x7FFFFFFF) return P2_EINVAL;
+  if (!p2_aligned8(src) || !p2_aligned8(dst) || (src_stride % (src_dtype == 0 ? 2 : 4)) != 0) return P2_EINVAL;
+  const dim3 grid((unsigned)k), block(p2::DG_BLOCK);
+  if (src_dtype == 0)
+    hipLaunchKernelGGL(p2::scatter_leaf_rows_kernel<0>, grid, block, 0, (hipStream_t)stream, src, src_stride, rows, total_rows, dst);
+  else if (src_dtype == 1)
+    hipLaunchKernelGGL(p2::scatter_leaf_rows_kernel<1>, grid, block, 0, (hipStream_t)stream, src, src_stride, rows, total_rows, dst);
+  else
+    hipLaunchKernelGGL(p2::scatter_leaf_rows_kernel<2>, grid, block, 0, (hipStream_t)stream, src, src_stride, rows, total_rows, dst);
   P2_LAUNCH_CHECK();
   return 0;
 }

@@ -633,26 +633,62 @@ class HipSparseCFREvaluator:
                                      enforce_zero_sum=self.enforce_zero_sum, ignore_mask=self.env.done)
 
     # ------------------------------------------------------------------ leaf values
+    _LEAF_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+    def gather_leaf_rows(self, table: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """``out[i, :2652] = table[rows[i]]`` in ``out``'s dtype (float32 / bfloat16 / float16), one
+        launch: the gather of the leaves' ranges with the cast to the network's dtype folded in.
+        ``out`` may be wider than 2652 columns (the network's input matrix); the rest is left alone."""
+        _req(table.dtype == torch.float32 and table.is_contiguous() and table.dim() == 3 and
+             tuple(table.shape[1:]) == (2, NUM_HANDS), "table: contiguous float32 [rows, 2, 1326]")
+        _req(out.dtype in self._LEAF_DTYPES and out.dim() == 2 and out.stride(1) == 1 and
+             out.shape == (rows.numel(), out.shape[1]) and out.shape[1] >= 2 * NUM_HANDS, "out: [len(rows), >= 2652]")
+        _req(rows.dtype == torch.int64 and rows.is_contiguous(), "rows: contiguous int64")
+        _lib.require_gpu(table, "gather_leaf_rows")
+        _lib.call("p2hip_gather_leaf_rows", _lib.ptr(table), _lib.ptr(rows), rows.numel(), table.shape[0], _lib.ptr(out),
+                  self._LEAF_DTYPES[out.dtype], out.stride(0), _lib.stream_ptr())
+        return out
+
+    def _scatter_leaf_values(self, values: torch.Tensor) -> None:
+        """``latest_values[model_indices] = values`` with the conversion to float32 folded in."""
+        k = self.model_indices.numel()
+        values = values.reshape(k, 2 * NUM_HANDS)
+        if values.dtype not in self._LEAF_DTYPES or values.stride(1) != 1 or values.stride(0) % 4:
+            values = values.to(self.float_dtype).contiguous()
+        _lib.call("p2hip_scatter_leaf_rows", _lib.ptr(values), self._LEAF_DTYPES[values.dtype], values.stride(0),
+                  _lib.ptr(self.model_indices), k, _lib.ptr(self.latest_values), self.total_nodes, _lib.stream_ptr())
+
     def _model_leaf_values(self, beliefs: torch.Tensor) -> torch.Tensor | None:
+        """The network's answer for the model leaves, [K, 2, 1326], in whatever dtype it answers in.
+        A model with ``leaf_values_from_nodes`` is handed the whole node table and gathers its rows
+        itself (``gather_leaf_rows``: straight into its input matrix, in its dtype)."""
         if self.model_indices.numel() == 0:
             return None
         if self.model is None:
             return torch.zeros(self.model_indices.numel(), 2, NUM_HANDS, dtype=self.float_dtype, device=self.device)
-        return self.model.leaf_values(beliefs[self.model_indices], self.model_indices, self).to(self.float_dtype)
+        if hasattr(self.model, "leaf_values_from_nodes") and beliefs.is_contiguous() and beliefs.dtype == torch.float32:
+            return self.model.leaf_values_from_nodes(beliefs, self.model_indices, self)
+        return self.model.leaf_values(beliefs[self.model_indices], self.model_indices, self)
 
     def _set_model_values_impl(self, t: int, beliefs: torch.Tensor) -> None:
         """fused_sparse_cfr_evaluator.py:420-445 (CFR-AVG de-averaging included)."""
         hv = self._model_leaf_values(beliefs)
         if hv is None:
             return
-        if (not self.cfr_avg) or t <= 1 or self.last_model_values is None:
-            self.latest_values.index_copy_(0, self.model_indices, hv)
+        if not self.cfr_avg:
+            # nothing reads the previous answer without CFR-AVG: no copy of it is kept
+            self._scatter_leaf_values(hv)
+            self.last_model_values = hv
+            return
+        hv = hv.to(self.float_dtype)
+        if t <= 1 or self.last_model_values is None:
+            self._scatter_leaf_values(hv)
         else:
             unmixed = torch.empty_like(hv)
             F.fused_model_values_mix_zero_sum(hv.contiguous(), self.last_model_values.contiguous(),
                                               beliefs[self.model_indices].contiguous(), self._t_scalars.mix_onon,
                                               self._t_scalars.mix_oon, unmixed, self.enforce_zero_sum)
-            self.latest_values.index_copy_(0, self.model_indices, unmixed)
+            self._scatter_leaf_values(unmixed)
         # The previous network output lives in a buffer of its own (the reference pins it the same
         # way, fused_sparse_cfr_evaluator.py:464-469): a captured graph keeps reading this address on
         # every replay, and a network that reuses its output tensor cannot alias "last" and "current".

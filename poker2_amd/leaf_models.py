@@ -39,6 +39,24 @@ class RangeBoardMLP(torch.nn.Module):
         onehot = torch.zeros(board.shape[0], 53, dtype=features.beliefs.dtype, device=board.device)
         onehot.scatter_(1, torch.where(board >= 0, board, torch.full_like(board, 52)), 1.0)
         x = torch.cat([features.beliefs, onehot[:, :52]], dim=1)
+        return self.forward_input(x)
+
+    # The input matrix is [ranges (2 x 1326) | board one-hot (52)].  Only the ranges change between the
+    # iterations of a search, so a caller may keep the matrix, have the ranges written into its first
+    # 2652 columns (HipSparseCFREvaluator.gather_leaf_rows does that in the matrix's dtype) and call
+    # forward_input: no concatenation and no separate cast per call.
+    input_width = 2 * NUM_HANDS + 52
+
+    def static_input_columns(self, features: MLPFeatures, dtype: torch.dtype) -> torch.Tensor:
+        """[N, input_width] with the columns that do not depend on the ranges filled in."""
+        board = features.board
+        onehot = torch.zeros(board.shape[0], 53, dtype=dtype, device=board.device)
+        onehot.scatter_(1, torch.where(board >= 0, board, torch.full_like(board, 52)), 1.0)
+        x = torch.zeros(board.shape[0], self.input_width, dtype=dtype, device=board.device)
+        x[:, 2 * NUM_HANDS:] = onehot[:, :52]
+        return x
+
+    def forward_input(self, x: torch.Tensor) -> SimpleNamespace:
         for lin in self.linears[:-1]:
             x = torch.relu(lin(x))
         x = self.linears[-1](x)
@@ -79,7 +97,33 @@ class NetworkLeafModel:
                 hv = self.net(feats).hand_values
         else:
             hv = self.net(feats).hand_values
-        return hv.to(beliefs.dtype)
+        return hv
+
+
+    @torch.no_grad()
+    def leaf_values_from_nodes(self, table: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
+        """The same answer from the whole node table ``table`` [total, 2, 1326]: for a network that
+        offers ``forward_input`` / ``static_input_columns`` the input matrix is kept for the subgame,
+        the leaves' ranges are written into it by one kernel in the network's dtype, and the answer is
+        returned in that dtype (the evaluator converts while it stores).  Other networks get the
+        gathered ranges through ``leaf_values``."""
+        net = self.net
+        if not (hasattr(net, "forward_input") and hasattr(net, "static_input_columns")):
+            return self.leaf_values(table[rows], rows, ev)
+        key = (id(ev), ev.subgame_serial, rows.data_ptr(), rows.numel(), "input")
+        if self._cached_for != key:
+            c = ev.feature_encoder.encode_rows(table[rows], rows, ev.new_street_mask[rows])
+            feats = MLPFeatures(context=c.context, street=c.street, to_act=c.to_act, board=c.board,
+                                beliefs=c.beliefs.reshape(rows.numel(), -1))
+            self._cached = net.static_input_columns(feats, self.autocast_dtype or torch.float32)
+            self._cached_for = key
+        x = ev.gather_leaf_rows(table, rows, self._cached)
+        if hasattr(net, "eval"):
+            net.eval()
+        if self.autocast_dtype is not None:
+            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                return net.forward_input(x).hand_values
+        return net.forward_input(x).hand_values
 
 
 class ChanceLeafModel:

@@ -633,3 +633,90 @@ def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
     assert ratio.max() <= LOOP_FACTOR, f"beliefs left behind: worst entry {ratio.max():.1f} tolerances"
     print(fixture, "loop: worst entry, in tolerances:", {k: round(v, 1) for k, v in WORST.items()},
           "beliefs left behind", round(float(ratio.max()), 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_leaf_rows_to_the_network_and_back(dtype):
+    """``gather_leaf_rows`` / the scatter behind ``set_leaf_values`` against the torch operations they
+    replace (``table[rows]`` + ``.to(dtype)`` + ``cat``; ``.to(float32)`` + ``index_copy_``):
+    bit-exact, conversions included (bfloat16 rounds to nearest even, NaN stays NaN), columns behind
+    the ranges untouched, rows outside the table skipped."""
+    from poker2_amd import _lib
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    from tests.helpers import random_boards
+    rng = np.random.default_rng(3)
+    n = 6
+    roots = RootStates.at_round_start(3, np.full(n, 200), np.tile([[800, 800]], (n, 1)), random_boards(rng, n, 5))
+    ev = HipSparseCFREvaluator(None, torch.device(DEV), river_dcfr_config(n, iterations=2, depth=2))
+    ev.initialize_subgame(roots, np.arange(n))
+    total = ev.total_nodes
+    table = torch.from_numpy(rng.standard_normal((total, 2, H)).astype(np.float32) * 3.0).to(DEV)
+    table[1, 0, 5] = float("nan")
+    table[2, 1, 7] = float("inf")
+    table[3, 0, 9] = 1e-41                                   # denormal
+    others = rng.permutation(np.arange(4, total))[:34]
+    rows = torch.from_numpy(np.concatenate([[1, 2, 3], others]).astype(np.int64)).to(DEV)      # distinct rows
+    width = 2 * H + 52
+    out = torch.full((37, width), 7.0, dtype=dtype, device=DEV)
+    ev.gather_leaf_rows(table, rows, out)
+    want = table[rows].reshape(37, -1).to(dtype)
+    assert torch.equal(out[:, :2 * H].view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       want.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    assert (out[:, 2 * H:] == 7.0).all()
+    # and back
+    answers = torch.from_numpy(rng.standard_normal((37, 2, H)).astype(np.float32)).to(DEV).to(dtype)
+    dst = torch.full((total, 2, H), -5.0, device=DEV)
+    bad = rows.clone()
+    bad[4], bad[5] = -1, total                               # outside the table: skipped
+    _lib.call("p2hip_scatter_leaf_rows", _lib.ptr(answers), {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}[dtype],
+              2 * H, _lib.ptr(bad), 37, _lib.ptr(dst), total, _lib.stream_ptr())
+    want = torch.full((total, 2, H), -5.0, device=DEV)
+    keep = torch.ones(37, dtype=torch.bool, device=DEV)
+    keep[4] = keep[5] = False
+    want.index_copy_(0, rows[keep], answers[keep].float())
+    assert torch.equal(dst, want)
+
+
+def test_network_answers_do_not_depend_on_how_the_ranges_reach_it():
+    """NetworkLeafModel over RangeBoardMLP: ranges written straight into the kept input matrix
+    (``leaf_values_from_nodes``) against gather + concatenate + cast (``leaf_values``), float32 and
+    bf16 autocast: identical answers, and identical searches."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel, RangeBoardMLP
+    from poker2_amd.tree import RootStates
+    from tests.helpers import random_boards, random_ranges
+    rng = np.random.default_rng(8)
+    n = 5
+    boards = random_boards(rng, n, 5)
+    boards[:3, 4] = -1                                        # three turn roots: street-end leaves go to the network
+    beliefs = torch.from_numpy(random_ranges(rng, boards))
+    roots = RootStates.at_round_start(np.where(boards[:, 4] < 0, 2, 3), np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards)
+    net = RangeBoardMLP(hidden=64, layers=2, seed=2).to(DEV)
+    for autocast in (None, torch.bfloat16):
+        states = []
+        for direct in (True, False):
+            model = NetworkLeafModel(net, DEV, autocast_dtype=autocast)
+            ev = HipSparseCFREvaluator(model if direct else _WithoutNodes(model), torch.device(DEV),
+                                       river_dcfr_config(n, iterations=4, depth=16), max_raises=1)
+            ev.initialize_subgame(roots, np.arange(n), beliefs)
+            ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+            assert ev.model_indices.numel() > 0
+            for t in range(3):
+                ev.cfr_iteration(t)
+            states.append({k: getattr(ev, k).clone() for k in OCFR.OracleCFR.STATE_NAMES})
+        for k in OCFR.OracleCFR.STATE_NAMES:
+            assert torch.equal(states[0][k], states[1][k]), (autocast, k)
+
+
+class _WithoutNodes:
+    """A leaf model that only offers ``leaf_values`` (the evaluator then gathers the ranges itself)."""
+
+    def __init__(self, inner):
+        self.inner = inner
+        self.enforce_zero_sum = inner.enforce_zero_sum
+
+    def leaf_values(self, beliefs, rows, ev):
+        return self.inner.leaf_values(beliefs, rows, ev)
