@@ -68,6 +68,7 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
 # — a quotient of differences of nearly equal values — amplifies them; that the iteration ITSELF
 # is right to well within the tolerance is what the one-step comparison shows.
 FREE_FACTOR_FIRST, FREE_FACTOR_LATER = 3.0, 5.0
+P999_FACTOR = 15.0        # largest seen: 9.9 (depth-3 tree, sixth iteration)
 
 
 class Lockstep:
@@ -450,7 +451,7 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
     orc.prepare()
     pack = PAR.OracleWithTwins(orc, seed=6)
     names = [s for s in OCFR.OracleCFR.STATE_NAMES if s not in left_out]
-    worst = {}
+    worst, p999 = {}, {}
 
     def check(tag, factor):
         got = {s: getattr(ev, s).cpu().numpy()[..., cols] for s in names}
@@ -462,6 +463,11 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
                                (lambda s: blocked if got[s].ndim == 2 else blocked[:, None, :]),
                                max_exempt=1.0 if blocked is not None else 0.25, what=f"{name} {tag}: ")
         worst[tag] = max(r["worst_over_tol"] for r in rep.values())
+        # and over EVERY compared entry, exempt or not: all but one in a thousand within P999_FACTOR tolerances
+        p999[tag] = max(r["p999_over_tol"] for r in rep.values())
+        # (against the fused-class fixture; the base class differs from it on board-blocked hands by design)
+        assert fixture != "fused" or p999[tag] <= P999_FACTOR, \
+            f"{name} {tag}: 99.9th percentile of all entries at {p999[tag]:.2f} tolerances"
     check("prep", FREE_FACTOR_FIRST)
     stored = set(g[f"{name}/stored"].tolist())
     for t in range(int(warm), int(iters)):
@@ -470,7 +476,8 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
         if t in stored:
             check(f"t{t}", FREE_FACTOR_FIRST if t == int(warm) else FREE_FACTOR_LATER)
     print(name, fixture, "fused" if fused else "per-op", "worst determined entry, in tolerances:",
-          {k: round(v, 2) for k, v in worst.items()})
+          {k: round(v, 2) for k, v in worst.items()}, "99.9th percentile of all entries:",
+          {k: round(v, 2) for k, v in p999.items()})
     if left_out:
         return
     stats = ev._compute_exploitability()
