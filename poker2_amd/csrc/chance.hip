@@ -13,6 +13,12 @@
 // The per-sample sum of a player's masked range is T - cs[c] (T = total of the board-masked
 // range, cs[c] = its mass on hands holding c), so one card-sum pass per state serves all of
 // its 46-49 samples.  The expansion is a pure write stream (about 48 x 10.6 KB per state).
+//
+// A state's samples are one contiguous run of 2652-float blocks.  The main kernel treats the run a
+// workgroup writes as a flat sequence of float4 and places its lanes on absolute 128-byte lines, so every
+// wave-wide store covers whole lines (rows of 5304 bytes never start on one); the state's masked ranges
+// and the hands' cards are staged in LDS and each float4 looks up its sample and hands there.  Buffers
+// that are only 8-byte aligned take the row-wise float2 kernel.
 #pragma once
 #include <mutex>
 #include "common.h"
@@ -41,6 +47,32 @@ __device__ __forceinline__ int chance_board(const int64_t* __restrict__ board5, 
   return n;
 }
 
+// Workgroup -> (state, run of candidate cards).  States are taken in groups of `group`; inside a
+// group the order is run-major.  The row-wise kernel takes groups of 2048: workgroups in flight at one
+// time then write chunks a megabyte apart (measured faster for it than neighbouring chunks), while a
+// group's ranges (22 MB) stay in the last-level cache for the 13 visits they get (16384 states as one
+// group: 2.61 ms; in groups of 2048: 1.85 ms).  The line kernel takes groups of 8 = the number of XCDs:
+// workgroup b runs on XCD b mod 8, so the four workgroups of a state follow each other on one XCD and
+// read its ranges from that XCD's L2 (3584 states: groups of 2048 392 us, of 8 375 us; 16384 states:
+// 1.81 ms and 1.68 ms).
+constexpr int CH_GROUP_ROWS = 2048;
+constexpr int CH_GROUP_LINES = 8;
+
+__device__ __forceinline__ bool chance_work(int64_t n, int parts, int group_size, int64_t& state, int& part) {
+  const int64_t per_group = (int64_t)group_size * parts;
+  const int64_t group = blockIdx.x / per_group, r = blockIdx.x - group * per_group;
+  const int64_t first = group * group_size;
+  const int64_t count = n - first < group_size ? n - first : group_size;   // the last group may be short
+  if (r >= count * parts) return false;   // the grid is sized for full groups
+  part = (int)(r / count);
+  state = first + (r - part * count);
+  return true;
+}
+
+static inline unsigned chance_grid(int64_t n, int parts, int group_size) {
+  return (unsigned)(((n + group_size - 1) / group_size) * group_size * parts);
+}
+
 __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __restrict__ pre_beliefs,
                                                                   const int64_t* __restrict__ root_indices,
                                                                   const int64_t* __restrict__ board,
@@ -48,10 +80,12 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
                                                                   int64_t source_rows, int64_t total_samples,
                                                                   float* __restrict__ post_beliefs,
                                                                   int64_t* __restrict__ board_samples,
-                                                                  int64_t* __restrict__ root_lookup) {
+                                                                  int64_t* __restrict__ root_lookup, int64_t n) {
   __shared__ __align__(8) float t[2][P2_H + 2];
   __shared__ double cs[2 * P2_CARDS];
-  const int64_t i = blockIdx.x;
+  int64_t i;
+  int part;
+  if (!chance_work(n, CH_SPLIT, CH_GROUP_ROWS, i, part)) return;
   const int64_t root = root_indices ? root_indices[i] : i;
   if (root < 0 || root >= source_rows) return;   // uniform per workgroup: nothing to read, nothing written
   int bcards[5];
@@ -95,13 +129,13 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
       const bool on_board = ((bits >> (ab[k][q] & 0xFFu)) | (bits >> (ab[k][q] >> 8))) & 1ull;
       uni[k][q] = on_board ? 0.f : uniform;
     }
-  // blockIdx.y splits the 52 candidate cards into CH_SPLIT runs: short-lived workgroups with few
+  // the 52 candidate cards are split into CH_SPLIT runs: short-lived workgroups with few
   // stores per lane keep the chip's write window dense (runs of 13 cards measured 514 us on
   // 3584 turn states, runs of 4 cards 435 us, single cards 782 us - the card-sum preamble is paid
   // per workgroup; re-reading the ranges from L2 per sample instead of keeping them in registers
   // measured slower than either); a sample's position counts the cards below it that are not on
   // the board
-  const int c_begin = blockIdx.y * (P2_CARDS / CH_SPLIT), c_end = c_begin + P2_CARDS / CH_SPLIT;
+  const int c_begin = part * (P2_CARDS / CH_SPLIT), c_end = c_begin + P2_CARDS / CH_SPLIT;
   int64_t s = sample_offsets[i] + c_begin - __popcll(bits & ((1ull << c_begin) - 1ull));
   for (int c = c_begin; c < c_end; ++c) {
     if ((bits >> c) & 1ull) continue;
@@ -136,6 +170,135 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
     }
     if (threadIdx.x == 0) root_lookup[s] = i;
     ++s;
+  }
+}
+
+// ---- the expansion on whole 128-byte lines ------------------------------------------------------
+constexpr int CH_QUADS = 2 * P2_H / 4;   // 663 float4 per state and per sample
+constexpr int CH_QPT = 3;                // float4 per lane when a state is staged: 3 x 256 >= 663
+constexpr int CH_MAX_RUN = 13;           // candidate cards per workgroup: 52 / parts with parts = 4 or 13
+static_assert((2 * P2_H) % 4 == 0 && CH_QPT * CH_BLOCK >= CH_QUADS, "a state is a whole number of float4");
+
+struct ChanceSample {   // what a float4 needs to know about its sample
+  float inv0, inv1;     // 1 / the surviving mass of player 0 / 1, or 0 where the uniform fallback applies
+  int card;
+  int pad;
+};
+
+__global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const float* __restrict__ pre_beliefs,
+                                                                        const int64_t* __restrict__ root_indices,
+                                                                        const int64_t* __restrict__ board,
+                                                                        const int64_t* __restrict__ sample_offsets,
+                                                                        int64_t source_rows, int64_t total_samples,
+                                                                        float* __restrict__ post_beliefs,
+                                                                        int64_t* __restrict__ board_samples,
+                                                                        int64_t* __restrict__ root_lookup, int64_t n,
+                                                                        int parts) {
+  __shared__ __align__(16) float t[2 * P2_H];            // the state's ranges without the board's hands
+  __shared__ __align__(16) uint16_t cards_of[2 * P2_H];  // a | b << 8 of the hand behind every float of t
+  __shared__ double cs[2 * P2_CARDS];
+  __shared__ __align__(16) ChanceSample sample[CH_MAX_RUN];
+  int64_t i;
+  int part;
+  if (!chance_work(n, parts, CH_GROUP_LINES, i, part)) return;
+  const int64_t root = root_indices ? root_indices[i] : i;
+  if (root < 0 || root >= source_rows) return;   // uniform per workgroup
+  int bcards[5];
+  uint64_t bits;
+  const int ncards = chance_board(board + root * 5, bcards, bits);
+  if (ncards >= 5) return;                       // no empty slot: nothing to expand
+
+  const float4* src = reinterpret_cast<const float4*>(pre_beliefs + root * (2 * P2_H));
+#pragma unroll
+  for (int k = 0; k < CH_QPT; ++k) {
+    const int j = threadIdx.x + k * CH_BLOCK;
+    if (j >= CH_QUADS) continue;
+    const float4 x = src[j];
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+    float y[4];
+    uint16_t packed[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int f = 4 * j + q;
+      const int h = f >= P2_H ? f - P2_H : f;
+      const uint32_t a = p2_combo.a[h], b = p2_combo.b[h];
+      packed[q] = (uint16_t)(a | (b << 8));
+      y[q] = (((bits >> a) | (bits >> b)) & 1ull) ? 0.f : xs[q];
+    }
+    reinterpret_cast<float4*>(t)[j] = make_float4(y[0], y[1], y[2], y[3]);
+    reinterpret_cast<uint2*>(cards_of)[j] = make_uint2((uint32_t)packed[0] | ((uint32_t)packed[1] << 16),
+                                                       (uint32_t)packed[2] | ((uint32_t)packed[3] << 16));
+  }
+  p2_sync_lds();
+  card_sums_multi(t, P2_H, 2, cs);
+  const double total0 = card_total(cs), total1 = card_total(cs + P2_CARDS);
+
+  // this workgroup's samples: the cards of its run that are not on the board, in ascending order
+  const int run = P2_CARDS / parts;
+  const int c_begin = part * run;
+  const uint64_t run_bits = ((1ull << run) - 1ull) << c_begin;
+  const uint64_t free_bits = ~bits & run_bits;
+  const int64_t s_first = sample_offsets[i] + c_begin - __popcll(bits & ((1ull << c_begin) - 1ull));
+  int count = __popcll(free_bits);
+  // outputs are sized for total_samples: samples beyond them are not written
+  if (s_first < 0) count = 0;
+  else if (s_first + count > total_samples) count = (int)(total_samples > s_first ? total_samples - s_first : 0);
+  if ((int)threadIdx.x < run) {
+    const int c = c_begin + threadIdx.x;
+    const int m = __popcll(free_bits & ((1ull << c) - 1ull));   // position among the run's samples
+    if (((free_bits >> c) & 1ull) && m < count) {
+      const float sum0 = (float)(total0 - cs[c]);
+      const float sum1 = (float)(total1 - cs[P2_CARDS + c]);
+      ChanceSample sm;
+      sm.inv0 = sum0 > 1e-12f ? 1.0f / fmaxf(sum0, 1e-12f) : 0.f;
+      sm.inv1 = sum1 > 1e-12f ? 1.0f / fmaxf(sum1, 1e-12f) : 0.f;
+      sm.card = c;
+      sm.pad = 0;
+      sample[m] = sm;
+    }
+  }
+  p2_sync_lds();
+  if (count <= 0) return;
+
+  // board_samples [S,5] and root_lookup [S]: lane 8 m + slot
+  {
+    const int m = threadIdx.x >> 3, slot = threadIdx.x & 7;
+    if (m < count) {
+      if (slot < 5) {
+        int64_t card = bcards[0];
+#pragma unroll
+        for (int q = 1; q < 5; ++q) card = slot == q ? (int64_t)bcards[q] : card;
+        if (slot == ncards) card = sample[m].card;
+        board_samples[(s_first + m) * 5 + slot] = card;
+      } else if (slot == 5) {
+        root_lookup[s_first + m] = i;
+      }
+    }
+  }
+
+  const int remaining = P2_CARDS - ncards - 1;          // cards left for the hands of a sample
+  const float uniform = 1.0f / fmaxf((float)(remaining * (remaining - 1) / 2), 1.0f);
+  float4* out = reinterpret_cast<float4*>(post_beliefs);
+  const int64_t g0 = s_first * CH_QUADS, g1 = g0 + (int64_t)count * CH_QUADS;   // float4 range of the workgroup
+  for (int64_t g = (g0 & ~7ll) + threadIdx.x; g < g1; g += CH_BLOCK) {
+    if (g < g0) continue;
+    const uint32_t local = (uint32_t)(g - g0);
+    const uint32_t m = local / CH_QUADS, j = local - m * CH_QUADS;
+    const ChanceSample sm = sample[m];
+    const float4 x = reinterpret_cast<const float4*>(t)[j];
+    const uint2 pk = reinterpret_cast<const uint2*>(cards_of)[j];
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+    const uint32_t cd[4] = {pk.x & 0xFFFFu, pk.x >> 16, pk.y & 0xFFFFu, pk.y >> 16};
+    float r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float inv = (4 * j + q >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
+      const uint32_t a = cd[q] & 0xFFu, b = cd[q] >> 8;
+      float val = xs[q] * inv;
+      if (inv == 0.f) val = (((bits >> a) | (bits >> b)) & 1ull) ? 0.f : uniform;   // no mass left: uniform
+      r[q] = (a == (uint32_t)sm.card || b == (uint32_t)sm.card) ? 0.f : val;
+    }
+    out[g] = make_float4(r[0], r[1], r[2], r[3]);
   }
 }
 
@@ -249,6 +412,112 @@ __global__ __launch_bounds__(CH_BLOCK) void flop_expand_kernel(const float* __re
       o0[idx] = make_float2(r0[0], r0[1]);
       o1[idx] = make_float2(r1[0], r1[1]);
     }
+  }
+}
+
+// The flop expansion on whole 128-byte lines: same scheme as chance_expand_lines_kernel.  out is one
+// run of 2652-float blocks in (state, flop) order; a workgroup writes `run` consecutive flops of a state.
+constexpr int FL_MAX_RUN = 16;
+
+struct FlopSample {
+  float inv0, inv1;    // 1 / surviving mass, or 0 where the uniform fallback applies
+  uint32_t cards;      // c0 | c1 << 8 | c2 << 16, or 0xFFFFFFFF for a flop that is not three distinct cards
+  uint32_t pad;
+};
+
+__global__ __launch_bounds__(CH_BLOCK) void flop_expand_lines_kernel(const float* __restrict__ pre_beliefs,
+                                                                      const int64_t* __restrict__ root_indices,
+                                                                      const int64_t* __restrict__ flops,
+                                                                      int64_t n_flops, float* __restrict__ out,
+                                                                      int64_t n, int run, int parts) {
+  __shared__ __align__(16) float t[2 * P2_H];
+  __shared__ __align__(16) uint16_t cards_of[2 * P2_H];
+  __shared__ double cs[2 * P2_CARDS];
+  __shared__ __align__(16) FlopSample sample[FL_MAX_RUN];
+  int64_t i;
+  int part;
+  if (!chance_work(n, parts, CH_GROUP_LINES, i, part)) return;
+  const int64_t root = root_indices ? root_indices[i] : i;
+  const float4* src = reinterpret_cast<const float4*>(pre_beliefs + root * (2 * P2_H));
+#pragma unroll
+  for (int k = 0; k < CH_QPT; ++k) {
+    const int j = threadIdx.x + k * CH_BLOCK;
+    if (j >= CH_QUADS) continue;
+    reinterpret_cast<float4*>(t)[j] = src[j];
+    uint32_t packed[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int f = 4 * j + q;
+      const int h = f >= P2_H ? f - P2_H : f;
+      packed[q] = (uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8);
+    }
+    reinterpret_cast<uint2*>(cards_of)[j] = make_uint2(packed[0] | (packed[1] << 16), packed[2] | (packed[3] << 16));
+  }
+  p2_sync_lds();
+  card_sums_multi(t, P2_H, 2, cs);
+  const double total[2] = {card_total(cs), card_total(cs + P2_CARDS)};
+
+  const int64_t f_begin = (int64_t)part * run;
+  const int count = (int)(n_flops - f_begin < run ? n_flops - f_begin : run);
+  if ((int)threadIdx.x < count) {
+    const int64_t f = f_begin + threadIdx.x;
+    int c[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) c[j] = (int)flops[f * 3 + j];
+    bool valid = true;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) valid = valid && c[j] >= 0 && c[j] < P2_CARDS;
+    valid = valid && c[0] != c[1] && c[0] != c[2] && c[1] != c[2];
+    FlopSample sm;
+    sm.cards = valid ? ((uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16)) : 0xFFFFFFFFu;
+    sm.pad = 0;
+    float inv[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      double sum = 0.0;
+      if (valid) {
+        sum = total[p];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) sum -= cs[p * P2_CARDS + c[j]];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          const int x = c[j], y = c[(j + 1) % 3];
+          sum += (double)t[p * P2_H + p2_combo_index(x < y ? x : y, x < y ? y : x)];
+        }
+      }
+      const float sf = (float)sum;
+      inv[p] = sf > 1e-12f ? 1.0f / fmaxf(sf, 1e-12f) : 0.f;
+    }
+    sm.inv0 = inv[0];
+    sm.inv1 = inv[1];
+    sample[threadIdx.x] = sm;
+  }
+  p2_sync_lds();
+  if (count <= 0) return;
+
+  const float uniform = 1.0f / (float)(49 * 48 / 2);   // hands left once three cards are out
+  float4* o = reinterpret_cast<float4*>(out);
+  const int64_t g0 = (i * n_flops + f_begin) * CH_QUADS, g1 = g0 + (int64_t)count * CH_QUADS;
+  for (int64_t g = (g0 & ~7ll) + threadIdx.x; g < g1; g += CH_BLOCK) {
+    if (g < g0) continue;
+    const uint32_t local = (uint32_t)(g - g0);
+    const uint32_t m = local / CH_QUADS, j = local - m * CH_QUADS;
+    const FlopSample sm = sample[m];
+    const float4 x = reinterpret_cast<const float4*>(t)[j];
+    const uint2 pk = reinterpret_cast<const uint2*>(cards_of)[j];
+    const float xs[4] = {x.x, x.y, x.z, x.w};
+    const uint32_t cd[4] = {pk.x & 0xFFFFu, pk.x >> 16, pk.y & 0xFFFFu, pk.y >> 16};
+    const uint32_t c0 = sm.cards & 0xFFu, c1 = (sm.cards >> 8) & 0xFFu, c2 = (sm.cards >> 16) & 0xFFu;
+    const bool valid = sm.cards != 0xFFFFFFFFu;
+    float r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float inv = (4 * j + q >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
+      const uint32_t a = cd[q] & 0xFFu, b = cd[q] >> 8;
+      const bool off = !valid || a == c0 || a == c1 || a == c2 || b == c0 || b == c1 || b == c2;
+      r[q] = off ? 0.f : (inv == 0.f ? uniform : xs[q] * inv);
+    }
+    o[g] = make_float4(r[0], r[1], r[2], r[3]);
   }
 }
 
@@ -461,10 +730,21 @@ int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, c
   if (n == 0) return 0;
   if (!pre_beliefs || !board || !sample_offsets || !post_beliefs || !board_samples || !root_lookup) return P2_EINVAL;
   if (!p2_aligned8(pre_beliefs) || !p2_aligned8(post_beliefs)) return P2_EINVAL;
-  if (n > 0x7FFFFFFF) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::chance_expand_kernel, dim3((unsigned)n, p2::CH_SPLIT), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
-                     pre_beliefs, root_indices, board, sample_offsets, source_rows, total_samples, post_beliefs,
-                     board_samples, root_lookup);
+  if (n > 0x7FFFFFFF / p2::CH_SPLIT - p2::CH_GROUP_ROWS) return P2_EINVAL;
+  const bool wide = ((reinterpret_cast<uintptr_t>(pre_beliefs) | reinterpret_cast<uintptr_t>(post_beliefs)) & 15u) == 0;
+  if (wide) {
+    // runs of 13 cards = 4 workgroups per state (3584 states: 375 us, in runs of 4 cards 465 us; 333 states:
+    // 37 and 42 us); runs of 4 cards only where there would be fewer workgroups than the chip takes at once
+    const int parts = n >= 256 ? 4 : p2::CH_SPLIT;
+    hipLaunchKernelGGL(p2::chance_expand_lines_kernel, dim3(p2::chance_grid(n, parts, p2::CH_GROUP_LINES)), dim3(p2::CH_BLOCK), 0,
+                       (hipStream_t)stream, pre_beliefs, root_indices, board, sample_offsets, source_rows,
+                       total_samples, post_beliefs, board_samples, root_lookup, n, parts);
+    P2_LAUNCH_CHECK();
+    return 0;
+  }
+  hipLaunchKernelGGL(p2::chance_expand_kernel, dim3(p2::chance_grid(n, p2::CH_SPLIT, p2::CH_GROUP_ROWS)), dim3(p2::CH_BLOCK), 0,
+                     (hipStream_t)stream, pre_beliefs, root_indices, board, sample_offsets, source_rows,
+                     total_samples, post_beliefs, board_samples, root_lookup, n);
   P2_LAUNCH_CHECK();
   return 0;
 }
@@ -487,8 +767,23 @@ int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int
   if (n == 0 || n_flops == 0) return 0;
   if (!pre_beliefs || !flops || !out || !p2_aligned8(pre_beliefs) || !p2_aligned8(out)) return P2_EINVAL;
   if (n > 0x7FFFFFFF) return P2_EINVAL;
-  // about four flops per workgroup: short workgroups keep the write window dense, fewer make the
-  // per-workgroup card-sum preamble dominate (1024 states x 256 flops: 16 per workgroup 874 us, 4: 658 us, 1: 1096 us)
+  const bool wide = ((reinterpret_cast<uintptr_t>(pre_beliefs) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  if (wide) {
+    // eight flops per workgroup (1024 states x 256 flops: 4 per workgroup 645 us, 8: 525 us, 16: 530 us; the
+    // row-wise kernel 585-625 us), four where eight would leave fewer than a thousand workgroups
+    const int run = n * ((n_flops + 7) / 8) >= 1024 ? 8 : 4;
+    static_assert(8 <= p2::FL_MAX_RUN, "run length");
+    const int64_t parts = (n_flops + run - 1) / run;
+    const int64_t groups = (n + p2::CH_GROUP_LINES - 1) / p2::CH_GROUP_LINES;
+    if (parts > 0x7FFFFFFF || groups * p2::CH_GROUP_LINES * parts > 0x7FFFFFFF) return P2_EINVAL;
+    hipLaunchKernelGGL(p2::flop_expand_lines_kernel, dim3(p2::chance_grid(n, (int)parts, p2::CH_GROUP_LINES)),
+                       dim3(p2::CH_BLOCK), 0, (hipStream_t)stream, pre_beliefs, root_indices, flops, n_flops, out, n,
+                       run, (int)parts);
+    P2_LAUNCH_CHECK();
+    return 0;
+  }
+  // row-wise kernel, about four flops per workgroup: fewer make the per-workgroup card-sum preamble dominate
+  // (1024 states x 256 flops: 16 per workgroup 874 us, 4: 658 us, 1: 1096 us)
   const int64_t want = (n_flops + 3) / 4;
   const unsigned split = (unsigned)(want < 65535 ? want : 65535);
   hipLaunchKernelGGL(p2::flop_expand_kernel, dim3((unsigned)n, split), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,

@@ -54,6 +54,50 @@ def test_expand_matches_oracle_mixed_streets(K):
     np.testing.assert_allclose(got, e_post, rtol=1e-5, atol=1e-9)        # float32 tolerance 1e-5 relative
 
 
+def _expand_through_abi(pre, roots, boards, offset_floats):
+    """p2hip_chance_expand with the output `offset_floats` floats into a buffer: 0 keeps it 16-byte
+    aligned (whole-line kernel), 2 leaves it 8-byte aligned (row-wise kernel)."""
+    from poker2_amd import _lib
+    b = roots.numel()
+    on_board = (boards[roots] >= 0).sum(1)
+    offsets = torch.zeros(b + 1, dtype=torch.int64, device=pre.device)
+    offsets[1:] = torch.cumsum(52 - on_board, 0)
+    total = int(offsets[-1])
+    buf = torch.full((total * 2 * H + 8,), float("nan"), device=pre.device)
+    post = buf[offset_floats:offset_floats + total * 2 * H]
+    bs = torch.full((total, 5), -7, dtype=torch.int64, device=pre.device)
+    lookup = torch.full((total,), -7, dtype=torch.int64, device=pre.device)
+    _lib.call("p2hip_chance_expand", _lib.ptr(pre), _lib.ptr(roots), _lib.ptr(boards), b, _lib.ptr(offsets),
+              pre.shape[0], total, post.data_ptr(), _lib.ptr(bs), _lib.ptr(lookup), _lib.stream_ptr())
+    torch.cuda.synchronize()
+    assert torch.isnan(buf[:offset_floats]).all() and torch.isnan(buf[offset_floats + total * 2 * H:]).all()
+    return post.view(total, 2, H), bs, lookup
+
+
+@pytest.mark.parametrize("n", [5, 261, 1030])
+def test_expand_whole_line_and_row_wise_kernels_agree_with_the_oracle(K, n):
+    """Both forms of the expansion (16-byte aligned buffers -> whole 128-byte lines; 8-byte aligned ->
+    rows as float2) on mixed boards: bit-identical to each other, and the oracle's samples to 1e-5.
+    261 and 1030 states take runs of 13 cards per workgroup and end in a short group of states."""
+    rng = np.random.default_rng(50 + n)
+    boards, pre = inputs(rng, n, [4, 3, 4, 0, 4])
+    pre[1, 0] = 0.0
+    pre[2, 1] = 0.0
+    pre[2, 1, 7] = 1.0
+    roots = rng.permutation(n)[: max(n - 3, 1)]
+    tp, tr, tb = torch.from_numpy(pre).cuda(), torch.from_numpy(roots).cuda(), torch.from_numpy(boards).cuda()
+    wide = _expand_through_abi(tp, tr, tb, 0)
+    narrow = _expand_through_abi(tp, tr, tb, 2)
+    for x, y in zip(wide, narrow):
+        assert torch.equal(x, y)
+    e_post, e_bs, e_lookup = OCH.expand(pre[roots], boards[roots])
+    assert torch.equal(wide[1].cpu(), torch.from_numpy(e_bs))
+    assert torch.equal(wide[2].cpu(), torch.from_numpy(e_lookup))
+    got = wide[0].cpu().numpy()
+    assert ((got == 0) == (e_post == 0)).all()
+    np.testing.assert_allclose(got, e_post, rtol=1e-5, atol=1e-9)
+
+
 def test_mean_matches_oracle_and_ragged_counts(K):
     rng = np.random.default_rng(6)
     counts = np.array([48, 49, 0, 52, 1])
@@ -276,6 +320,38 @@ def test_flop_expand_matches_oracle(K):
     # no flops: an empty result, no launch
     assert K.flop_expand(torch.from_numpy(pre).cuda(), torch.from_numpy(roots).cuda(),
                          torch.zeros(0, 3, dtype=torch.long).cuda()).shape == (5, 0, 2, H)
+
+
+@pytest.mark.parametrize("n,k", [(3, 5), (13, 37), (70, 129)])
+def test_flop_expand_whole_line_and_row_wise_kernels_agree(K, n, k):
+    """p2hip_flop_expand into a 16-byte aligned and into an 8-byte aligned buffer: bit-identical, and equal
+    to the oracle to 1e-5 (70 x 129 takes eight flops per workgroup, the others four)."""
+    from poker2_amd import _lib
+    rng = np.random.default_rng(n * 100 + k)
+    pre = rng.gamma(0.5, size=(n, 2, H)).astype(np.float32)
+    pre /= pre.sum(-1, keepdims=True)
+    pre[1, 0] = 0.0
+    flops = np.stack([rng.permutation(52)[:3] for _ in range(k)]).astype(np.int64)
+    flops[2] = [9, 9, 30]                # not three distinct cards: an all-zero sample
+    tp, tf = torch.from_numpy(pre).cuda(), torch.from_numpy(flops).cuda()
+    roots = torch.arange(n).cuda()
+    outs = []
+    for offset in (0, 2):
+        buf = torch.full((n * k * 2 * H + 8,), float("nan"), device="cuda")
+        out = buf[offset:offset + n * k * 2 * H]
+        _lib.call("p2hip_flop_expand", _lib.ptr(tp), _lib.ptr(roots), n, _lib.ptr(tf), k, out.data_ptr(),
+                  _lib.stream_ptr())
+        torch.cuda.synchronize()
+        assert torch.isnan(buf[:offset]).all() and torch.isnan(buf[offset + n * k * 2 * H:]).all()
+        outs.append(out.view(n, k, 2, H))
+    assert torch.equal(outs[0], outs[1])
+    ok = np.ones(k, dtype=bool)
+    ok[2] = False
+    exp = OCH.flop_expand(pre, flops[ok])
+    got = outs[0].cpu().numpy()
+    assert (got[:, 2] == 0).all()
+    assert ((got[:, ok] == 0) == (exp == 0)).all()
+    np.testing.assert_allclose(got[:, ok], exp, rtol=1e-5, atol=1e-9)
 
 
 @pytest.mark.parametrize("lead", [(5,), (3, 2), (2, 3, 2), (0, 2)])
