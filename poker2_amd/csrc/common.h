@@ -46,22 +46,47 @@ __device__ __forceinline__ int p2_combo_index(int lo, int hi) {
 }
 
 // ---- wave64 primitives ------------------------------------------------------
-// DPP move with zero fill: lanes without a source (row edge, masked row) read 0.
-template <int CTRL, int ROW_MASK>
+// DPP move with zero fill: lanes without a source (row edge) read 0.
+template <int CTRL>
 __device__ __forceinline__ float p2_dpp0(float v) {
-  return __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+
+// The two row-broadcast steps that end a wave scan: the last lane of row 0 / 2 is added to rows 1 / 3,
+// then lane 31 to rows 2 and 3.  Written as the add with a DPP operand and a row mask (lanes of the
+// masked rows keep their value); from the builtin the compiler makes a zero, a DPP move and an add for
+// each.  The leading s_nop covers the wait states a DPP read needs after a VALU write of its source
+// (2) or of EXEC (5), which nobody inserts around inline assembly; inside, the other value's
+// instruction and one s_nop separate each write from the DPP read of the same register.
+__device__ __forceinline__ void p2_scan_row_carries(float& a, float& b) {
+  asm volatile(
+      "s_nop 4\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void p2_scan_row_carries(float& a) {
+  asm volatile(
+      "s_nop 4\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(a));
 }
 
 // Inclusive prefix sum over the 64 lanes: four row shifts inside each 16-lane row, then two
 // row broadcasts carry the row totals across (six VALU ops, no LDS traffic).
 __device__ __forceinline__ float p2_wave_scan_incl(float v) {
-  v += p2_dpp0<0x111, 0xF>(v);  // row_shr:1
-  v += p2_dpp0<0x112, 0xF>(v);  // row_shr:2
-  v += p2_dpp0<0x114, 0xF>(v);  // row_shr:4
-  v += p2_dpp0<0x118, 0xF>(v);  // row_shr:8
-  v += p2_dpp0<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
-  v += p2_dpp0<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+  v += p2_dpp0<0x111>(v);  // row_shr:1
+  v += p2_dpp0<0x112>(v);  // row_shr:2
+  v += p2_dpp0<0x114>(v);  // row_shr:4
+  v += p2_dpp0<0x118>(v);  // row_shr:8
+  p2_scan_row_carries(v);
   return v;
 }
 __device__ __forceinline__ float p2_wave_scan_incl(float v, int /*lane*/) { return p2_wave_scan_incl(v); }
@@ -69,12 +94,11 @@ __device__ __forceinline__ float p2_wave_scan_incl(float v, int /*lane*/) { retu
 // Two independent scans in lockstep: each DPP step of one fills the two wait states the other
 // needs between writing a register and reading it through DPP.
 __device__ __forceinline__ void p2_wave_scan_incl2(float& a, float& b) {
-  a += p2_dpp0<0x111, 0xF>(a); b += p2_dpp0<0x111, 0xF>(b);
-  a += p2_dpp0<0x112, 0xF>(a); b += p2_dpp0<0x112, 0xF>(b);
-  a += p2_dpp0<0x114, 0xF>(a); b += p2_dpp0<0x114, 0xF>(b);
-  a += p2_dpp0<0x118, 0xF>(a); b += p2_dpp0<0x118, 0xF>(b);
-  a += p2_dpp0<0x142, 0xA>(a); b += p2_dpp0<0x142, 0xA>(b);
-  a += p2_dpp0<0x143, 0xC>(a); b += p2_dpp0<0x143, 0xC>(b);
+  a += p2_dpp0<0x111>(a); b += p2_dpp0<0x111>(b);
+  a += p2_dpp0<0x112>(a); b += p2_dpp0<0x112>(b);
+  a += p2_dpp0<0x114>(a); b += p2_dpp0<0x114>(b);
+  a += p2_dpp0<0x118>(a); b += p2_dpp0<0x118>(b);
+  p2_scan_row_carries(a, b);
 }
 
 __device__ __forceinline__ float p2_wave_sum(float v) {

@@ -279,13 +279,18 @@ __global__ __launch_bounds__(SD_BLOCK) void showdown_setup_sorted_kernel(const i
 // ---- per-call evaluation ---------------------------------------------------------
 constexpr int SD_PPT = 6;  // consecutive sorted positions per thread: 256 * 6 = 1536 >= 1326
 
+// Row pitch of the per-card prefixes in float2.  With 52 a card's row starts 104 banks after its
+// neighbour's, so cards 8 apart share their banks and the look-ups of a card's total (column 51) of 32
+// lanes fall on 8 bank pairs; 53 spreads rows over all 32 pairs.
+constexpr int SD_PC_STRIDE = 53;
+
 // Everything the evaluation of one node needs in LDS.  The two heroes index every table alike
 // (positions, tie groups and card lists depend on the board only), so their values sit side by
 // side and one 64-bit LDS access serves both.
 struct ShowdownLds {
   __align__(8) float2 v[P2_H + 2];        // .x / .y = villain-of-hero-0 / -1 range in strength order (beliefs[1] / [0] sorted)
   float2 P[P2_H + 2];                     // exclusive prefix, k = 0..1326
-  float2 Pc[P2_CARDS][52];                // per-card exclusive prefix, Pc[c][j], j = 0..51
+  float2 Pc[P2_CARDS][SD_PC_STRIDE];      // per-card exclusive prefix, Pc[c][j], j = 0..51
   float part[2][SD_WAVES];
 };
 

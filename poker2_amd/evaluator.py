@@ -74,6 +74,11 @@ _PHASE_12, _PHASE_3, _PHASE_1, _PHASE_2 = 1, 2, 4, 8
 # half the tree, deeper cuts put more of the tree into the few top items.
 SPLIT_ROOTS_BELOW = 400
 SPLIT_CUT_LEVEL = 2
+# Trees with raises (57 and 105 nodes per root against 21) gain from the cut at every batch size: their
+# subtrees differ in size and the items are started largest first (three raises: 1024 roots 3.96 -> 3.73 ms,
+# 4096 roots 14.75 -> 14.41 ms; two raises: 1024 roots 2.15 -> 2.07 ms, 4096 roots 7.93 -> 7.76 ms; the
+# 21-node trees lose 3-7 % above 400 roots).
+SPLIT_NODES_PER_ROOT = 50
 
 
 def _cfr_type_name(x) -> str:
@@ -316,7 +321,7 @@ class HipSparseCFREvaluator:
         self._iter_args_sub = None
         split = self.split_small_batches
         if split is None:
-            split = N < SPLIT_ROOTS_BELOW
+            split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
         self._items = self._split_items(tree) if split else None
         self._root_items = None
         if self._items is None and T:
