@@ -66,41 +66,89 @@ __global__ __launch_bounds__(DG_BLOCK) void bet_amounts_kernel(const int64_t* __
 
 // out[k, h, a] = policy_avg[c, h] for the child c of node rows[k] reached by action a, 0 where the
 // action has no child.  One workgroup per node: the children's rows are read whole (coalesced
-// float2), transposed through LDS and written as one contiguous [H * A] run of float2.  A is a
-// template parameter so that the (hand, action) split of an output index is a multiplication.
-template <int A>
+// float2) and scattered into LDS in the output's own [hand][action] order, so the node's output is
+// a plain copy of that LDS image as one contiguous run.  A is a template parameter.
+template <int A, bool WIDE>
 __global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* __restrict__ policy_avg,
                                                                    const int64_t* __restrict__ rows,
                                                                    const int64_t* __restrict__ child_offsets,
                                                                    const int64_t* __restrict__ child_count,
                                                                    const int64_t* __restrict__ action_from_parent,
                                                                    float* __restrict__ out) {
-  constexpr int STRIDE = P2_H + 2;                 // floats between action rows in LDS (keeps float2 alignment)
-  __shared__ __align__(8) float tile[A][STRIDE];
+  constexpr int HA = P2_H * A;                     // even: 1326 is
+  __shared__ __align__(16) float tile[HA + 4];     // tile[h * A + a]
   const int64_t k = blockIdx.x;
   const int64_t r = rows[k];
   const int64_t first = child_offsets[r];
   const int n_children = (int)child_count[r];
+  // All of the node's rows are requested before the first is scattered: one round trip to memory per
+  // node instead of one per child and piece (children beyond A cannot exist; the loop after the
+  // unrolled part only keeps such input from being dropped silently).
+  constexpr int PIECES = (P2_HPAIRS + DG_BLOCK - 1) / DG_BLOCK;
+  float2 x[A][PIECES];
+  int act[A];
+#pragma unroll
+  for (int j = 0; j < A; ++j) {
+    const bool have = j < n_children;
+    const int64_t row = first + (have ? j : 0);
+    const int a = have ? (int)action_from_parent[row] : -1;
+    act[j] = (a >= 0 && a < A) ? a : -1;
+    const float2* src = p2_row2(policy_avg, row);
+#pragma unroll
+    for (int q = 0; q < PIECES; ++q) {
+      const int idx = threadIdx.x + q * DG_BLOCK;
+      x[j][q] = idx < P2_HPAIRS ? src[idx] : make_float2(0.f, 0.f);
+    }
+  }
   uint32_t present = 0;
-  for (int j = 0; j < n_children; ++j) {
+#pragma unroll
+  for (int j = 0; j < A; ++j) {
+    if (act[j] < 0) continue;
+    present |= 1u << act[j];
+#pragma unroll
+    for (int q = 0; q < PIECES; ++q) {
+      const int idx = threadIdx.x + q * DG_BLOCK;
+      if (idx >= P2_HPAIRS) continue;
+      tile[2 * idx * A + act[j]] = x[j][q].x;
+      tile[(2 * idx + 1) * A + act[j]] = x[j][q].y;
+    }
+  }
+  for (int j = A; j < n_children; ++j) {
     const int a = (int)action_from_parent[first + j];
     if (a < 0 || a >= A) continue;
     present |= 1u << a;
     const float2* src = p2_row2(policy_avg, first + j);
-    for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += DG_BLOCK) reinterpret_cast<float2*>(tile[a])[idx] = src[idx];
+    for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += DG_BLOCK) {
+      const float2 v = src[idx];
+      tile[2 * idx * A + a] = v.x;
+      tile[(2 * idx + 1) * A + a] = v.y;
+    }
   }
 #pragma unroll
   for (int a = 0; a < A; ++a)
     if (!((present >> a) & 1u))
-      for (int idx = threadIdx.x; idx < P2_HPAIRS; idx += DG_BLOCK)
-        reinterpret_cast<float2*>(tile[a])[idx] = make_float2(0.f, 0.f);
+      for (int h = threadIdx.x; h < P2_H; h += DG_BLOCK) tile[h * A + a] = 0.f;
   p2_sync_lds();
-  float2* dst = reinterpret_cast<float2*>(out + k * (int64_t)P2_H * A);   // 8-byte aligned: H * A * 4 is a multiple of 8
-  for (int e2 = threadIdx.x; e2 < P2_H * A / 2; e2 += DG_BLOCK) {
-    const int e = 2 * e2;
-    const int h0 = e / A, a0 = e - h0 * A;
-    const int h1 = (e + 1) / A, a1 = (e + 1) - h1 * A;
-    dst[e2] = make_float2(tile[a0][h0], tile[a1][h1]);
+  const float2* tile2 = reinterpret_cast<const float2*>(tile);
+  if (!WIDE) {
+    float2* dst = reinterpret_cast<float2*>(out + k * (int64_t)HA);   // 8-byte aligned: HA * 4 is a multiple of 8
+    for (int e2 = threadIdx.x; e2 < HA / 2; e2 += DG_BLOCK) dst[e2] = tile2[e2];
+    return;
+  }
+  // `out` is 16-byte aligned: float4 at absolute positions, lanes placed on absolute 128-byte lines,
+  // so every wave-wide store covers whole lines although a node's run starts on none (HA * 4 bytes
+  // is a multiple of 8 only).  A float4 that straddles the run's start or end (at most one each) is
+  // written as the float2 that belongs to this node.
+  const int64_t span0 = k * (int64_t)HA;           // first float of the node, even
+  const int64_t g_first = span0 >> 2, g_end = (span0 + HA + 3) >> 2;
+  for (int64_t g = (g_first & ~7ll) + threadIdx.x; g < g_end; g += DG_BLOCK) {
+    const int e = (int)((g << 2) - span0);         // the float4's first float inside the node: even, may be < 0
+    const bool lo_ok = e >= 0 && e + 2 <= HA, hi_ok = e + 2 >= 0 && e + 4 <= HA;
+    const int i2 = e >= 0 ? e >> 1 : 0;
+    const float2 lo = tile2[i2], hi = tile2[e + 2 >= 0 ? (e + 2) >> 1 : 0];   // inside the padded tile either way
+    if (lo_ok && hi_ok) reinterpret_cast<float4*>(out)[g] = make_float4(lo.x, lo.y, hi.x, hi.y);
+    else if (lo_ok) reinterpret_cast<float2*>(out)[2 * g] = lo;
+    else if (hi_ok) reinterpret_cast<float2*>(out)[2 * g + 1] = hi;
   }
 }
 
@@ -227,11 +275,17 @@ int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n
   if (!policy_avg || !rows || !child_offsets || !child_count || !action_from_parent || !out) return P2_EINVAL;
   if (n_rows > 0x7FFFFFFF) return P2_EINVAL;
   if ((reinterpret_cast<uintptr_t>(policy_avg) & 7u) || (reinterpret_cast<uintptr_t>(out) & 7u)) return P2_EINVAL;
+  const bool wide = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
 #define P2_PT_CASE(A)                                                                                          \
   case A:                                                                                                      \
-    hipLaunchKernelGGL(p2::policy_targets_kernel<A>, dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), 0,            \
-                       (hipStream_t)stream, policy_avg, rows, child_offsets, child_count, action_from_parent,  \
-                       out);                                                                                   \
+    if (wide)                                                                                                  \
+      hipLaunchKernelGGL((p2::policy_targets_kernel<A, true>), dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), 0,  \
+                         (hipStream_t)stream, policy_avg, rows, child_offsets, child_count,                    \
+                         action_from_parent, out);                                                             \
+    else                                                                                                       \
+      hipLaunchKernelGGL((p2::policy_targets_kernel<A, false>), dim3((unsigned)n_rows), dim3(p2::DG_BLOCK), 0, \
+                         (hipStream_t)stream, policy_avg, rows, child_offsets, child_count,                    \
+                         action_from_parent, out);                                                             \
     break;
   switch (num_actions) {
     P2_PT_CASE(1) P2_PT_CASE(2) P2_PT_CASE(3) P2_PT_CASE(4) P2_PT_CASE(5) P2_PT_CASE(6) P2_PT_CASE(7) P2_PT_CASE(8)

@@ -355,6 +355,18 @@ def test_policy_targets_kernel_matches_pull_back_on_a_deep_tree():
     rows = torch.from_numpy(rng.permutation(top)[: top // 2]).to(DEV)             # any rows, any order, leaves too
     got = ev._policy_targets(rows).cpu().numpy()
     assert np.array_equal(got, exp[rows.cpu().numpy()])                             # a gather: exact
+    # the same into a buffer that is only 8-byte aligned (rows as float2 instead of whole 128-byte lines),
+    # with guard floats on both sides
+    from poker2_amd import _lib
+    k, a = rows.numel(), ev.num_actions
+    for offset in (0, 2):
+        buf = torch.full((k * H * a + 8,), float("nan"), device=DEV)
+        out = buf[offset:offset + k * H * a]
+        _lib.call("p2hip_policy_targets", _lib.ptr(ev.policy_probs_avg), _lib.ptr(rows), k, _lib.ptr(ev.child_offsets),
+                  _lib.ptr(ev.child_count), _lib.ptr(ev.action_from_parent), a, out.data_ptr(), _lib.stream_ptr())
+        torch.cuda.synchronize()
+        assert torch.isnan(buf[:offset]).all() and torch.isnan(buf[offset + k * H * a:]).all()
+        assert np.array_equal(out.view(k, H, a).cpu().numpy(), got)
     assert ev._policy_targets(rows[:0]).shape == (0, H, ev.num_actions)
     with pytest.raises(IndexError):
         ev._policy_targets(torch.tensor([ev.total_nodes], device=DEV))
