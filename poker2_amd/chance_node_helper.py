@@ -151,7 +151,12 @@ def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, fl
     return post
 
 
-PERM_MEAN_TARGET_WORKGROUPS = 2048   # 256 CUs x 8
+# Workgroups wanted from the (state, player) x share split of the flop means.  perm_mean keeps six
+# workgroups per CU resident, so 2048 leave a second, quarter-full round (1024 states x 256 flops:
+# 812 us with one share, 688 us with two, 670 us with three); orbit_mean is lighter per row and fastest
+# with the fewest shares that fill the chip once (470 us against 494 us with two).
+PERM_MEAN_TARGET_WORKGROUPS = 4096
+ORBIT_MEAN_TARGET_WORKGROUPS = 2048   # 256 CUs x 8
 
 
 def perm_mean(hand_values: torch.Tensor, perms: torch.Tensor, weight: torch.Tensor,
@@ -232,7 +237,7 @@ def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tenso
     else:
         _req(out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous(),
              "out.shape == (b, 2, NUM_HANDS) and out.dtype == torch.float32 and out.is_contiguous()")
-    shares = max(1, min(k, -(-PERM_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
+    shares = max(1, min(k, -(-ORBIT_MEAN_TARGET_WORKGROUPS // max(1, 2 * b))))
     if static_scratch:
         if not accumulate:
             raise ValueError("static_scratch=True allocates nothing: pass the output tensor as `out`")

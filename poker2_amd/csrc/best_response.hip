@@ -21,6 +21,7 @@ namespace p2 {
 constexpr int BR_BLOCK = 256;
 constexpr int BR_PPT = 3;
 constexpr int BR_MAXC = 8;
+constexpr int BR_GRP = 4;   // children whose rows are in flight together
 constexpr int BR_STRIDE = P2_H + 2;
 static_assert(BR_BLOCK == UB_BLOCK, "card_sums_multi assumes the block size");
 
@@ -56,23 +57,45 @@ __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
     }
     if (in) reinterpret_cast<float2*>(t[nc])[idx] = x;
   }
+  // Children are taken in groups of BR_GRP whose rows are all requested before the first is used
+  // (indices beyond the last child repeat it: a cache hit instead of a branch around every load), so a
+  // parent with up to four children costs one round trip to memory per pass instead of one per child.
+  auto load_group = [&](const float* __restrict__ base, int64_t row0, int64_t row_step, int plane, int g0,
+                        float2 (&dst)[BR_GRP][BR_PPT]) {
+#pragma unroll
+    for (int j = 0; j < BR_GRP; ++j) {
+      const int c = g0 + j < nc ? g0 + j : nc - 1;
+      const float2* src = p2_row2(base, (row0 + c) * row_step + plane);
+#pragma unroll
+      for (int k = 0; k < BR_PPT; ++k) {
+        const int idx = threadIdx.x + k * BR_BLOCK;
+        dst[j][k] = src[idx < P2_HPAIRS ? idx : 0];
+      }
+    }
+  };
   // pass 1: the actor's value and (for a deviating actor) each hand's maximising child
-  for (int c = 0; c < nc; ++c) {
+  for (int g0 = 0; g0 < nc; g0 += BR_GRP) {
+    float2 v[BR_GRP][BR_PPT], pi[BR_GRP][BR_PPT];
+    load_group(values, c0, 2, actor, g0, v);
+    if (!is_dev) load_group(policy, c0, 1, 0, g0, pi);
 #pragma unroll
-    for (int k = 0; k < BR_PPT; ++k) {
-      const int idx = threadIdx.x + k * BR_BLOCK;
-      if (idx >= P2_HPAIRS) continue;
-      const float2 v = p2_row2(values, (c0 + c) * 2 + actor)[idx];
-      const float vv[2] = {v.x, v.y};
-      if (is_dev) {
+    for (int j = 0; j < BR_GRP; ++j) {
+      const int c = g0 + j;
+      if (c >= nc) break;
 #pragma unroll
-        for (int q = 0; q < 2; ++q)
-          if (vv[q] > av[k][q]) { av[k][q] = vv[q]; best[k][q] = c; }
-      } else {
-        const float2 pi = p2_row2(policy, c0 + c)[idx];
-        av[k][0] += vv[0] * pi.x;
-        av[k][1] += vv[1] * pi.y;
-        reinterpret_cast<float2*>(t[c])[idx] = make_float2(b[k][0] * pi.x, b[k][1] * pi.y);
+      for (int k = 0; k < BR_PPT; ++k) {
+        const int idx = threadIdx.x + k * BR_BLOCK;
+        if (idx >= P2_HPAIRS) continue;
+        const float vv[2] = {v[j][k].x, v[j][k].y};
+        if (is_dev) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+            if (vv[q] > av[k][q]) { av[k][q] = vv[q]; best[k][q] = c; }
+        } else {
+          av[k][0] += vv[0] * pi[j][k].x;
+          av[k][1] += vv[1] * pi[j][k].y;
+          reinterpret_cast<float2*>(t[c])[idx] = make_float2(b[k][0] * pi[j][k].x, b[k][1] * pi[j][k].y);
+        }
       }
     }
   }
@@ -87,6 +110,9 @@ __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
       }
     }
   }
+  // the other player's values of the first group are requested before the card sums and arrive behind them
+  float2 vo[BR_GRP][BR_PPT];
+  load_group(values, c0, 2, 1 - actor, 0, vo);
   p2_sync_lds();
   card_sums_multi(t[0], BR_STRIDE, nc + 1, cs);
   // pass 2: the other player's value under the projected action probabilities
@@ -100,22 +126,27 @@ __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
       ub[k][q] = fmaxf((float)v, 0.f);
       ov[k][q] = 0.f;
     }
-  for (int c = 0; c < nc; ++c) {
-    const double* csc = cs + c * P2_CARDS;
-    const double total_c = card_total(csc);
+  for (int g0 = 0; g0 < nc; g0 += BR_GRP) {
+    if (g0 > 0) load_group(values, c0, 2, 1 - actor, g0, vo);
 #pragma unroll
-    for (int k = 0; k < BR_PPT; ++k) {
-      const int idx = threadIdx.x + k * BR_BLOCK;
-      if (idx >= P2_HPAIRS) continue;
-      const float2 vo = p2_row2(values, (c0 + c) * 2 + (1 - actor))[idx];
-      const float2 m = reinterpret_cast<const float2*>(t[c])[idx];
-      const float mm[2] = {m.x, m.y}, vv[2] = {vo.x, vo.y};
+    for (int j = 0; j < BR_GRP; ++j) {
+      const int c = g0 + j;
+      if (c >= nc) break;
+      const double* csc = cs + c * P2_CARDS;
+      const double total_c = card_total(csc);
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const double u = total_c - csc[ab[k][q] & 0xFFu] - csc[ab[k][q] >> 8] + (double)mm[q];
-        const float uc = fmaxf((float)u, 0.f);
-        const float prob = ub[k][q] > 1e-5f ? uc / ub[k][q] : 0.f;
-        ov[k][q] += prob * vv[q];
+      for (int k = 0; k < BR_PPT; ++k) {
+        const int idx = threadIdx.x + k * BR_BLOCK;
+        if (idx >= P2_HPAIRS) continue;
+        const float2 m = reinterpret_cast<const float2*>(t[c])[idx];
+        const float mm[2] = {m.x, m.y}, vv[2] = {vo[j][k].x, vo[j][k].y};
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const double u = total_c - csc[ab[k][q] & 0xFFu] - csc[ab[k][q] >> 8] + (double)mm[q];
+          const float uc = fmaxf((float)u, 0.f);
+          const float prob = ub[k][q] > 1e-5f ? uc / ub[k][q] : 0.f;
+          ov[k][q] += prob * vv[q];
+        }
       }
     }
   }

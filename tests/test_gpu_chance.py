@@ -367,10 +367,20 @@ def test_avg_over_perms_any_leading_shape(K, lead):
     np.testing.assert_allclose(got.cpu().numpy(), exp, rtol=1e-5, atol=2e-6)
 
 
-@pytest.mark.parametrize("n_perms", [1, 6, 24])
-def test_perm_mean_matches_numpy(K, n_perms):
-    rng = np.random.default_rng(22 + n_perms)
-    perms = OCH.combo_suit_perms()[rng.permutation(24)[:n_perms]]
+@pytest.mark.parametrize("n_perms,kind", [(1, "suits"), (6, "suits"), (8, "suits"), (24, "suits"),
+                                          (6, "any"), (6, "one_off"), (3, "not_bijective")])
+def test_perm_mean_matches_numpy(K, n_perms, kind):
+    """Suit permutations (up to 8 of them sit in registers, more in LDS), arbitrary permutations of
+    the hands, a suit permutation with two hands swapped, and a table that is no permutation at all
+    (every hand reads the same source): all are plain gathers."""
+    rng = np.random.default_rng(22 + n_perms + len(kind))
+    perms = OCH.combo_suit_perms()[rng.permutation(24)[:n_perms]].copy()
+    if kind == "any":
+        perms[2] = rng.permutation(H)
+    elif kind == "one_off":
+        perms[4, [700, 701]] = perms[4, [701, 700]]
+    elif kind == "not_bijective":
+        perms[1] = perms[1][0]
     hv = rng.standard_normal((3, 11, 2, H)).astype(np.float32)
     w = rng.random(11).astype(np.float32)
     exp = np.zeros((3, 2, H))
