@@ -79,7 +79,7 @@ def test_turn_subgames_with_chance_leaves_B512():
         for lin in net.linears:
             lin.weight.mul_(2.0)
 
-    def run(n):
+    def run(n, iters=iters):
         roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards[:n],
                                           button=np.arange(n) % 2)
         ev = HipSparseCFREvaluator(ChanceLeafModel(net, dev), dev, river_dcfr_config(n, iterations=iters, depth=16,
@@ -89,9 +89,16 @@ def test_turn_subgames_with_chance_leaves_B512():
         for t in range(iters):
             ev.cfr_iteration(t)
         return ev
-    ev = run(b)
+    # the configuration's own length: 100 iterations at the full batch, checked by what every state must satisfy
+    ev = run(b, 100)
     assert ev.total_nodes == 21 * b and ev.model_indices.numel() == 7 * b        # 7 street-end leaves per root
     assert float(ev.latest_values[ev.model_indices].abs().max()) > 1e-3          # the network matters
+    check_distributions(ev, rng)
+    stats = ev._compute_exploitability()
+    assert torch.isfinite(stats.local_exploitability).all() and float(stats.local_exploitability.min()) > -1e-4
+    del ev, stats
+    # batch independence over a few iterations (longer runs of two float32 programs drift apart on their own)
+    ev = run(b)
     check_distributions(ev, rng)
     ref = run(small)
     rows = rows_of_first_roots(ev, small)
@@ -115,7 +122,7 @@ def test_data_generation_step_B16384():
         for lin in net.linears:
             lin.weight.mul_(2.0)
 
-    def run(n, autocast):
+    def run(n, autocast, iters=iters):
         gen = torch.Generator(device=dev)
         gen.manual_seed(1)
         model = NetworkLeafModel(net, dev, autocast_dtype=autocast)
@@ -124,7 +131,7 @@ def test_data_generation_step_B16384():
         ev.initialize_subgame(roots.select(np.arange(n)), np.arange(n), bel[:n])
         nxt = ev.evaluate_cfr()
         return ev, nxt
-    ev, nxt = run(b, torch.bfloat16)
+    ev, nxt = run(b, torch.bfloat16, 64)                                          # the configuration's own 64 iterations
     assert ev.total_nodes > 20 * b and ev.model_indices.numel() > b and ev.showdown_indices.numel() > b
     check_distributions(ev, rng)
     assert nxt.roots.n == b                                                       # one sampled leaf per root
