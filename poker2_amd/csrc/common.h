@@ -69,6 +69,20 @@ __device__ __forceinline__ void p2_scan_row_carries(float& a, float& b) {
       "s_nop 1"
       : "+v"(a), "+v"(b));
 }
+__device__ __forceinline__ void p2_scan_row_carries(float& a, float& b, float& c, float& d) {
+  asm volatile(
+      "s_nop 4\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+      "s_nop 1"
+      : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
 __device__ __forceinline__ void p2_scan_row_carries(float& a) {
   asm volatile(
       "s_nop 4\n\t"
@@ -99,6 +113,16 @@ __device__ __forceinline__ void p2_wave_scan_incl2(float& a, float& b) {
   a += p2_dpp0<0x114>(a); b += p2_dpp0<0x114>(b);
   a += p2_dpp0<0x118>(a); b += p2_dpp0<0x118>(b);
   p2_scan_row_carries(a, b);
+}
+
+// Four scans in lockstep (two cards' lists of both players): every DPP step has three independent
+// instructions between a register's write and its next DPP read.
+__device__ __forceinline__ void p2_wave_scan_incl4(float& a, float& b, float& c, float& d) {
+  a += p2_dpp0<0x111>(a); b += p2_dpp0<0x111>(b); c += p2_dpp0<0x111>(c); d += p2_dpp0<0x111>(d);
+  a += p2_dpp0<0x112>(a); b += p2_dpp0<0x112>(b); c += p2_dpp0<0x112>(c); d += p2_dpp0<0x112>(d);
+  a += p2_dpp0<0x114>(a); b += p2_dpp0<0x114>(b); c += p2_dpp0<0x114>(c); d += p2_dpp0<0x114>(d);
+  a += p2_dpp0<0x118>(a); b += p2_dpp0<0x118>(b); c += p2_dpp0<0x118>(c); d += p2_dpp0<0x118>(d);
+  p2_scan_row_carries(a, b, c, d);
 }
 
 __device__ __forceinline__ float p2_wave_sum(float v) {

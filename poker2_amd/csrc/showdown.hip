@@ -386,17 +386,42 @@ __device__ __forceinline__ void showdown_scans(const float (&vk)[2][SD_PPT], con
     }
   }
   // per-card prefixes: one wave scan per (player, card); this wave owns cards wave, wave+4, ...
-  // Both players' lists of a card share the positions, so they are scanned in lockstep.
+  // Both players' lists of a card share the positions, so they are scanned in lockstep, two cards at
+  // a time; the lists of the next four cards are read from LDS before the current four are scanned.
+  auto fetch4 = [&](int i0, float2 (&x)[4]) {
 #pragma unroll
-  for (int i = 0; i < 13; ++i) {
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j < 13 ? i0 + j : 12;
+      const uint32_t pos = R.clist[i];
+      const float2 y = s.v[pos < (uint32_t)P2_H ? pos : 0u];
+      x[j] = pos < (uint32_t)P2_H ? y : make_float2(0.f, 0.f);
+    }
+  };
+  auto put = [&](int i, float x0, float x1) {
     const int c = wave + 4 * i;
-    const uint32_t pos = R.clist[i];
-    const bool in = pos < (uint32_t)P2_H;
-    const float2 x = in ? s.v[pos] : make_float2(0.f, 0.f);
-    float x0 = x.x, x1 = x.y;
-    p2_wave_scan_incl2(x0, x1);
     if (lane < 51) s.Pc[c][lane + 1] = make_float2(x0, x1);
     if (lane == 0) s.Pc[c][0] = make_float2(0.f, 0.f);
+  };
+  float2 cur[4], nxt[4];
+  fetch4(0, cur);
+#pragma unroll
+  for (int i0 = 0; i0 < 13; i0 += 4) {
+    if (i0 + 4 < 13) fetch4(i0 + 4, nxt);
+    if (i0 + 1 < 13) {
+      p2_wave_scan_incl4(cur[0].x, cur[0].y, cur[1].x, cur[1].y);
+      put(i0, cur[0].x, cur[0].y);
+      put(i0 + 1, cur[1].x, cur[1].y);
+    } else {
+      p2_wave_scan_incl2(cur[0].x, cur[0].y);
+      put(i0, cur[0].x, cur[0].y);
+    }
+    if (i0 + 3 < 13) {
+      p2_wave_scan_incl4(cur[2].x, cur[2].y, cur[3].x, cur[3].y);
+      put(i0 + 2, cur[2].x, cur[2].y);
+      put(i0 + 3, cur[3].x, cur[3].y);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cur[j] = nxt[j];
   }
   p2_sync_lds();
 }
