@@ -125,7 +125,7 @@ def cases(repeats: int):
     pre = bel[:k].contiguous()
     post, _, _, offsets = CH.chance_expand(pre, roots, tb, cards_on_board=4)
     yield ("chance_expand states=3584 x48", k * (2 + 2 * 48) * H * 4,
-           lambda: CH.chance_expand(pre, roots, tb, cards_on_board=4))
+           lambda: CH.chance_expand(pre, roots, tb, cards_on_board=4, check_rows=False))
     yield ("chance_mean states=3584 x48", k * (2 * 48 + 2) * H * 4, lambda: CH.chance_mean(post, offsets))
     del post
 
@@ -136,7 +136,7 @@ def cases(repeats: int):
     flops = torch.from_numpy(canonical[rng.integers(0, canonical.shape[0], kf)]).to(dev)
     pre_f = bel[:ks].contiguous()
     roots_f = torch.arange(ks, device=dev)
-    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops))
+    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops, check_rows=False))
     hv = CH.flop_expand(pre_f, roots_f, flops)
     perms = combo_suit_permutation_tensor(dev)[:6].to(torch.int16).contiguous()
     w = torch.full((kf,), 1.0 / kf, device=dev)
@@ -148,7 +148,7 @@ def cases(repeats: int):
     pre_f = (torch.rand(ks, 2, H, device=dev) + 1e-3)
     pre_f = pre_f / pre_f.sum(-1, keepdim=True)
     roots_f = torch.arange(ks, device=dev)
-    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops))
+    yield (f"flop_expand states={ks} x{kf}", ks * (2 + 2 * kf) * H * 4, lambda: CH.flop_expand(pre_f, roots_f, flops, check_rows=False))
     hv = CH.flop_expand(pre_f, roots_f, flops)
     yield (f"perm_mean states={ks} x{kf} perms=6", ks * (2 * kf + 2) * H * 4, lambda: CH.perm_mean(hv, perms, w, check_perms=False))
     yield (f"orbit_mean states={ks} x{kf} (all 24)", ks * (2 * kf + 2) * H * 4, lambda: CH.orbit_mean(hv, w))
@@ -167,7 +167,7 @@ def cases(repeats: int):
     rows = torch.nonzero(~ev.leaf_mask[:top]).squeeze(1)
     n_children = int(ev.child_count[rows].sum())
     yield (f"policy_targets nodes={rows.numel()}", (n_children + rows.numel() * ev.num_actions) * H * 4,
-           lambda: ev._policy_targets(rows))
+           lambda: ev._policy_targets(rows, check_rows=False))
     yield (f"encode nodes={ev.total_nodes}", ev.total_nodes * (13 * 8 + 16 + 5 * 8 + 10 * 8),
            lambda: ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask))
 

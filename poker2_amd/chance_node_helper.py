@@ -68,14 +68,21 @@ class MLPFeatures:
                    beliefs=torch.cat([f.beliefs for f in features_list], dim=0))
 
 
+def _rows_out_of_range(rows: torch.Tensor, n: int) -> bool:
+    """One device read: does any index lie outside 0..n-1?"""
+    return bool(rows.numel()) and bool(((rows < 0) | (rows >= n)).any())
+
+
 def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, board_pre: torch.Tensor,
-                  cards_on_board: int | None = None):
+                  cards_on_board: int | None = None, check_rows: bool = True):
     """Every (state, next card) sample of a single-card chance node.
 
     pre_chance_beliefs [R,2,1326] fp32, board_pre [R,5] int64 (-1 = empty), root_indices [B].
     Returns (post_beliefs [S,2,1326], board_samples [S,5], root_lookup [S], sample_offsets [B+1])
     with samples in (state, card) ascending order.  ``cards_on_board`` (same count for every
-    selected state) skips the device-to-host read of the sample count.
+    selected state) skips the device-to-host read of the sample count; ``check_rows=False`` skips the
+    one that checks ``root_indices`` (for callers whose indices are valid by construction; the kernel
+    itself leaves rows outside the table alone).
     """
     if not _lib.hip_is_available():
         raise RuntimeError("chance_expand needs libp2hip.so and a GPU (no CPU fallback exists).")
@@ -89,19 +96,21 @@ def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, 
     roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
     b = roots.numel()
     source_rows = min(pre.shape[0], board.shape[0])
-    if b and (int(roots.min()) < 0 or int(roots.max()) >= source_rows):
+    if check_rows and _rows_out_of_range(roots, source_rows):
         raise IndexError("root_indices out of range")
-    on_board = ((board[roots] >= 0) & (board[roots] < 52)).sum(dim=1)
-    offsets = torch.zeros(b + 1, dtype=torch.int64, device=dev)
-    torch.cumsum(52 - on_board, dim=0, out=offsets[1:])
     if cards_on_board is None:
+        on_board = ((board[roots] >= 0) & (board[roots] < 52)).sum(dim=1)
+        offsets = torch.zeros(b + 1, dtype=torch.int64, device=dev)
+        torch.cumsum(52 - on_board, dim=0, out=offsets[1:])
         if b and int(on_board.max().item()) >= 5:
             raise ValueError("single-card chance expansion needs an empty board slot (at most 4 cards dealt)")
         total = int(offsets[-1].item()) if b else 0
     else:
         if not 0 <= cards_on_board <= 4:
             raise ValueError("cards_on_board must be in 0..4")
-        total = b * (52 - cards_on_board)
+        per_state = 52 - cards_on_board
+        total = b * per_state
+        offsets = torch.arange(0, total + 1, per_state, dtype=torch.int64, device=dev)   # one launch, no board read
     post = torch.empty(total, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     board_samples = torch.empty(total, 5, dtype=torch.int64, device=dev)
     root_lookup = torch.empty(total, dtype=torch.int64, device=dev)
@@ -128,10 +137,12 @@ def chance_mean(hand_values: torch.Tensor, sample_offsets: torch.Tensor) -> torc
     return out
 
 
-def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, flops: torch.Tensor) -> torch.Tensor:
+def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, flops: torch.Tensor,
+                check_rows: bool = True) -> torch.Tensor:
     """pre_chance_beliefs [R,2,1326] fp32, root_indices [B], flops [K,3] card ids ->
     [B,K,2,1326]: the ranges of each selected state without the hands that touch each flop,
-    renormalised per player (uniform over the 1176 hands left where the sum is <= 1e-12)."""
+    renormalised per player (uniform over the 1176 hands left where the sum is <= 1e-12).
+    ``check_rows=False`` skips the device read that checks ``root_indices`` (the kernel does not check them)."""
     if not _lib.hip_is_available():
         raise RuntimeError("flop_expand needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(pre_chance_beliefs, "flop_expand")
@@ -141,7 +152,7 @@ def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, fl
     _req(flops.dim() == 2 and flops.shape[1] == 3, "flops.dim() == 2 and flops.shape[1] == 3")
     pre = pre_chance_beliefs.contiguous().float()
     roots = root_indices.to(device=dev, dtype=torch.int64).contiguous()
-    if roots.numel() and (int(roots.min()) < 0 or int(roots.max()) >= pre.shape[0]):
+    if check_rows and _rows_out_of_range(roots, pre.shape[0]):
         raise IndexError("root_indices out of range")
     fl = flops.to(device=dev, dtype=torch.int64).contiguous()
     b, k = roots.numel(), fl.shape[0]
@@ -346,6 +357,8 @@ class ChanceNodeHelper:
         b = roots.numel()
         pre = pre_chance_beliefs.to(device=dev).contiguous().float()
         _lib.require_gpu(pre, "flop_chance_values")
+        if _rows_out_of_range(roots, pre.shape[0]):          # once, not per chunk of flops
+            raise IndexError("root_indices out of range")
         context_root = root_features.context[roots]
         street_root = root_features.street[roots]
         to_act_root = root_features.to_act[roots]
@@ -356,7 +369,7 @@ class ChanceNodeHelper:
         def eval_chunk(canonical_chunk: torch.Tensor, weight: torch.Tensor) -> None:
             k = canonical_chunk.shape[0]
             flops = canonical_chunk.contiguous()
-            post = flop_expand(pre, roots, flops)
+            post = flop_expand(pre, roots, flops, check_rows=False)
             board5 = torch.cat([flops, torch.full((k, 2), -1, device=dev, dtype=torch.int64)], dim=1)
             feats = MLPFeatures(
                 context=context_root.unsqueeze(1).expand(-1, k, -1).reshape(-1, context_root.shape[1]),

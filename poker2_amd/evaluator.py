@@ -1011,11 +1011,11 @@ class HipSparseCFREvaluator:
             self._chance_helper = helper
         return self._chance_helper
 
-    def _policy_targets(self, rows: torch.Tensor) -> torch.Tensor:
+    def _policy_targets(self, rows: torch.Tensor, check_rows: bool = True) -> torch.Tensor:
         """[K, 1326, num_actions]: the average policy of the children of ``rows`` by action, zero
         for actions without a child (cfr_evaluator.py:1392-1393 on the selected rows)."""
         rows = rows.to(device=self.device, dtype=torch.int64).contiguous()
-        if rows.numel() and (int(rows.min()) < 0 or int(rows.max()) >= self.total_nodes):
+        if check_rows and rows.numel() and bool(((rows < 0) | (rows >= self.total_nodes)).any()):
             raise IndexError("policy target rows out of range")
         out = torch.empty(rows.numel(), NUM_HANDS, self.num_actions, dtype=self.float_dtype, device=self.device)
         _lib.call("p2hip_policy_targets", _lib.ptr(self.policy_probs_avg), _lib.ptr(rows), rows.numel(),
@@ -1053,7 +1053,7 @@ class HipSparseCFREvaluator:
         actions_root = self.env.actions_this_round[:N]
         if exclude_start:
             value_batch = value_batch[~((street_root == 0) & (actions_root == 0))]
-        policy_batch = RebelBatch(features=features[valid_top], policy_targets=self._policy_targets(policy_rows),
+        policy_batch = RebelBatch(features=features[valid_top], policy_targets=self._policy_targets(policy_rows, check_rows=False),
                                   legal_masks=legal_masks[:top][valid_top], statistics=policy_statistics)
 
         pre_features_root = self.feature_encoder.encode(self.beliefs, pre_chance_node=True,

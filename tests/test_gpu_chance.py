@@ -54,12 +54,13 @@ def test_expand_matches_oracle_mixed_streets(K):
     np.testing.assert_allclose(got, e_post, rtol=1e-5, atol=1e-9)        # float32 tolerance 1e-5 relative
 
 
-def _expand_through_abi(pre, roots, boards, offset_floats):
+def _expand_through_abi(pre, roots, boards, offset_floats, claimed_cards=None):
     """p2hip_chance_expand with the output `offset_floats` floats into a buffer: 0 keeps it 16-byte
-    aligned (whole-line kernel), 2 leaves it 8-byte aligned (row-wise kernel)."""
+    aligned (whole-line kernel), 2 leaves it 8-byte aligned (row-wise kernel).  `claimed_cards`: size
+    the offsets and the buffers for that many cards on every board, whatever the boards hold."""
     from poker2_amd import _lib
     b = roots.numel()
-    on_board = (boards[roots] >= 0).sum(1)
+    on_board = (boards[roots] >= 0).sum(1) if claimed_cards is None else torch.full((b,), claimed_cards, device=pre.device)
     offsets = torch.zeros(b + 1, dtype=torch.int64, device=pre.device)
     offsets[1:] = torch.cumsum(52 - on_board, 0)
     total = int(offsets[-1])
@@ -188,12 +189,17 @@ def test_helper_edge_cases(K):
     # where 48 were sized) cannot make the kernel write past the buffers: it stops at their end
     boards3 = boards.copy()
     boards3[1, 3] = -1
+    boards3[2, 3] = -1                                       # the last state's 49th sample would lie past the end
     c = K.chance_expand(torch.from_numpy(pre).cuda(), torch.arange(3).cuda(), torch.from_numpy(boards3).cuda(),
                         cards_on_board=4)
     torch.cuda.synchronize()
-    assert c[0].shape[0] == 3 * 48 and int(c[3][-1]) == 3 * 48 + 1      # offsets say 145, the buffers hold 144
+    assert c[0].shape[0] == 3 * 48 and int(c[3][-1]) == 3 * 48          # offsets and buffers as claimed
     assert torch.equal(c[0][:48], a[0][:48]) and torch.equal(c[2][:48], a[2][:48])
     assert int(c[2].max()) <= 2 and int(c[2].min()) >= 0
+    for offset in (0, 2):                                    # both kernels, with guard floats around the output
+        g = _expand_through_abi(torch.from_numpy(pre).cuda(), torch.arange(3).cuda(), torch.from_numpy(boards3).cuda(),
+                                offset, claimed_cards=4)
+        assert torch.equal(g[0][:48], a[0][:48])
 
 
 # ---- turn subgame: street-end leaves valued through the chance node + a small network --------
