@@ -399,13 +399,14 @@ class ChanceNodeHelper:
     @torch.no_grad()
     def single_card_chance_values(self, root_indices: torch.Tensor, root_features: MLPFeatures,
                                   pre_chance_beliefs: torch.Tensor, board_pre: torch.Tensor,
-                                  cards_on_board: int | None = None) -> torch.Tensor:
-        """Expected network values over a single-card chance node (turn or river card)."""
+                                  cards_on_board: int | None = None, check_rows: bool = True) -> torch.Tensor:
+        """Expected network values over a single-card chance node (turn or river card).
+        ``cards_on_board`` / ``check_rows``: see ``chance_expand`` (two device reads a caller can spare)."""
         if root_indices.numel() == 0:
             return torch.zeros(0, self.num_players, NUM_HANDS, device=self.device, dtype=self.float_dtype)
         root_indices = root_indices.to(self.device)
         post, board_samples, root_lookup, offsets = chance_expand(pre_chance_beliefs, root_indices, board_pre,
-                                                                  cards_on_board)
+                                                                  cards_on_board, check_rows)
         if post.shape[0] == 0:
             return torch.zeros(root_indices.numel(), self.num_players, NUM_HANDS, device=self.device,
                                dtype=self.float_dtype)

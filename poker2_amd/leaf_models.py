@@ -191,7 +191,7 @@ class ChanceLeafModel:
             for lo in range(0, plan.chance.numel(), step):
                 sel = plan.chance[lo:lo + step]
                 ev_chance = self.helper.single_card_chance_values(sel, feats, beliefs, plan.board,
-                                                                  cards_on_board=plan.cards)
+                                                                  cards_on_board=plan.cards, check_rows=False)
                 out.index_copy_(0, sel, ev_chance.to(out.dtype))
         if plan.flop.numel():
             feats = self._features(beliefs, plan)
