@@ -74,6 +74,10 @@ _PHASE_12, _PHASE_3, _PHASE_1, _PHASE_2 = 1, 2, 4, 8
 # half the tree, deeper cuts put more of the tree into the few top items.
 SPLIT_ROOTS_BELOW = 400
 SPLIT_CUT_LEVEL = 2
+# With few roots the tree tops (one workgroup per root, five families in a row) are themselves too few and
+# too long: a second cut right under the root makes the root's family one item and each of its children's
+# families another (six launches per iteration instead of four).
+SPLIT_MID_LEVEL = 1
 # Trees with raises (57 and 105 nodes per root against 21) gain from the cut at every batch size: their
 # subtrees differ in size and the items are started largest first (three raises: 1024 roots 3.96 -> 3.73 ms,
 # 4096 roots 14.75 -> 14.41 ms; two raises: 1024 roots 2.15 -> 2.07 ms, 4096 roots 7.93 -> 7.76 ms; the
@@ -187,7 +191,7 @@ class HipSparseCFREvaluator:
         self._fscal_host = (ctypes.c_float * 8)()
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
-        self._iter_args_sub = None
+        self._iter_args_tiers = None
         self._chance_helper = None
         self.subgame_serial = 0
 
@@ -318,11 +322,11 @@ class HipSparseCFREvaluator:
         self._max_children = int(tree.child_count.max()) if T else 1
         self._has_model_leaves = bool(model_mask.any())
         self._iter_args = None
-        self._iter_args_sub = None
+        self._iter_args_tiers = None
         split = self.split_small_batches
         if split is None:
             split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
-        self._items = self._split_items(tree) if split else None
+        self._items = self._split_items(tree, SPLIT_MID_LEVEL if N < SPLIT_ROOTS_BELOW else None) if split else None
         self._root_items = None
         if self._items is None and T:
             # Roots of unequal size (mixed streets, stacks, pots): one work item per root, largest tree
@@ -344,12 +348,14 @@ class HipSparseCFREvaluator:
                                                    showdown_offsets=showdown_offsets, item_root=self._t(order),
                                                    item_top=self._t(np.ones(N, np.uint8)))
 
-    def _split_items(self, tree: SparseTree):
-        """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h):
-        items 0..N-1 are the tops of the roots' trees above the cut level, items N.. the subtrees under
-        the cut level's nodes that have children.  Returns device arrays (family rows + offsets, showdown
-        rows + offsets, item_root, item_top) and the number of subtree items; None if the tree is too
-        shallow to cut."""
+    def _split_items(self, tree: SparseTree, mid_level: int | None = None):
+        """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h), in
+        tiers: tier 0 holds one item per root, the top of its tree above the first cut level; every further
+        tier one item per node of its cut level that has children, with the families from that level down
+        to the next cut level (the last tier: to the leaves).  Cut levels: ``mid_level`` (optional, must lie
+        above the main one) and SPLIT_CUT_LEVEL.  Returns device arrays over all items in tier order (family
+        rows + offsets, showdown rows + offsets, item_root, item_top) and the tiers' item counts; None if
+        the tree is too shallow to cut."""
         N, T = self.root_nodes, tree.total
         offs = tree.depth_offsets
         n_levels = len(offs) - 1
@@ -359,13 +365,7 @@ class HipSparseCFREvaluator:
             cut -= 1                                            # the deepest level that still has families below it
         if cut < 1:
             return None
-        anchor = np.full(T, -1, dtype=np.int64)                 # the cut-level node a deeper row sits under (itself there)
-        anchor[offs[cut]:offs[cut + 1]] = np.arange(offs[cut], offs[cut + 1])
-        for d in range(cut + 1, n_levels):
-            rows = np.arange(offs[d], offs[d + 1])
-            anchor[rows] = anchor[tree.parent_index[rows]]
-        subs = np.nonzero(has_children[offs[cut]:offs[cut + 1]])[0] + offs[cut]        # ascending rows
-        M = len(subs)
+        cuts = [cut] if mid_level is None or not 1 <= mid_level < cut else [mid_level, cut]
 
         def grouped(rows, keys, groups):
             """rows ordered by group (ascending inside a group) and offsets [len(groups) + 1]."""
@@ -373,40 +373,62 @@ class HipSparseCFREvaluator:
             order = np.argsort(slot, kind="stable")
             counts = np.bincount(slot, minlength=len(groups))
             return rows[order], np.concatenate([[0], np.cumsum(counts)])
-        roots = np.arange(N)
-        upper = np.nonzero(has_children[:offs[cut]])[0]
-        top_parents, top_po = grouped(upper, tree.root_index[upper], roots)
-        upper_sd = np.nonzero(tree.showdown_mask[:offs[cut + 1]])[0]
-        top_sd, top_so = grouped(upper_sd, tree.root_index[upper_sd], roots)
-        deep = np.arange(offs[cut], T)
-        sub_parent_rows = deep[has_children[deep]]
-        sub_parents, sub_po = grouped(sub_parent_rows, anchor[sub_parent_rows], subs)
-        deep_sd = np.arange(offs[cut + 1], T)
-        deep_sd = deep_sd[tree.showdown_mask[deep_sd]]
-        sub_sd, sub_so = grouped(deep_sd, anchor[deep_sd], subs)
-        # Largest subtrees first: a launch lasts until its last work item ends, and items are handed to
-        # the compute units in index order, so the long ones must not be the ones that start last.
-        size = np.bincount(np.searchsorted(subs, anchor[deep][np.isin(anchor[deep], subs)]), minlength=M)
-        order = np.argsort(-size, kind="stable")
 
-        def reordered(rows, offsets):
+        def reordered(rows, offsets, order):
             pieces = [rows[offsets[g]:offsets[g + 1]] for g in order]
             lengths = np.array([len(x) for x in pieces], dtype=np.int64)
             return (np.concatenate(pieces) if pieces else rows), np.concatenate([[0], np.cumsum(lengths)])
-        sub_parents, sub_po = reordered(sub_parents, sub_po)
-        sub_sd, sub_so = reordered(sub_sd, sub_so)
-        subs = subs[order]
-        parents = np.concatenate([top_parents, sub_parents]).astype(np.int64)
-        parent_offsets = np.concatenate([top_po, top_po[-1] + sub_po[1:]]).astype(np.int64)
-        showdown = np.concatenate([top_sd, sub_sd]).astype(np.int64)
-        showdown_offsets = np.concatenate([top_so, top_so[-1] + sub_so[1:]]).astype(np.int64)
-        item_root = np.concatenate([roots, tree.root_index[subs]]).astype(np.int64)
-        item_top = np.concatenate([np.ones(N, np.uint8), np.zeros(M, np.uint8)])
+        roots = np.arange(N)
+        # tier 0: families whose parent lies above the first cut, showdown rows down to that cut, per root
+        upper = np.nonzero(has_children[:offs[cuts[0]]])[0]
+        lists_p = [grouped(upper, tree.root_index[upper], roots)]
+        upper_sd = np.nonzero(tree.showdown_mask[:offs[cuts[0] + 1]])[0]
+        lists_s = [grouped(upper_sd, tree.root_index[upper_sd], roots)]
+        item_root, item_top, tiers = [roots], [np.ones(N, np.uint8)], [N]
+        for j, lo in enumerate(cuts):
+            hi = cuts[j + 1] if j + 1 < len(cuts) else n_levels          # parent levels lo .. hi-1
+            anchor = np.full(T, -1, dtype=np.int64)    # the level-`lo` node a deeper row sits under (itself there)
+            anchor[offs[lo]:offs[lo + 1]] = np.arange(offs[lo], offs[lo + 1])
+            for d in range(lo + 1, n_levels):
+                rows = np.arange(offs[d], offs[d + 1])
+                anchor[rows] = anchor[tree.parent_index[rows]]
+            heads = np.nonzero(has_children[offs[lo]:offs[lo + 1]])[0] + offs[lo]        # ascending rows
+            span = np.arange(offs[lo], offs[hi] if hi < n_levels else T)
+            parent_rows = span[has_children[span]]
+            tp, tpo = grouped(parent_rows, anchor[parent_rows], heads)
+            sd_rows = np.arange(offs[lo + 1], offs[hi + 1] if hi < n_levels else T)
+            sd_rows = sd_rows[tree.showdown_mask[sd_rows]]
+            sd_rows = sd_rows[np.isin(anchor[sd_rows], heads)]
+            ts, tso = grouped(sd_rows, anchor[sd_rows], heads)
+            # Largest items first: a launch lasts until its last work item ends, and items are handed to
+            # the compute units in index order, so the long ones must not be the ones that start last.
+            below = np.arange(offs[lo], offs[hi + 1] if hi < n_levels else T)
+            below = below[np.isin(anchor[below], heads)]
+            size = np.bincount(np.searchsorted(heads, anchor[below]), minlength=len(heads))
+            order = np.argsort(-size, kind="stable")
+            lists_p.append(reordered(tp, tpo, order))
+            lists_s.append(reordered(ts, tso, order))
+            heads = heads[order]
+            item_root.append(tree.root_index[heads])
+            item_top.append(np.zeros(len(heads), np.uint8))
+            tiers.append(len(heads))
+
+        def joined(lists):
+            rows = np.concatenate([r for r, _ in lists]).astype(np.int64)
+            offsets, base = [np.zeros(1, np.int64)], 0
+            for _, o in lists:
+                offsets.append(base + o[1:])
+                base += o[-1]
+            return rows, np.concatenate(offsets).astype(np.int64)
+        parents, parent_offsets = joined(lists_p)
+        showdown, showdown_offsets = joined(lists_s)
         _req(len(parents) == int(has_children.sum()) and len(showdown) == int(tree.showdown_mask.sum()),
              "every family and every showdown row must belong to exactly one work item")
         return SimpleNamespace(parents=self._t(parents), parent_offsets=self._t(parent_offsets),
                                showdown=self._t(showdown), showdown_offsets=self._t(showdown_offsets),
-                               item_root=self._t(item_root), item_top=self._t(item_top), n_sub=M, cut=cut)
+                               item_root=self._t(np.concatenate(item_root).astype(np.int64)),
+                               item_top=self._t(np.concatenate(item_top)), tiers=tiers, n_sub=sum(tiers[1:]), cut=cut,
+                               cuts=cuts)
 
     def initialize_subgame(self, src_env, src_indices, initial_beliefs: torch.Tensor | None = None) -> None:
         """cfr_evaluator.py:770-828."""
@@ -749,23 +771,29 @@ class HipSparseCFREvaluator:
         if self._iter_args is None:
             self._iter_args = self._build_iter_args()
             if self._items is not None:
-                # the subtree items alone: the same lists entered behind the N root items
-                sub, N = self._build_iter_args(), self.root_nodes
-                sub.root_parent_offsets += 8 * N
-                sub.root_showdown_offsets += 8 * N
-                sub.item_root += 8 * N
-                sub.item_top += N
-                self._iter_args_sub = sub
+                # one argument block per tier: the same lists entered behind the items of the tiers before
+                self._iter_args_tiers, first = [], 0
+                for count in self._items.tiers:
+                    tier = self._build_iter_args()
+                    tier.root_parent_offsets += 8 * first
+                    tier.root_showdown_offsets += 8 * first
+                    tier.item_root += 8 * first
+                    tier.item_top += first
+                    self._iter_args_tiers.append((tier, count))
+                    first += count
         if self._items is None:
             self._launch_items(self._iter_args, self.root_nodes, phases)
             return
-        N, M = self.root_nodes, self._items.n_sub
+        tiers = self._iter_args_tiers
         if phases & _PHASE_12:
-            self._launch_items(self._iter_args, N + M, _PHASE_1)          # regrets of every family, all items at once
-            self._launch_items(self._iter_args, N, _PHASE_2)              # tree tops, top-down
-        self._launch_items(self._iter_args_sub, M, (_PHASE_2 if phases & _PHASE_12 else 0) | (phases & _PHASE_3))
+            self._launch_items(self._iter_args, sum(self._items.tiers), _PHASE_1)   # regrets of every family, all items at once
+            for args, count in tiers[:-1]:
+                self._launch_items(args, count, _PHASE_2)                           # upper tiers, top-down
+        args, count = tiers[-1]
+        self._launch_items(args, count, (_PHASE_2 if phases & _PHASE_12 else 0) | (phases & _PHASE_3))
         if phases & _PHASE_3:
-            self._launch_items(self._iter_args, N, _PHASE_3)              # the tops' backup comes last
+            for args, count in reversed(tiers[:-1]):
+                self._launch_items(args, count, _PHASE_3)                           # the upper tiers' backup comes last
 
     def cfr_iteration(self, t: int) -> None:
         """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533)."""

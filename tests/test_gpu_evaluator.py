@@ -658,13 +658,14 @@ def test_negative_beta_from_iteration_zero(fused):
     PAR.compare_free(PAR.state_of(ev), twins, factor=FREE_FACTOR_LATER, what="beta = -1, after five iterations: ")
 
 
-@pytest.mark.parametrize("cut", [1, 2, 9])
+@pytest.mark.parametrize("cut,mid", [(1, None), (2, None), (9, None), (2, 1), (9, 1), (9, 3)])
 @pytest.mark.parametrize("seed", range(10))
-def test_split_work_items_give_bit_identical_results(seed, cut, monkeypatch):
+def test_split_work_items_give_bit_identical_results(seed, cut, mid, monkeypatch):
     """With few roots the iteration kernel gives every root several workgroups: the tree is cut at a
     level (1: right under the root; 2: the default; 9: as deep as families go), the top of each tree
     is one work item, every subtree under the cut another, and an iteration takes four launches
-    instead of one.  Every family still goes through the same arithmetic, so all eleven state
+    instead of one; with a second cut above the first (`mid`: 1 is the default for few roots) the tops
+    are cut again and it takes six.  Every family still goes through the same arithmetic, so all eleven state
     tensors must be bit-identical to the one-workgroup-per-root launch — over random trees, CFR variants, mid-round roots, a sampling
     iteration, river and (odd seeds) turn roots; depth-limit and street-end leaves get their values
     from a leaf model between the two halves of an iteration."""
@@ -674,6 +675,7 @@ def test_split_work_items_give_bit_identical_results(seed, cut, monkeypatch):
     from poker2_amd.tree import RootStates
     import poker2_amd.evaluator as evaluator_module
     monkeypatch.setattr(evaluator_module, "SPLIT_CUT_LEVEL", cut)
+    monkeypatch.setattr(evaluator_module, "SPLIT_MID_LEVEL", mid)
     rng = np.random.default_rng(7000 + seed)
     n = int(rng.integers(1, 7))
     bins = sorted(rng.choice([0.25, 0.5, 0.75, 1.0, 2.0], size=int(rng.integers(1, 5)), replace=False).tolist())
@@ -709,6 +711,7 @@ def test_split_work_items_give_bit_identical_results(seed, cut, monkeypatch):
         return ev
     a, b = run(True), run(False)
     assert a._items.n_sub > 0 and 1 <= a._items.cut <= cut
+    assert len(a._items.tiers) == (3 if mid is not None and mid < a._items.cut else 2)
     for name in OCFR.OracleCFR.STATE_NAMES:
         assert torch.equal(getattr(a, name), getattr(b, name)), \
             f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type} street {street}: {name}"
