@@ -192,6 +192,7 @@ class HipSparseCFREvaluator:
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_args = None
         self._iter_args_tiers = None
+        self._iter_args_regret = None
         self._chance_helper = None
         self.subgame_serial = 0
 
@@ -323,10 +324,15 @@ class HipSparseCFREvaluator:
         self._has_model_leaves = bool(model_mask.any())
         self._iter_args = None
         self._iter_args_tiers = None
+        self._iter_args_regret = None
         split = self.split_small_batches
         if split is None:
             split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
         self._items = self._split_items(tree, SPLIT_MID_LEVEL if N < SPLIT_ROOTS_BELOW else None) if split else None
+        # The regret part has no order among families: it runs over the coarser of the two partitions
+        # (whole tree tops), which makes fewer and longer workgroups of the same work.
+        self._items_regret = (self._split_items(tree) if self._items is not None and len(self._items.tiers) > 2
+                              else self._items)
         self._root_items = None
         if self._items is None and T:
             # Roots of unequal size (mixed streets, stacks, pots): one work item per root, largest tree
@@ -736,7 +742,7 @@ class HipSparseCFREvaluator:
             self.latest_values[self.showdown_indices] = self._showdown_value_both(beliefs[self.showdown_indices])
 
     # ------------------------------------------------------------------ iteration
-    def _build_iter_args(self) -> _IterArgs:
+    def _build_iter_args(self, items=None) -> _IterArgs:
         a = _IterArgs()
         p = _lib.ptr
         a.child_offsets, a.child_count, a.to_act = p(self.child_offsets), p(self.child_count), p(self.env.to_act)
@@ -752,7 +758,7 @@ class HipSparseCFREvaluator:
         a.reach, a.reach_avg = p(self.self_reach), p(self.self_reach_avg)
         a.latest, a.values_avg, a.scratch = p(self.latest_values), p(self.values_avg), p(self._scratch)
         a.fscal, a.iscal = p(self._fscal), p(self._iscal)
-        it = self._items if self._items is not None else self._root_items
+        it = items if items is not None else (self._items if self._items is not None else self._root_items)
         if it is not None:
             a.root_parent_offsets, a.root_parents = p(it.parent_offsets), p(it.parents)
             a.root_showdown_offsets, a.root_showdown_nodes = p(it.showdown_offsets), p(it.showdown)
@@ -771,6 +777,7 @@ class HipSparseCFREvaluator:
         if self._iter_args is None:
             self._iter_args = self._build_iter_args()
             if self._items is not None:
+                self._iter_args_regret = (self._build_iter_args(self._items_regret), sum(self._items_regret.tiers))
                 # one argument block per tier: the same lists entered behind the items of the tiers before
                 self._iter_args_tiers, first = [], 0
                 for count in self._items.tiers:
@@ -786,7 +793,7 @@ class HipSparseCFREvaluator:
             return
         tiers = self._iter_args_tiers
         if phases & _PHASE_12:
-            self._launch_items(self._iter_args, sum(self._items.tiers), _PHASE_1)   # regrets of every family, all items at once
+            self._launch_items(*self._iter_args_regret, _PHASE_1)                 # regrets of every family, all items at once
             for args, count in tiers[:-1]:
                 self._launch_items(args, count, _PHASE_2)                           # upper tiers, top-down
         args, count = tiers[-1]
