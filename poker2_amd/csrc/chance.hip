@@ -535,7 +535,7 @@ __global__ __launch_bounds__(CH_BLOCK) void perm_mean_kernel(const float* __rest
                                                               const float* __restrict__ weight, int64_t n_flops,
                                                               int64_t flops_per_share, int accumulate,
                                                               float* __restrict__ dst, int64_t dst_share_stride) {
-  extern __shared__ __align__(8) unsigned char lds_raw[];
+  extern __shared__ __align__(16) unsigned char lds_raw[];
   float* rows = reinterpret_cast<float*>(lds_raw);                                  // [2][H + 2]
   uint32_t* ptab = reinterpret_cast<uint32_t*>(lds_raw + 2 * (P2_H + 2) * 4);       // [n_perms][HPAIRS]
   const int64_t i = blockIdx.x >> 1;
@@ -561,6 +561,66 @@ __global__ __launch_bounds__(CH_BLOCK) void perm_mean_kernel(const float* __rest
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) acc[k][0] = acc[k][1] = 0.0;
   const float inv_perms = 1.0f / (float)n_perms;
+  if (in_regs) {
+    // Two rows per step, interleaved hand by hand in LDS: one 64-bit gather serves both rows (the gathers
+    // keep the LDS pipe busy most of the time; this halves their number) and six row pieces are in flight
+    // per lane instead of three.  A share with an odd number of rows repeats its last row with weight 0.
+    float2* pairs = reinterpret_cast<float2*>(lds_raw);            // [2][H + 2] of (row f, row f + 1)
+    float2 na[CH_PPT], nb[CH_PPT];
+    auto fetch2 = [&](int64_t f) {
+      const float2* a = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
+      const float2* b = p2_row2(hand_values, ((int64_t)i * n_flops + (f + 1 < f1 ? f + 1 : f)) * 2 + p);
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) {
+        const int idx = threadIdx.x + k * CH_BLOCK;
+        na[k] = a[idx < P2_HPAIRS ? idx : 0];
+        nb[k] = b[idx < P2_HPAIRS ? idx : 0];
+      }
+    };
+    if (f0 < f1) fetch2(f0);
+    int buf = 0;
+    for (int64_t f = f0; f < f1; f += 2, buf ^= 1) {
+      float2* row = pairs + buf * (P2_H + 2);
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) {
+        const int idx = threadIdx.x + k * CH_BLOCK;
+        if (idx < P2_HPAIRS)
+          reinterpret_cast<float4*>(row)[idx] = make_float4(na[k].x, nb[k].x, na[k].y, nb[k].y);
+      }
+      if (f + 2 < f1) fetch2(f + 2);
+      p2_sync_lds();   // rows f, f+1 are complete; the other buffer was consumed before this barrier
+      const float wa = weight[f] * inv_perms;
+      const float wb = f + 1 < f1 ? weight[f + 1] * inv_perms : 0.f;
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) {
+        const int idx = threadIdx.x + k * CH_BLOCK;
+        if (idx >= P2_HPAIRS) continue;
+        float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
+#pragma unroll
+        for (int q = 0; q < CH_REG_PERMS; ++q)
+          if (q < n_perms) {
+            const float2 u = row[preg[q][k] & 0xFFFFu], v = row[preg[q][k] >> 16];
+            a0 += u.x; b0 += u.y;
+            a1 += v.x; b1 += v.y;
+          }
+        acc[k][0] += (double)(wa * a0);
+        acc[k][1] += (double)(wa * a1);
+        if (f + 1 < f1) {
+          acc[k][0] += (double)(wb * b0);
+          acc[k][1] += (double)(wb * b1);
+        }
+      }
+    }
+    float2* o = p2_row2(dst + (int64_t)blockIdx.y * dst_share_stride, i * 2 + p);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      if (idx >= P2_HPAIRS) continue;
+      const float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
+      o[idx] = make_float2(prev.x + (float)acc[k][0], prev.y + (float)acc[k][1]);
+    }
+    return;
+  }
   float2 next[CH_PPT];
   auto fetch = [&](int64_t f) {
     const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
@@ -800,8 +860,8 @@ int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const 
   if (((uintptr_t)perms & 3) != 0) return P2_EINVAL;
   if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
   if (shares > 1 && (!workspace || !p2_aligned8(workspace))) return P2_EINVAL;
-  const size_t lds = (size_t)2 * (P2_H + 2) * 4 +
-                     (n_perms > p2::CH_REG_PERMS ? (size_t)n_perms * P2_HPAIRS * 4 : 0);   // 10.6 KB, or 74 KB with all 24
+  const size_t lds = n_perms > p2::CH_REG_PERMS ? (size_t)2 * (P2_H + 2) * 4 + (size_t)n_perms * P2_HPAIRS * 4
+                                                : (size_t)2 * (P2_H + 2) * 8;   // 74 KB with all 24, or 21 KB
   if (lds > 64 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(p2::perm_mean_kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
