@@ -302,26 +302,51 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
   }
 }
 
-// expected[i][p][h] = mean over the samples of state i.  blockIdx.y picks a run of 256 hand pairs,
-// so a lane carries one pair of each player through all samples of its state.
+// expected[i][p][h] = mean over the samples of state i.  blockIdx.y picks the player: a workgroup walks the
+// whole 5304-byte rows of one player through all samples of its state (three pairs per lane), four
+// samples' rows in flight at a time.
 __global__ __launch_bounds__(CH_BLOCK) void chance_mean_kernel(const float* __restrict__ hand_values,
                                                                 const int64_t* __restrict__ sample_offsets,
                                                                 float* __restrict__ expected) {
   const int64_t i = blockIdx.x;
-  const int idx = blockIdx.y * CH_BLOCK + threadIdx.x;
-  if (idx >= P2_HPAIRS) return;
+  const int p = blockIdx.y;
   const int64_t s0 = sample_offsets[i], s1 = sample_offsets[i + 1];
-  float2 acc0 = make_float2(0.f, 0.f), acc1 = make_float2(0.f, 0.f);
-#pragma unroll 4
-  for (int64_t s = s0; s < s1; ++s) {
-    const float2 x = p2_row2(hand_values, s * 2)[idx];
-    const float2 y = p2_row2(hand_values, s * 2 + 1)[idx];
-    acc0.x += x.x; acc0.y += x.y;
-    acc1.x += y.x; acc1.y += y.y;
+  float2 acc[CH_PPT];
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) acc[k] = make_float2(0.f, 0.f);
+  int64_t s = s0;
+  for (; s + 4 <= s1; s += 4) {
+    float2 x[4][CH_PPT];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float2* row = p2_row2(hand_values, (s + j) * 2 + p);
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) {
+        const int idx = threadIdx.x + k * CH_BLOCK;
+        x[j][k] = row[idx < P2_HPAIRS ? idx : 0];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) { acc[k].x += x[j][k].x; acc[k].y += x[j][k].y; }
+  }
+  for (; s < s1; ++s) {
+    const float2* row = p2_row2(hand_values, s * 2 + p);
+#pragma unroll
+    for (int k = 0; k < CH_PPT; ++k) {
+      const int idx = threadIdx.x + k * CH_BLOCK;
+      const float2 v = row[idx < P2_HPAIRS ? idx : 0];
+      acc[k].x += v.x; acc[k].y += v.y;
+    }
   }
   const float count = fmaxf((float)(s1 - s0), 1.0f);
-  p2_row2(expected, i * 2)[idx] = make_float2(acc0.x / count, acc0.y / count);
-  p2_row2(expected, i * 2 + 1)[idx] = make_float2(acc1.x / count, acc1.y / count);
+  float2* o = p2_row2(expected, i * 2 + p);
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    if (idx < P2_HPAIRS) o[idx] = make_float2(acc[k].x / count, acc[k].y / count);
+  }
 }
 
 // ---- three-card (flop) chance node ------------------------------------------------------
@@ -815,7 +840,7 @@ int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, i
   if (n == 0) return 0;
   if (!hand_values || !sample_offsets || !expected) return P2_EINVAL;
   if (!p2_aligned8(hand_values) || !p2_aligned8(expected)) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)n, p2::CH_PPT), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+  hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)n, 2), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
                      hand_values, sample_offsets, expected);
   P2_LAUNCH_CHECK();
   return 0;
