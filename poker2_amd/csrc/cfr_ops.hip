@@ -237,17 +237,44 @@ __global__ __launch_bounds__(OPS_BLOCK) void parent_sum_kernel(const float* __re
   const int64_t p = blockIdx.x;
   const int64_t first = child_offsets[p];
   const int count = (int)child_count[p];
-  P2_ROW_LOOP(i) {
-    float2 acc = make_float2(0.f, 0.f);
-    for (int k = 0; k < count; ++k) {
-      const float2 v = p2_row2(values, first + k)[i];
-      acc.x += v.x;
-      acc.y += v.y;
+  // a lane's three pairs of every child row; the rows of two children are requested before either is added
+  // (children are still added in ascending order)
+  float2 acc[OPS_PAIRS_PER_THREAD];
+#pragma unroll
+  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) acc[j] = make_float2(0.f, 0.f);
+  auto fetch = [&](int k, float2 (&v)[OPS_PAIRS_PER_THREAD]) {
+    const float2* row = p2_row2(values, first + k);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      v[j] = row[i < P2_HPAIRS ? i : 0];
     }
+  };
+  int k = 0;
+  for (; k + 2 <= count; k += 2) {
+    float2 a[OPS_PAIRS_PER_THREAD], b[OPS_PAIRS_PER_THREAD];
+    fetch(k, a);
+    fetch(k + 1, b);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      acc[j].x += a[j].x; acc[j].y += a[j].y;
+      acc[j].x += b[j].x; acc[j].y += b[j].y;
+    }
+  }
+  if (k < count) {
+    float2 a[OPS_PAIRS_PER_THREAD];
+    fetch(k, a);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) { acc[j].x += a[j].x; acc[j].y += a[j].y; }
+  }
+#pragma unroll
+  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+    const int i = threadIdx.x + j * OPS_BLOCK;
+    if (i >= P2_HPAIRS) continue;
     if (broadcast) {
-      for (int k = 0; k < count; ++k) p2_row2(out, first + k - out_offset)[i] = acc;
+      for (int c = 0; c < count; ++c) p2_row2(out, first + c - out_offset)[i] = acc[j];
     } else {
-      p2_row2(out, p)[i] = acc;
+      p2_row2(out, p)[i] = acc[j];
     }
   }
 }
