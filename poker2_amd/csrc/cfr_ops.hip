@@ -362,17 +362,44 @@ __global__ __launch_bounds__(OPS_BLOCK) void weighted_parent_sum_kernel(
   const int count = (int)child_count[p];
   if (count == 0) return;  // leaf at an intermediate depth keeps its value
   float2* o2 = p2_row2(values, (parent_base + p) * 2 + player);
-  P2_ROW_LOOP(i) {
-    float2 acc = make_float2(0.f, 0.f);
-    for (int k = 0; k < count; ++k) {
-      const int64_t child = first + k;
-      const float* pol = (prev_actor[child] == (int64_t)player) ? pol_hero : pol_opp;
-      const float2 w = p2_row2(pol, child)[i];
-      const float2 v = p2_row2(values, child * 2 + player)[i];
-      acc.x += v.x * w.x;
-      acc.y += v.y * w.y;
+  // a lane's three pairs of every child; value and policy rows of two children are requested before
+  // either is used (children are still added in ascending order)
+  float2 acc[OPS_PAIRS_PER_THREAD];
+#pragma unroll
+  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) acc[j] = make_float2(0.f, 0.f);
+  auto fetch = [&](int k, float2 (&v)[OPS_PAIRS_PER_THREAD], float2 (&w)[OPS_PAIRS_PER_THREAD]) {
+    const int64_t child = first + k;
+    const float* pol = (prev_actor[child] == (int64_t)player) ? pol_hero : pol_opp;
+    const float2* wr = p2_row2(pol, child);
+    const float2* vr = p2_row2(values, child * 2 + player);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      w[j] = wr[i < P2_HPAIRS ? i : 0];
+      v[j] = vr[i < P2_HPAIRS ? i : 0];
     }
-    o2[i] = acc;
+  };
+  int k = 0;
+  for (; k + 2 <= count; k += 2) {
+    float2 va[OPS_PAIRS_PER_THREAD], wa[OPS_PAIRS_PER_THREAD], vb[OPS_PAIRS_PER_THREAD], wb[OPS_PAIRS_PER_THREAD];
+    fetch(k, va, wa);
+    fetch(k + 1, vb, wb);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      acc[j].x += va[j].x * wa[j].x; acc[j].y += va[j].y * wa[j].y;
+      acc[j].x += vb[j].x * wb[j].x; acc[j].y += vb[j].y * wb[j].y;
+    }
+  }
+  if (k < count) {
+    float2 va[OPS_PAIRS_PER_THREAD], wa[OPS_PAIRS_PER_THREAD];
+    fetch(k, va, wa);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) { acc[j].x += va[j].x * wa[j].x; acc[j].y += va[j].y * wa[j].y; }
+  }
+#pragma unroll
+  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+    const int i = threadIdx.x + j * OPS_BLOCK;
+    if (i < P2_HPAIRS) o2[i] = acc[j];
   }
 }
 
