@@ -19,6 +19,7 @@ call remain.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from types import SimpleNamespace
 
 import numpy as np
 from ._guards import require as _req
@@ -336,6 +337,87 @@ def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
                       legal_mask=legal, leaf_mask=leaf, new_street_mask=new_street,
                       fold_mask=(action == 0) & state["done"], showdown_mask=state["street"] == 4,
                       reward=reward, state=state, board=np.array(roots.board))
+
+
+def split_work_items(tree: "SparseTree", n_roots: int, cut_level: int, mid_level: int | None = None):
+    """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h), in
+    tiers: tier 0 holds one item per root, the top of its tree above the first cut level; every further
+    tier one item per node of its cut level that has children, with the families from that level down
+    to the next cut level (the last tier: to the leaves).  Cut levels: ``mid_level`` (optional, must lie
+    above the main one) and ``cut_level``.  Returns numpy arrays over all items in tier order (family
+    rows + offsets, showdown rows + offsets, item_root, item_top) and the tiers' item counts; None if
+    the tree is too shallow to cut."""
+    N, T = n_roots, tree.total
+    offs = tree.depth_offsets
+    n_levels = len(offs) - 1
+    has_children = tree.child_count > 0
+    cut = min(cut_level, n_levels - 2)
+    while cut >= 1 and not has_children[offs[cut]:offs[cut + 1]].any():
+        cut -= 1                                            # the deepest level that still has families below it
+    if cut < 1:
+        return None
+    cuts = [cut] if mid_level is None or not 1 <= mid_level < cut else [mid_level, cut]
+
+    def grouped(rows, keys, groups):
+        """rows ordered by group (ascending inside a group) and offsets [len(groups) + 1]."""
+        slot = np.searchsorted(groups, keys)
+        order = np.argsort(slot, kind="stable")
+        counts = np.bincount(slot, minlength=len(groups))
+        return rows[order], np.concatenate([[0], np.cumsum(counts)])
+
+    def reordered(rows, offsets, order):
+        pieces = [rows[offsets[g]:offsets[g + 1]] for g in order]
+        lengths = np.array([len(x) for x in pieces], dtype=np.int64)
+        return (np.concatenate(pieces) if pieces else rows), np.concatenate([[0], np.cumsum(lengths)])
+    roots = np.arange(N)
+    # tier 0: families whose parent lies above the first cut, showdown rows down to that cut, per root
+    upper = np.nonzero(has_children[:offs[cuts[0]]])[0]
+    lists_p = [grouped(upper, tree.root_index[upper], roots)]
+    upper_sd = np.nonzero(tree.showdown_mask[:offs[cuts[0] + 1]])[0]
+    lists_s = [grouped(upper_sd, tree.root_index[upper_sd], roots)]
+    item_root, item_top, tiers = [roots], [np.ones(N, np.uint8)], [N]
+    for j, lo in enumerate(cuts):
+        hi = cuts[j + 1] if j + 1 < len(cuts) else n_levels          # parent levels lo .. hi-1
+        anchor = np.full(T, -1, dtype=np.int64)    # the level-`lo` node a deeper row sits under (itself there)
+        anchor[offs[lo]:offs[lo + 1]] = np.arange(offs[lo], offs[lo + 1])
+        for d in range(lo + 1, n_levels):
+            rows = np.arange(offs[d], offs[d + 1])
+            anchor[rows] = anchor[tree.parent_index[rows]]
+        heads = np.nonzero(has_children[offs[lo]:offs[lo + 1]])[0] + offs[lo]        # ascending rows
+        span = np.arange(offs[lo], offs[hi] if hi < n_levels else T)
+        parent_rows = span[has_children[span]]
+        tp, tpo = grouped(parent_rows, anchor[parent_rows], heads)
+        sd_rows = np.arange(offs[lo + 1], offs[hi + 1] if hi < n_levels else T)
+        sd_rows = sd_rows[tree.showdown_mask[sd_rows]]
+        sd_rows = sd_rows[np.isin(anchor[sd_rows], heads)]
+        ts, tso = grouped(sd_rows, anchor[sd_rows], heads)
+        # Largest items first: a launch lasts until its last work item ends, and items are handed to
+        # the compute units in index order, so the long ones must not be the ones that start last.
+        below = np.arange(offs[lo], offs[hi + 1] if hi < n_levels else T)
+        below = below[np.isin(anchor[below], heads)]
+        size = np.bincount(np.searchsorted(heads, anchor[below]), minlength=len(heads))
+        order = np.argsort(-size, kind="stable")
+        lists_p.append(reordered(tp, tpo, order))
+        lists_s.append(reordered(ts, tso, order))
+        heads = heads[order]
+        item_root.append(tree.root_index[heads])
+        item_top.append(np.zeros(len(heads), np.uint8))
+        tiers.append(len(heads))
+
+    def joined(lists):
+        rows = np.concatenate([r for r, _ in lists]).astype(np.int64)
+        offsets, base = [np.zeros(1, np.int64)], 0
+        for _, o in lists:
+            offsets.append(base + o[1:])
+            base += o[-1]
+        return rows, np.concatenate(offsets).astype(np.int64)
+    parents, parent_offsets = joined(lists_p)
+    showdown, showdown_offsets = joined(lists_s)
+    _req(len(parents) == int(has_children.sum()) and len(showdown) == int(tree.showdown_mask.sum()),
+         "every family and every showdown row must belong to exactly one work item")
+    return SimpleNamespace(parents=parents, parent_offsets=parent_offsets, showdown=showdown,
+                           showdown_offsets=showdown_offsets, item_root=np.concatenate(item_root).astype(np.int64),
+                           item_top=np.concatenate(item_top), tiers=tiers, n_sub=sum(tiers[1:]), cut=cut, cuts=cuts)
 
 
 # ---------------------------------------------------------------------------------------------

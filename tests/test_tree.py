@@ -114,3 +114,63 @@ def test_roots_of_the_flop_showdown_variant_are_refused():
     env = types.SimpleNamespace(flop_showdown=True)
     with pytest.raises(NotImplementedError):
         RootStates.from_env(env, np.arange(1))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_work_items_partition_the_tree(seed):
+    """split_work_items on random trees and cut levels: every family and every showdown row belongs to
+    exactly one item; an item's rows lie under its head (tier 0: under its root) and inside its tier's
+    levels; a showdown row sits in the item that owns its parent's family; inside a tier the items come
+    largest first; the tiers' counts add up."""
+    from poker2_amd.tree import split_work_items
+    rng = np.random.default_rng(900 + seed)
+    n = int(rng.integers(1, 6))
+    street = int(rng.integers(1, 4))
+    bins = sorted(rng.choice([0.25, 0.5, 1.0, 2.0], size=int(rng.integers(1, 4)), replace=False).tolist())
+    roots = RootStates.at_round_start(street, rng.integers(40, 900, n), rng.integers(30, 2500, (n, 2)),
+                                      np.full((n, 5), -1), button=rng.integers(0, 2, n), bb=int(rng.choice([10, 100])))
+    tree = build_sparse_tree(roots, bins, int(rng.integers(2, 7)), max_raises=[None, 2, 3][seed % 3])
+    offs = np.asarray(tree.depth_offsets)
+    level = np.searchsorted(offs, np.arange(tree.total), side="right") - 1
+    has_children = tree.child_count > 0
+    for cut, mid in ((1, None), (2, None), (2, 1), (9, None), (9, 1), (9, 2)):
+        it = split_work_items(tree, n, cut, mid)
+        if it is None:
+            assert len(offs) - 1 < 3 or not has_children[offs[1]:].any()
+            continue
+        assert sum(it.tiers) == len(it.item_root) == len(it.item_top) == len(it.parent_offsets) - 1
+        assert it.tiers[0] == n and (it.item_top[:n] == 1).all() and (it.item_top[n:] == 0).all()
+        assert len(it.tiers) == 1 + len(it.cuts) and it.n_sub == sum(it.tiers[1:])
+        assert np.array_equal(np.sort(it.parents), np.nonzero(has_children)[0])            # each family once
+        assert np.array_equal(np.sort(it.showdown), np.nonzero(tree.showdown_mask)[0])     # each showdown row once
+        owner = np.full(tree.total, -1)
+        bounds = [0] + list(it.cuts) + [len(offs) - 1]
+        first_item = np.concatenate([[0], np.cumsum(it.tiers)])
+        for tier in range(len(it.tiers)):
+            for w in range(first_item[tier], first_item[tier + 1]):
+                rows = it.parents[it.parent_offsets[w]:it.parent_offsets[w + 1]]
+                assert (np.diff(rows) > 0).all()                                           # ascending: top-down order
+                assert ((level[rows] >= bounds[tier]) & (level[rows] < bounds[tier + 1])).all()
+                assert (tree.root_index[rows] == it.item_root[w]).all()
+                if tier > 0:                                                               # one head per item, at the cut
+                    heads = rows[level[rows] == bounds[tier]]
+                    assert len(heads) == 1
+                    up = rows.copy()
+                    while (level[up] > bounds[tier]).any():
+                        deeper = level[up] > bounds[tier]
+                        up[deeper] = tree.parent_index[up[deeper]]
+                    assert (up == heads[0]).all()
+                owner[rows] = w
+            if tier > 0:                       # largest first, by the rows from the head down to the next cut
+                hi_level = min(bounds[tier + 1], len(offs) - 2)
+                below = np.arange(offs[bounds[tier]], offs[hi_level + 1])
+                top = below.copy()
+                while (level[top] > bounds[tier]).any():
+                    deeper = level[top] > bounds[tier]
+                    top[deeper] = tree.parent_index[top[deeper]]
+                head_of = [it.parents[it.parent_offsets[w]] for w in range(first_item[tier], first_item[tier + 1])]
+                rows_under = [int((top == h).sum()) for h in head_of]
+                assert all(a >= b for a, b in zip(rows_under, rows_under[1:]))
+        for w in range(len(it.item_root)):
+            sd = it.showdown[it.showdown_offsets[w]:it.showdown_offsets[w + 1]]
+            assert (owner[tree.parent_index[sd]] == w).all()                               # with its parent's family
