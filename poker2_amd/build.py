@@ -27,8 +27,16 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found; libp2hip.so cannot be built")
 
 
-def build_library(verbose: bool = False) -> str:
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", LIB_PATH, os.path.join(CSRC, "p2hip.hip")]
+SWEEP_TIMER_LIB_PATH = os.path.join(PKG_DIR, "libp2hip_sweep_timers.so")
+
+
+def build_library(verbose: bool = False, sweep_timers: bool = False) -> str:
+    """The library; with ``sweep_timers`` a second one, beside it, whose iteration kernel also adds up the
+    clock ticks each workgroup spends in each of its sweeps (a tuning build: ``poker2_amd.bench_sweeps``
+    reads them; the product never loads it)."""
+    out = SWEEP_TIMER_LIB_PATH if sweep_timers else LIB_PATH
+    extra = ["-DP2_ITER_PROFILE"] if sweep_timers else []
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra, "-o", out, os.path.join(CSRC, "p2hip.hip")]
     res = subprocess.run(cmd, cwd=CSRC, capture_output=True, text=True)
     if verbose or res.returncode != 0:
         print(" ".join(cmd))
@@ -36,8 +44,9 @@ def build_library(verbose: bool = False) -> str:
         print(res.stderr)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed with exit code {res.returncode}")
-    return LIB_PATH
+    return out
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    import sys
+    print(build_library(verbose=True, sweep_timers="--sweep-timers" in sys.argv[1:]))

@@ -116,7 +116,8 @@ struct IterLds {
 __device__ long long g_iter_prof[8192][8];
 #define PROF_BEGIN(var) const long long var = wall_clock64()
 #define PROF_END(slot, var) \
-  do { if (threadIdx.x == 0) g_iter_prof[blockIdx.x & 8191][slot] += wall_clock64() - (var); } while (0)
+  do { if (threadIdx.x == 0) atomicAdd((unsigned long long*)&g_iter_prof[blockIdx.x & 8191][slot], \
+                                       (unsigned long long)(wall_clock64() - (var))); } while (0)
 #else
 #define PROF_BEGIN(var)
 #define PROF_END(slot, var)
