@@ -325,6 +325,48 @@ def test_unblocked_mass_grid_stride_ragged_and_empty(F):
     assert F.unblocked_mass_ratio_triton(empty, empty).shape == (0, H)
 
 
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 7, 1030])
+def test_unblocked_mass_at_every_buffer_alignment_and_ragged_row_counts(rows):
+    """Through the C ABI with buffers at several offsets inside a 128-byte line (8-byte alignment is all the
+    entry points ask for): the oracle's values, nothing written outside the output rows, bit-identical
+    results whatever the alignment, for row counts that leave the last group of four rows ragged, and
+    for rows picked by player."""
+    from poker2_amd import _lib
+    rng = np.random.default_rng(600 + rows)
+    t = rng.random((rows, H)).astype(np.float32)
+    t[rows // 2, ::3] = 0.0
+    exp = OU.calculate_unblocked_mass(t)
+    stream = _lib.stream_ptr()
+    results = []
+    for offset in (0, 2, 4, 8, 12, 28):               # in floats
+        src = torch.zeros(rows * H + 64, device="cuda")
+        dst = torch.full((rows * H + 64,), -7.0, device="cuda")
+        a, b = src[offset:offset + rows * H], dst[offset:offset + rows * H]
+        a.copy_(torch.from_numpy(t).reshape(-1))
+        _lib.call("p2hip_unblocked_mass", a.data_ptr(), rows, b.data_ptr(), stream)
+        torch.cuda.synchronize()
+        assert (dst[:offset] == -7.0).all() and (dst[offset + rows * H:] == -7.0).all()   # nothing outside
+        results.append(b.reshape(rows, H).cpu().numpy())
+        close(b.reshape(rows, H), exp, rtol=1e-6, atol=1e-5)
+    for r in results[1:]:
+        assert np.array_equal(r, results[0])
+    # by player: rows 2 r + (to_act[r] ^ flip) of a [rows, 2, H] tensor
+    bel = rng.random((rows, 2, H)).astype(np.float32)
+    to_act = rng.integers(0, 2, rows).astype(np.int64)
+    exp2 = OU.calculate_unblocked_mass(bel[np.arange(rows), 1 - to_act])
+    got = []
+    for offset in (0, 2):
+        dst = torch.full((rows * H + 64,), -7.0, device="cuda")
+        b = dst[offset:offset + rows * H]
+        _lib.call("p2hip_unblocked_mass_by_player", dev(bel).data_ptr(), dev(to_act).data_ptr(), rows, 1,
+                  b.data_ptr(), stream)
+        torch.cuda.synchronize()
+        assert (dst[:offset] == -7.0).all() and (dst[offset + rows * H:] == -7.0).all()
+        got.append(b.reshape(rows, H).cpu().numpy())
+        close(b.reshape(rows, H), exp2, rtol=1e-6, atol=1e-5)
+    assert np.array_equal(got[0], got[1])
+
+
 def test_wrappers_refuse_arguments_that_would_index_out_of_bounds(F):
     """Sizes, dtypes and row bounds the kernels index with are checked on the host (and stay
     checked under ``python -O``): none of these calls may reach the GPU."""
