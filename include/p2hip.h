@@ -181,14 +181,16 @@ int p2hip_policy_targets(const float* policy_avg, const int64_t* rows, int64_t n
 
 /* One tree level of _best_response_values (search/cfr_evaluator.py:636-714), in place on
  * values [total,2,H]: for the parents parent_base .. parent_base+num_parents-1 that have
- * children (rows child_offsets[p] .. +child_count[p], at most 8), the player to act takes the
+ * children (rows child_offsets[p] .. +child_count[p], at most max_children <= 8: a parent with more
+ * is skipped), the player to act takes the
  * per-hand maximum over children where deviating_player[p] == to_act[p] and the policy-weighted
  * mean elsewhere; the other player gets the expectation of its child values under the
  * blocker-projected action probabilities.  Rows without children are left as they are (leaf
  * values).  Call once per level, deepest parents first.  All index arrays are [total] int64. */
 int p2hip_best_response_level(float* values, const float* policy, const float* beliefs, const int64_t* to_act,
                               const int64_t* deviating_player, const int64_t* child_offsets,
-                              const int64_t* child_count, int64_t parent_base, int64_t num_parents, void* stream);
+                              const int64_t* child_count, int64_t parent_base, int64_t num_parents,
+                              int max_children, void* stream);
 
 /* ---- betting tree on the device ----------------------------------------------------------- */
 

@@ -33,7 +33,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_showdown_setup": [_P, _I, _L, _I, _P, _P, _P, _P],
     "p2hip_showdown_setup_sorted": [_P, _P, _P, _P, _L, _P, _P, _P],
     "p2hip_showdown_both": [_P, _P, _P, _P, _P, _L, _P, _P],
-    "p2hip_best_response_level": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _P],
+    "p2hip_best_response_level": [_P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _P],
     "p2hip_upload_floats": [_P, _P, _I, _P],
     "p2hip_tree_node_columns": [],
     "p2hip_tree_legal": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _P],

@@ -182,7 +182,8 @@ def cases(repeats: int):
     yield (f"best_response_level parents={n_par}", (3 * n_par + 3 * n_ch) * H * 4,
            lambda: _lib.call("p2hip_best_response_level", _lib.ptr(vals), _lib.ptr(ev.policy_probs_avg),
                              _lib.ptr(ev.beliefs), _lib.ptr(ev.env.to_act), _lib.ptr(deviator),
-                             _lib.ptr(ev.child_offsets), _lib.ptr(ev.child_count), base, n_par, _lib.stream_ptr()))
+                             _lib.ptr(ev.child_offsets), _lib.ptr(ev.child_count), base, n_par,
+                             int(ev._max_children), _lib.stream_ptr()))
 
 
 def main() -> None:

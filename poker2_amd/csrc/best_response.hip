@@ -11,7 +11,8 @@
 // which covers the reference's four cases (:690-703) because the opponent-conditioned policy
 // of the ordinary backup is the same ratio with w_c = policy[c].  Rows without children keep
 // the leaf values the caller put there.  One workgroup per parent; the weighted beliefs of all
-// children and b_a are card-summed in one pass.
+// children and b_a are card-summed in one pass.  The kernel is compiled for at most five and at most
+// eight children per parent: 34 KB of LDS (four workgroups per CU) against 51 KB (three).
 #pragma once
 #include "common.h"
 #include "unblocked.hip"
@@ -25,15 +26,16 @@ constexpr int BR_GRP = 4;   // children whose rows are in flight together
 constexpr int BR_STRIDE = P2_H + 2;
 static_assert(BR_BLOCK == UB_BLOCK, "card_sums_multi assumes the block size");
 
+template <int MAXC>
 __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
     float* __restrict__ values, const float* __restrict__ policy, const float* __restrict__ beliefs,
     const int64_t* __restrict__ to_act, const int64_t* __restrict__ deviating_player,
     const int64_t* __restrict__ child_offsets, const int64_t* __restrict__ child_count, int64_t parent_base) {
-  __shared__ __align__(8) float t[BR_MAXC + 1][BR_STRIDE];
-  __shared__ double cs[(BR_MAXC + 1) * P2_CARDS];
+  __shared__ __align__(8) float t[MAXC + 1][BR_STRIDE];
+  __shared__ double cs[(MAXC + 1) * P2_CARDS];
   const int64_t p = parent_base + blockIdx.x;
   const int nc = (int)child_count[p];
-  if (nc <= 0 || nc > BR_MAXC) return;
+  if (nc <= 0 || nc > MAXC) return;
   const int64_t c0 = child_offsets[p];
   const int actor = (int)to_act[p];
   const bool is_dev = (int)deviating_player[p] == actor;
@@ -168,14 +170,20 @@ extern "C" {
 
 int p2hip_best_response_level(float* values, const float* policy, const float* beliefs, const int64_t* to_act,
                               const int64_t* deviating_player, const int64_t* child_offsets,
-                              const int64_t* child_count, int64_t parent_base, int64_t num_parents, void* stream) {
-  if (num_parents < 0 || parent_base < 0) return P2_EINVAL;
+                              const int64_t* child_count, int64_t parent_base, int64_t num_parents,
+                              int max_children, void* stream) {
+  if (num_parents < 0 || parent_base < 0 || max_children < 1 || max_children > p2::BR_MAXC) return P2_EINVAL;
   if (num_parents == 0) return 0;
   if (!values || !policy || !beliefs || !to_act || !deviating_player || !child_offsets || !child_count) return P2_EINVAL;
   if (!p2_aligned8(values) || !p2_aligned8(policy) || !p2_aligned8(beliefs)) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::best_response_level_kernel, dim3((unsigned)num_parents), dim3(p2::BR_BLOCK), 0,
-                     (hipStream_t)stream, values, policy, beliefs, to_act, deviating_player, child_offsets,
-                     child_count, parent_base);
+  if (max_children <= 5)
+    hipLaunchKernelGGL((p2::best_response_level_kernel<5>), dim3((unsigned)num_parents), dim3(p2::BR_BLOCK), 0,
+                       (hipStream_t)stream, values, policy, beliefs, to_act, deviating_player, child_offsets,
+                       child_count, parent_base);
+  else
+    hipLaunchKernelGGL((p2::best_response_level_kernel<p2::BR_MAXC>), dim3((unsigned)num_parents),
+                       dim3(p2::BR_BLOCK), 0, (hipStream_t)stream, values, policy, beliefs, to_act,
+                       deviating_player, child_offsets, child_count, parent_base);
   P2_LAUNCH_CHECK();
   return 0;
 }

@@ -1066,7 +1066,8 @@ class HipSparseCFREvaluator:
             base, end = self.depth_offsets[depth], self.depth_offsets[depth + 1]
             _lib.call("p2hip_best_response_level", _lib.ptr(values_br), _lib.ptr(policy), _lib.ptr(beliefs),
                       _lib.ptr(self.env.to_act), _lib.ptr(deviating_player), _lib.ptr(self.child_offsets),
-                      _lib.ptr(self.child_count), int(base), int(end - base), _lib.stream_ptr())
+                      _lib.ptr(self.child_count), int(base), int(end - base), int(self._max_children),
+                      _lib.stream_ptr())
         return values_br
 
     def _compute_exploitability(self) -> ExploitabilityStats:
