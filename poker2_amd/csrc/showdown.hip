@@ -434,7 +434,7 @@ __device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], co
   for (int i = 0; i < SD_PPT; ++i) {
     if (R.perm[i] == 0xFFFFFFFFu) continue;
     const int h = (int)(R.perm[i] & 0x7FFFu);
-    const float keep = (R.perm[i] & 0x8000u) ? 0.f : 1.f;
+    const bool live = !(R.perm[i] & 0x8000u);   // not blocked by the board
     const int L = (int)(R.lr[i] & 0xFFFFu), Rr = (int)(R.lr[i] >> 16);
     const int a = (int)(R.ab[i] & 0xFFu), b = (int)(R.ab[i] >> 8);
     const int iLa = (int)(R.cidx[i] & 0xFFu), iRa = (int)((R.cidx[i] >> 8) & 0xFFu);
@@ -456,13 +456,14 @@ __device__ __forceinline__ void showdown_finish(const float (&vk)[2][SD_PPT], co
       // The kernel is VALU-issue bound and an IEEE division is about ten instructions, so both
       // quotients share one hardware reciprocal and are corrected by one fused residual step
       // each, which keeps x/x == 1 and 0/x == 0 exact (an all-tie board stays exactly zero).
-      const bool valid = den > 1e-8f;
+      // a hand the board blocks goes the way of an empty denominator: every quotient 0, EV 0
+      const bool valid = live && den > 1e-8f;
       const float inv = valid ? __builtin_amdgcn_rcpf(den) : 0.f;
       float wp = win * inv, tp = tie * inv;
       wp = __builtin_fmaf(__builtin_fmaf(-wp, den, win), inv, wp);
       tp = __builtin_fmaf(__builtin_fmaf(-tp, den, tie), inv, tp);
       const float lp = valid ? 1.0f - wp - tp : 0.f;
-      e[p] = (wp - lp) * keep;
+      e[p] = wp - lp;
     }
     ev[h] = make_float2(e[0] * r0, e[1] * r1);
   }
