@@ -315,28 +315,30 @@ __device__ __forceinline__ void showdown_load_regs(const uint8_t* __restrict__ t
                                                    const uint16_t* ab_lds = nullptr) {
   const uint16_t* clist = reinterpret_cast<const uint16_t*>(tab + SD_OFF_CLIST);
   const bool ok = threadIdx.x * SD_PPT < P2_H;
-  if (ok) {
-    const SdU3 pm = *reinterpret_cast<const SdU3*>(tab + SD_OFF_PERM + threadIdx.x * (SD_PPT * 2));
-    const SdU3* lr = reinterpret_cast<const SdU3*>(tab + SD_OFF_LR + threadIdx.x * (SD_PPT * 4));
-    const SdU3* cx = reinterpret_cast<const SdU3*>(tab + SD_OFF_CIDX + threadIdx.x * (SD_PPT * 4));
-    const SdU3 l0 = lr[0], l1 = lr[1], c0 = cx[0], c1 = cx[1];
-    R.perm[0] = pm.x & 0xFFFFu; R.perm[1] = pm.x >> 16;
-    R.perm[2] = pm.y & 0xFFFFu; R.perm[3] = pm.y >> 16;
-    R.perm[4] = pm.z & 0xFFFFu; R.perm[5] = pm.z >> 16;
-    R.lr[0] = l0.x; R.lr[1] = l0.y; R.lr[2] = l0.z; R.lr[3] = l1.x; R.lr[4] = l1.y; R.lr[5] = l1.z;
-    R.cidx[0] = c0.x; R.cidx[1] = c0.y; R.cidx[2] = c0.z; R.cidx[3] = c1.x; R.cidx[4] = c1.y; R.cidx[5] = c1.z;
-  } else {
+  // Lanes past the end of the table repeat lane 0's loads and drop what they get (no branch around
+  // the loads, no defaults to set up): only `perm` marks them, nothing reads their lr / cidx / ab.
+  const int t = ok ? (int)threadIdx.x : 0;
+  const SdU3 pm = *reinterpret_cast<const SdU3*>(tab + SD_OFF_PERM + t * (SD_PPT * 2));
+  const SdU3* lr = reinterpret_cast<const SdU3*>(tab + SD_OFF_LR + t * (SD_PPT * 4));
+  const SdU3* cx = reinterpret_cast<const SdU3*>(tab + SD_OFF_CIDX + t * (SD_PPT * 4));
+  const SdU3 l0 = lr[0], l1 = lr[1], c0 = cx[0], c1 = cx[1];
+  // this lane's entry of the card lists of cards wave, wave + 4, ...: one base address, constant steps
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint16_t* mine = clist + wave * 51 + (lane < 51 ? lane : 50);
+  uint32_t cl[13];
 #pragma unroll
-    for (int i = 0; i < SD_PPT; ++i) { R.perm[i] = 0xFFFFFFFFu; R.lr[i] = 0u; R.cidx[i] = 0u; }
-  }
+  for (int i = 0; i < 13; ++i) cl[i] = mine[i * (4 * 51)];
+  const uint32_t raw[SD_PPT] = {pm.x & 0xFFFFu, pm.x >> 16, pm.y & 0xFFFFu, pm.y >> 16, pm.z & 0xFFFFu, pm.z >> 16};
+  R.lr[0] = l0.x; R.lr[1] = l0.y; R.lr[2] = l0.z; R.lr[3] = l1.x; R.lr[4] = l1.y; R.lr[5] = l1.z;
+  R.cidx[0] = c0.x; R.cidx[1] = c0.y; R.cidx[2] = c0.z; R.cidx[3] = c1.x; R.cidx[4] = c1.y; R.cidx[5] = c1.z;
 #pragma unroll
   for (int i = 0; i < SD_PPT; ++i) {
-    const int h = ok ? (int)(R.perm[i] & 0x7FFFu) : 0;
+    const int h = (int)(raw[i] & 0x7FFFu);
+    R.perm[i] = ok ? raw[i] : 0xFFFFFFFFu;
     R.ab[i] = ab_lds ? (uint32_t)ab_lds[h] : ((uint32_t)p2_combo.a[h] | ((uint32_t)p2_combo.b[h] << 8));
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int i = 0; i < 13; ++i) R.clist[i] = lane < 51 ? clist[(wave + 4 * i) * 51 + lane] : 0xFFFFu;
+  for (int i = 0; i < 13; ++i) R.clist[i] = lane < 51 ? cl[i] : 0xFFFFu;
 }
 
 // Gather both ranges of the node whose beliefs start at `bel` ([2,H]) into strength order:
