@@ -253,13 +253,16 @@ def test_structural_invariants_after_many_iterations():
     assert (ev.self_reach[n:, 0][blocked] == 0).all() and (ev.self_reach[n:, 1][blocked] == 0).all()
 
 
-@pytest.mark.parametrize("depth,max_raises", [(2, None), (16, 2)])
-def test_best_response_and_exploitability_match_oracle(depth, max_raises):
+@pytest.mark.parametrize("depth,max_raises,bins", [(2, None, (0.5, 1.0)), (16, 2, (0.5, 1.0)),
+                                                   (3, None, (0.25, 0.5, 1.0, 2.0))])
+def test_best_response_and_exploitability_match_oracle(depth, max_raises, bins):
     """The best-response kernels against the oracle ON THE SAME STATE (the evaluator's tensors are
-    copied into the oracle first), so that only the operation under test is compared."""
+    copied into the oracle first), so that only the operation under test is compared.  Four bet sizes
+    give parents of up to seven children: the kernel build for more than five."""
     from oracle import best_response as OBR
     iters = 6
-    ev, orc = make_pair(3, depth, max_raises, seed=31, fused=True, iters=iters)
+    ev, orc = make_pair(3, depth, max_raises, seed=31, fused=True, iters=iters, bins=bins, stacks=(3000, 3000))
+    assert (ev._max_children > 5) == (len(bins) > 2)
     for t in range(iters):
         ev.cfr_iteration(t)
     for name in OCFR.OracleCFR.STATE_NAMES:
