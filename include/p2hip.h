@@ -234,6 +234,13 @@ int p2hip_unblocked_mass_by_player(const float* beliefs, const int64_t* to_act, 
 int p2hip_unblocked_mass_ratio(const float* numer, const float* denom, const int64_t* parent_index,
                                int64_t rows, float eps, float* out, void* stream);
 
+/* The same quotient from denominators that are already unblocked masses: d = denom_unblocked[parent_index[c]]
+ * ([parents,H], e.g. from p2hip_unblocked_mass).  Siblings share their parent's row, so its card sums are
+ * taken once per parent; the reference passes precomputed denominator statistics for the same purpose
+ * (denom_stats of unblocked_mass_ratio_indirect_triton, search/fused_cfr_triton.py:1499-1556). */
+int p2hip_unblocked_mass_ratio_of(const float* numer, const float* denom_unblocked, const int64_t* parent_index,
+                                  int64_t rows, float eps, float* out, void* stream);
+
 /* ---- per-operation CFR kernels (search/fused_cfr_triton.py) ------------------------- */
 /* Scalars that depend on the iteration number are 0-D device tensors (const float*). */
 

@@ -52,6 +52,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_unblocked_mass": [_P, _L, _P, _P],
     "p2hip_unblocked_mass_by_player": [_P, _P, _L, _I, _P, _P],
     "p2hip_unblocked_mass_ratio": [_P, _P, _P, _L, _F, _P, _P],
+    "p2hip_unblocked_mass_ratio_of": [_P, _P, _P, _L, _F, _P, _P],
     "p2hip_dcfr_update": [_P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _P, _P],
     "p2hip_block_and_normalize": [_P, _P, _P, _L, _I, _F, _P],
     "p2hip_regret_matching_divide": [_P, _P, _P, _P, _L, _F, _P],

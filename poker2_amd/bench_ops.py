@@ -171,6 +171,71 @@ def cases(repeats: int):
     yield (f"encode nodes={ev.total_nodes}", ev.total_nodes * (13 * 8 + 16 + 5 * 8 + 10 * 8),
            lambda: ev.feature_encoder.encode(ev.beliefs, pre_chance_node=ev.new_street_mask))
 
+    # --- the remaining per-operation kernels, on the tensors of the same search: T = 86 016 nodes in three
+    # levels (4096 roots, 16 384 children of the roots, 65 536 leaves); rows counted: read once, written once,
+    # a parent's rows once per parent
+    T, N = ev.total_nodes, n
+    top = int(ev.depth_offsets[-2])                          # rows that can have children
+    C = T - N
+    l1, l2 = int(ev.depth_offsets[1]), int(ev.depth_offsets[2])
+    n_l1, n_l2 = l2 - l1, T - l2
+    row = H * 4
+    bel3 = torch.rand(T, 2, H, device=dev)
+    yield (f"block_and_normalize rows={T}x2", 4 * T * row + T * H,
+           lambda: F.fused_block_and_normalize_beliefs_(bel3, ev.allowed_hands, ev.allowed_hands_prob))
+    posr = torch.rand(C, H, device=dev)
+    den = torch.rand(C, H, device=dev)
+    uni = torch.full((C, H), 0.25, device=dev)
+    outc = torch.empty(C, H, device=dev)
+    yield (f"regret_matching_divide children={C}", 4 * C * row,
+           lambda: F.fused_regret_matching_divide_(posr, den, uni, outc))
+    vals3 = torch.rand(T, 2, H, device=dev)
+    vsrc = vals3[N:].contiguous()
+    outv = torch.empty_like(vsrc)
+    prev_c = ev.prev_actor[N:].contiguous()
+    yield (f"weight_child_values children={C}", 6 * C * row,
+           lambda: F.fused_weight_child_values(vsrc, prev_c, posr, den, outv))
+    del vsrc, outv
+    vavg = torch.rand(T, 2, H, device=dev)
+    yield (f"update_average_values rows={T}x2", 6 * T * row,
+           lambda: F.fused_update_average_values_(vavg, vals3, 3.0, 1.0))
+    o_t, n_t, inv_t = (torch.tensor(x, device=dev) for x in (3.0, 1.0, 0.25))
+    yield (f"avg_values_zero_sum rows={T}x2", 8 * T * row,
+           lambda: F.fused_avg_values_zero_sum_(vavg, vals3, bel3, o_t, n_t, inv_t, True))
+    regrets = torch.zeros(T, H, device=dev)
+    actor_v = torch.rand(top, H, device=dev)
+    src_w = torch.rand(top, H, device=dev)
+    yield (f"regret_tail children={C}", (2 * C + 2 * top) * row,
+           lambda: F.fused_regret_tail_(regrets, vals3, actor_v, src_w, ev.parent_index, ev.prev_actor, N))
+    pavg = torch.rand(T, H, device=dev)
+    pol = torch.rand(T, H, device=dev)
+    reach_avg3 = torch.rand(T, 2, H, device=dev)
+    yield (f"average_policy_mix children={C}", (3 * C + 2 * top) * row,
+           lambda: F.fused_average_policy_mix_(pavg, pol, bel3, reach_avg3, ev.env.to_act, ev.parent_index, 3.0, 1.0, N))
+    co1, cc1 = ev.child_offsets[l1:l2].contiguous(), ev.child_count[l1:l2].contiguous()
+    yield (f"weighted_parent_sum parents={n_l1}", (4 * n_l2 + 2 * n_l1) * row,
+           lambda: F.fused_weighted_parent_sum(vals3, ev.prev_actor, pol, pavg, co1, cc1, l1))
+    yield (f"reach_weights_depth children={n_l2}", (3 * n_l2 + 2 * n_l1) * row + n_l2 * H,
+           lambda: F.fused_reach_weights_depth_(reach_avg3, pol, ev.allowed_hands, ev.parent_index, ev.prev_actor, l2, T))
+    root_b = ev.beliefs[:N].contiguous()
+    yield (f"deep_beliefs rows={C}x2", (4 * C + 2 * N) * row,
+           lambda: F.fused_deep_beliefs_(bel3, root_b, reach_avg3, ev.allowed_hands_prob, ev._root_index, N))
+    t_all = torch.zeros(T, dtype=torch.int64, device=dev)
+    t0 = torch.zeros((), dtype=torch.int64, device=dev)
+    yield (f"sample_snapshot rows={T}", 2 * T * row, lambda: F.fused_sample_snapshot_(pavg, pol, t_all, t0))
+    yield (f"unblocked_mass_opp_at_parents parents={top}", 2 * top * row,
+           lambda: F.unblocked_mass_opp_at_parents_triton(bel3, ev.env.to_act, top))
+    par_c = ev.parent_index[N:].contiguous()
+    yield (f"unblocked_mass_ratio_indirect children={C}", (2 * C + top) * row,
+           lambda: F.unblocked_mass_ratio_indirect_triton(posr, actor_v, par_c))
+    m_leaves = 20_000
+    hv, last, outm = (torch.rand(m_leaves, 2, H, device=dev) for _ in range(3))
+    bl = bel3[:m_leaves]
+    onon, oon = torch.tensor(1.25, device=dev), torch.tensor(0.25, device=dev)
+    yield (f"model_values_mix_zero_sum leaves={m_leaves}", 8 * m_leaves * row,
+           lambda: F.fused_model_values_mix_zero_sum(hv, last, bl, onon, oon, outm, True))
+    del bel3, posr, den, uni, outc, vals3, vavg, regrets, actor_v, src_w, pavg, pol, reach_avg3, hv, last, outm
+
     # --- local best response, one tree level of the same search: the 16 384 parents of level 1, four
     # children each (per parent: the actor's range, per child its policy row and both value rows in,
     # both value rows of the parent out)

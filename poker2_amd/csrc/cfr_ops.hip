@@ -64,35 +64,64 @@ __global__ __launch_bounds__(FLAT_BLOCK) void dcfr_update_kernel(
   }
 }
 
-// K2 -- fused_cfr_triton.py:245-283.  target row r uses mask / fallback row r / stride.
+// K2 -- fused_cfr_triton.py:245-283.  target row r uses mask / fallback row r / stride.  A workgroup takes
+// two rows: both are requested before either is used and their sums share one block reduction (a row's
+// own sum is formed exactly as when it had the workgroup to itself).
+constexpr int K2_ROWS = 2;
 __global__ __launch_bounds__(OPS_BLOCK) void block_normalize_kernel(float* __restrict__ target,
                                                                      const uint8_t* __restrict__ allowed,
                                                                      const float* __restrict__ allowed_prob,
-                                                                     int stride, float eps) {
-  __shared__ float red[OPS_WAVES];
-  const int64_t row = blockIdx.x, outer = row / stride;
-  float2* t2 = p2_row2(target, row);
-  const uchar2* m2 = reinterpret_cast<const uchar2*>(allowed + outer * P2_H);
-  float2 v[OPS_PAIRS_PER_THREAD];
-  float local = 0.f;
+                                                                     int64_t rows, int stride, float eps) {
+  __shared__ float red[K2_ROWS][OPS_WAVES];
+  const int64_t row0 = (int64_t)blockIdx.x * K2_ROWS;
+  float2 x[K2_ROWS][OPS_PAIRS_PER_THREAD];
+  uchar2 m[K2_ROWS][OPS_PAIRS_PER_THREAD];
 #pragma unroll
-  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
-    const int i = threadIdx.x + j * OPS_BLOCK;
-    v[j] = make_float2(0.f, 0.f);
-    if (i < P2_HPAIRS) {
-      const float2 x = t2[i];
-      const uchar2 m = m2[i];
-      v[j].x = m.x ? x.x : 0.f;
-      v[j].y = m.y ? x.y : 0.f;
-      local += v[j].x + v[j].y;
+  for (int r = 0; r < K2_ROWS; ++r) {
+    const int64_t row = row0 + r < rows ? row0 + r : rows - 1;   // past the end: the last row again, not stored
+    const float2* t2 = p2_row2(target, row);
+    const uchar2* m2 = reinterpret_cast<const uchar2*>(allowed + (row / stride) * P2_H);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      const int ic = i < P2_HPAIRS ? i : 0;
+      x[r][j] = t2[ic];
+      m[r][j] = m2[ic];
     }
   }
-  const float total = p2_block_sum<OPS_WAVES>(local, red);
-  const float2* f2 = p2_row2(allowed_prob, outer);
+  float local[K2_ROWS];
 #pragma unroll
-  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
-    const int i = threadIdx.x + j * OPS_BLOCK;
-    if (i < P2_HPAIRS) t2[i] = total > eps ? make_float2(v[j].x / total, v[j].y / total) : f2[i];
+  for (int r = 0; r < K2_ROWS; ++r) {
+    local[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      const bool in = i < P2_HPAIRS;
+      x[r][j].x = (in && m[r][j].x) ? x[r][j].x : 0.f;
+      x[r][j].y = (in && m[r][j].y) ? x[r][j].y : 0.f;
+      if (in) local[r] += x[r][j].x + x[r][j].y;
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int r = 0; r < K2_ROWS; ++r) {
+    const float w = p2_wave_sum(local[r]);
+    if (lane == 0) red[r][wave] = w;
+  }
+  p2_sync_lds();
+#pragma unroll
+  for (int r = 0; r < K2_ROWS; ++r) {
+    if (row0 + r >= rows) break;
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < OPS_WAVES; ++w) total += red[r][w];
+    float2* t2 = p2_row2(target, row0 + r);
+    const float2* f2 = p2_row2(allowed_prob, (row0 + r) / stride);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      if (i < P2_HPAIRS) t2[i] = total > eps ? make_float2(x[r][j].x / total, x[r][j].y / total) : f2[i];
+    }
   }
 }
 
@@ -428,38 +457,53 @@ __global__ __launch_bounds__(OPS_BLOCK) void reach_weights_kernel(float* __restr
   }
 }
 
-// K16 -- fused_cfr_triton.py:1996-2036; grid (total - N, 2); rows below N are skipped
+// K16 -- fused_cfr_triton.py:1996-2036; one workgroup per row below the roots, both players: the four input
+// rows are requested together and the two sums share one block reduction.
 __global__ __launch_bounds__(OPS_BLOCK) void deep_beliefs_kernel(const float* __restrict__ root_beliefs,
                                                                   const float* __restrict__ reach,
                                                                   const float* __restrict__ allowed_prob,
                                                                   const int64_t* __restrict__ root_index,
                                                                   float* __restrict__ out, int64_t n_roots,
                                                                   float eps) {
-  __shared__ float red[OPS_WAVES];
+  __shared__ float red[2][OPS_WAVES];
   const int64_t i_row = blockIdx.x + n_roots;
-  const int p = blockIdx.y;
   const int64_t root = root_index[i_row];
-  const float2* rb2 = p2_row2(root_beliefs, root * 2 + p);
-  const float2* rw2 = p2_row2(reach, i_row * 2 + p);
-  float2 v[OPS_PAIRS_PER_THREAD];
-  float local = 0.f;
+  float2 v[2][OPS_PAIRS_PER_THREAD];
 #pragma unroll
-  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
-    const int i = threadIdx.x + j * OPS_BLOCK;
-    v[j] = make_float2(0.f, 0.f);
-    if (i < P2_HPAIRS) {
-      const float2 a = rb2[i], b = rw2[i];
-      v[j] = make_float2(a.x * b.x, a.y * b.y);
-      local += v[j].x + v[j].y;
+  for (int p = 0; p < 2; ++p) {
+    const float2* rb2 = p2_row2(root_beliefs, root * 2 + p);
+    const float2* rw2 = p2_row2(reach, i_row * 2 + p);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      const int ic = i < P2_HPAIRS ? i : 0;
+      const float2 a = rb2[ic], b = rw2[ic];
+      v[p][j] = i < P2_HPAIRS ? make_float2(a.x * b.x, a.y * b.y) : make_float2(0.f, 0.f);
     }
   }
-  const float total = p2_block_sum<OPS_WAVES>(local, red);
-  const float2* f2 = p2_row2(allowed_prob, i_row);
-  float2* o2 = p2_row2(out, i_row * 2 + p);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
-    const int i = threadIdx.x + j * OPS_BLOCK;
-    if (i < P2_HPAIRS) o2[i] = total > eps ? make_float2(v[j].x / total, v[j].y / total) : f2[i];
+  for (int p = 0; p < 2; ++p) {
+    float local = 0.f;
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j)
+      if (threadIdx.x + j * OPS_BLOCK < P2_HPAIRS) local += v[p][j].x + v[p][j].y;
+    const float w = p2_wave_sum(local);
+    if (lane == 0) red[p][wave] = w;
+  }
+  p2_sync_lds();
+  const float2* f2 = p2_row2(allowed_prob, i_row);
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < OPS_WAVES; ++w) total += red[p][w];
+    float2* o2 = p2_row2(out, i_row * 2 + p);
+#pragma unroll
+    for (int j = 0; j < OPS_PAIRS_PER_THREAD; ++j) {
+      const int i = threadIdx.x + j * OPS_BLOCK;
+      if (i < P2_HPAIRS) o2[i] = total > eps ? make_float2(v[p][j].x / total, v[p][j].y / total) : f2[i];
+    }
   }
 }
 
@@ -507,8 +551,8 @@ int p2hip_block_and_normalize(float* target, const uint8_t* allowed, const float
   if (rows == 0) return 0;
   P2_REQ(target && allowed && allowed_prob && p2_aligned8(target) && p2_aligned8(allowed_prob) &&
          (reinterpret_cast<uintptr_t>(allowed) & 1u) == 0);
-  hipLaunchKernelGGL(p2::block_normalize_kernel, dim3((unsigned)rows), dim3(p2::OPS_BLOCK), 0, P2_ST, target,
-                     allowed, allowed_prob, players_per_row, eps);
+  hipLaunchKernelGGL(p2::block_normalize_kernel, dim3((unsigned)((rows + p2::K2_ROWS - 1) / p2::K2_ROWS)),
+                     dim3(p2::OPS_BLOCK), 0, P2_ST, target, allowed, allowed_prob, rows, players_per_row, eps);
   P2_LAUNCH_CHECK();
   return 0;
 }
@@ -685,7 +729,7 @@ int p2hip_deep_beliefs(float* out, const float* root_beliefs, const float* reach
   if (total <= n_roots) return 0;
   P2_REQ(out && root_beliefs && reach && allowed_prob && root_index);
   P2_REQ(p2_aligned8(out) && p2_aligned8(root_beliefs) && p2_aligned8(reach) && p2_aligned8(allowed_prob));
-  hipLaunchKernelGGL(p2::deep_beliefs_kernel, dim3((unsigned)(total - n_roots), 2), dim3(p2::OPS_BLOCK), 0, P2_ST,
+  hipLaunchKernelGGL(p2::deep_beliefs_kernel, dim3((unsigned)(total - n_roots)), dim3(p2::OPS_BLOCK), 0, P2_ST,
                      root_beliefs, reach, allowed_prob, root_index, out, n_roots, eps);
   P2_LAUNCH_CHECK();
   return 0;

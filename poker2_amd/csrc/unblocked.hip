@@ -258,6 +258,50 @@ __global__ __launch_bounds__(UB_BLOCK) void unblocked_ratio_kernel(const float* 
   }
 }
 
+// out[c] = d > eps ? unblocked(numer[c]) / d : 0 with d = denom_unblocked[parent(c)] already computed
+// (one row per parent): siblings share their parent's row, so the denominator's card sums are taken once
+// per parent instead of once per child.  Four numerators per group.
+__global__ __launch_bounds__(UB_BLOCK) void unblocked_ratio_of_kernel(const float* __restrict__ numer,
+                                                                       const float* __restrict__ denom_unblocked,
+                                                                       const int64_t* __restrict__ parent_index,
+                                                                       float eps, int64_t rows, float* __restrict__ out) {
+  __shared__ UnblockedLds s;
+  const int64_t g = blockIdx.x;
+  const int nv = (int)(rows - g * UB_ROWS < UB_ROWS ? rows - g * UB_ROWS : UB_ROWS);
+  CardLane cl;
+  HandCards hc;
+  card_lane_init(cl);
+  hand_cards_init(hc);
+  float2 pre[UB_ROWS][UB_PPT], den[UB_ROWS][UB_PPT];
+#pragma unroll
+  for (int v = 0; v < UB_ROWS; ++v) {
+    const int64_t c = g * UB_ROWS + (v < nv ? v : nv - 1);       // past the end: the last one again, not stored
+    fetch_row(numer + c * P2_H, pre[v]);
+    fetch_row(denom_unblocked + parent_index[c] * P2_H, den[v]);
+  }
+#pragma unroll
+  for (int v = 0; v < UB_ROWS; ++v) stage_row(pre[v], s.t[v]);
+  p2_sync_lds();
+  card_sums_fixed(cl, s.t[0], UB_STRIDE, nv, s.cs);
+#pragma unroll
+  for (int v = 0; v < UB_ROWS; ++v) {
+    if (v >= nv) break;
+    const double* cs = s.cs + v * P2_CARDS;
+    const double total = card_total(cs);
+    float2* o2 = p2_row2(out, g * UB_ROWS + v);
+#pragma unroll
+    for (int k = 0; k < UB_PPT; ++k) {
+      const int i = threadIdx.x + k * UB_BLOCK;
+      if (i < P2_HPAIRS) {
+        const float n0 = unblocked_of(pre[v][k].x, cs, total, hc.ab[k][0]);
+        const float n1 = unblocked_of(pre[v][k].y, cs, total, hc.ab[k][1]);
+        const float d0 = den[v][k].x, d1 = den[v][k].y;
+        o2[i] = make_float2(d0 > eps ? n0 / d0 : 0.f, d1 > eps ? n1 / d1 : 0.f);
+      }
+    }
+  }
+}
+
 // One workgroup per group of rows, dispatched in address order (measured 3 % faster than a
 // resident grid walking the groups with a stride, although each workgroup then recomputes its
 // lanes' combo offsets); the kernels' loops only run more than once beyond 2^30 groups.
@@ -298,6 +342,18 @@ int p2hip_unblocked_mass_ratio(const float* numer, const float* denom, const int
   if (!p2_aligned8(numer) || !p2_aligned8(denom) || !p2_aligned8(out)) return P2_EINVAL;
   hipLaunchKernelGGL(p2::unblocked_ratio_kernel, dim3(p2::ub_grid((rows + 1) / 2, 4)), dim3(p2::UB_BLOCK), 0,
                      (hipStream_t)stream, numer, denom, parent_index, eps, rows, out);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_unblocked_mass_ratio_of(const float* numer, const float* denom_unblocked, const int64_t* parent_index,
+                                  int64_t rows, float eps, float* out, void* stream) {
+  if (rows < 0 || rows > ((int64_t)0x7FFFFFFF) * p2::UB_ROWS) return P2_EINVAL;
+  if (rows > 0 && (!numer || !denom_unblocked || !parent_index || !out)) return P2_EINVAL;
+  if (rows == 0) return 0;
+  if (!p2_aligned8(numer) || !p2_aligned8(denom_unblocked) || !p2_aligned8(out)) return P2_EINVAL;
+  hipLaunchKernelGGL(p2::unblocked_ratio_of_kernel, dim3((unsigned)((rows + p2::UB_ROWS - 1) / p2::UB_ROWS)),
+                     dim3(p2::UB_BLOCK), 0, (hipStream_t)stream, numer, denom_unblocked, parent_index, eps, rows, out);
   P2_LAUNCH_CHECK();
   return 0;
 }

@@ -370,8 +370,15 @@ def unblocked_mass_ratio_indirect_triton(numer_target, denom_target, parent_inde
     _f32(numer_target=numer_target, denom_target=denom_target)
     _i64(num_children, parent_index=parent_index)
     out = torch.empty_like(numer_target)
-    _lib.call("p2hip_unblocked_mass_ratio", _p(numer_target), _p(denom_target), _p(parent_index), num_children,
-              float(eps), _p(out), _S())
+    if num_children > top:
+        # siblings share a denominator: its unblocked mass once per parent, then the quotients
+        denom_unblocked = torch.empty_like(denom_target)
+        _lib.call("p2hip_unblocked_mass", _p(denom_target), top, _p(denom_unblocked), _S())
+        _lib.call("p2hip_unblocked_mass_ratio_of", _p(numer_target), _p(denom_unblocked), _p(parent_index),
+                  num_children, float(eps), _p(out), _S())
+    else:
+        _lib.call("p2hip_unblocked_mass_ratio", _p(numer_target), _p(denom_target), _p(parent_index), num_children,
+                  float(eps), _p(out), _S())
     return out
 
 
