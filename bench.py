@@ -123,6 +123,30 @@ def cpu_baseline(tree: str, seed: int, budget_s: float = 20.0) -> dict:
                       f"of the numpy oracle, {med * 1e3:.1f} ms per iteration"}
 
 
+def flat_stream_rate(pairs: int = 1 << 26, reps: int = 5) -> float:
+    """GB/s of a structure-free element-wise stream with the iteration kernel's read / write mix (5 input
+    and 7 output arrays of 512 MiB each, one 8-byte access per lane and array): what HBM gives such a
+    kernel on THIS machine when nothing else limits it.  Measurement aid of the library
+    (p2hip_stream_probe); runs after the timed region, on its own buffers."""
+    import torch
+    from poker2_amd import _lib
+    src = torch.zeros(5 * pairs * 2, dtype=torch.float32, device="cuda")
+    dst = torch.empty(7 * pairs * 2, dtype=torch.float32, device="cuda")
+    run = lambda: _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, _lib.stream_ptr())
+    for _ in range(2):
+        run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    del src, dst
+    torch.cuda.empty_cache()
+    return 12 * pairs * 8 / (ms * 1e-3) / 1e9
+
+
 def side_metrics() -> dict:
     """Showdown evaluations/s (B=4096 public states) and hands ranked/s (2^20 hands)."""
     import torch
@@ -297,6 +321,8 @@ def main() -> None:
     del ev
     torch.cuda.empty_cache()
 
+    flat = flat_stream_rate()
+    moved = traffic if traffic else algo_bytes
     result = {
         "metric": "river CFR iters/sec x subgames",
         "value": value,
@@ -323,7 +349,12 @@ def main() -> None:
                      "traffic_read_write": list(rw) if rw else None,
                      "frac_of_peak_on_measured_traffic": (traffic / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if traffic else None,
                      "kernel": "cfr_iteration_kernel", "kernel_ms": kernel_ms,
-                     "algorithmic_bytes_per_launch": algo_bytes},
+                     "algorithmic_bytes_per_launch": algo_bytes,
+                     "flat_stream_same_mix_GBps": flat,
+                     "flat_stream_note": "p2hip_stream_probe: 5 arrays read + 7 written, 512 MiB each, measured by "
+                                         "this run after the timed region; the kernel's bytes (counted traffic where "
+                                         "a counter run exists, else algorithmic) over its time, as a share of it",
+                     "frac_of_flat_stream": moved / (kernel_ms * 1e-3) / 1e9 / flat},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.tree, args.seed)

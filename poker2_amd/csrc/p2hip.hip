@@ -10,6 +10,7 @@
 #include "best_response.hip"
 #include "tree.hip"
 #include "datagen.hip"
+#include "stream_probe.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.

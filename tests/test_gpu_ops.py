@@ -367,6 +367,27 @@ def test_unblocked_mass_at_every_buffer_alignment_and_ragged_row_counts(rows):
     assert np.array_equal(got[0], got[1])
 
 
+def test_stream_probe_moves_what_it_says():
+    """The measurement aid behind bench.py's flat-stream figure: every output array holds the sum of the input
+    arrays plus its own number (so every load and every store happens), and unsupported mixes are refused."""
+    from poker2_amd import _lib
+    pairs = 1000 * 256 + 77
+    rng = np.random.default_rng(3)
+    src = torch.from_numpy(rng.random((5, pairs, 2)).astype(np.float32)).cuda()
+    dst = torch.full((7, pairs, 2), -1.0, device="cuda")
+    _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, _lib.stream_ptr())
+    torch.cuda.synchronize()
+    acc = torch.tensor([1.0, 2.0], device="cuda").expand(pairs, 2).clone()
+    for k in range(5):
+        acc = acc + src[k]
+    for k in range(7):
+        exp = acc.clone()
+        exp[:, 0] += float(k)
+        assert torch.equal(dst[k], exp)
+    code = _lib.load().p2hip_stream_probe(src.data_ptr(), dst.data_ptr(), pairs, 3, 3, _lib.stream_ptr())
+    assert code != 0
+
+
 def test_wrappers_refuse_arguments_that_would_index_out_of_bounds(F):
     """Sizes, dtypes and row bounds the kernels index with are checked on the host (and stay
     checked under ``python -O``): none of these calls may reach the GPU."""
