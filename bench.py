@@ -123,28 +123,30 @@ def cpu_baseline(tree: str, seed: int, budget_s: float = 20.0) -> dict:
                       f"of the numpy oracle, {med * 1e3:.1f} ms per iteration"}
 
 
-def flat_stream_rate(pairs: int = 1 << 26, reps: int = 5) -> float:
+def flat_stream_rate(pairs: int = 1 << 26, reps: int = 5) -> dict:
     """GB/s of a structure-free element-wise stream with the iteration kernel's read / write mix (5 input
-    and 7 output arrays of 512 MiB each, one 8-byte access per lane and array): what HBM gives such a
-    kernel on THIS machine when nothing else limits it.  Measurement aid of the library
-    (p2hip_stream_probe); runs after the timed region, on its own buffers."""
+    and 7 output arrays of 512 MiB each, one 8-byte access per lane and array), with ordinary and with
+    non-temporal accesses: what HBM gives such a kernel on THIS machine when nothing else limits it.
+    Measurement aid of the library (p2hip_stream_probe); runs after the timed region, on its own buffers."""
     import torch
     from poker2_amd import _lib
     src = torch.zeros(5 * pairs * 2, dtype=torch.float32, device="cuda")
     dst = torch.empty(7 * pairs * 2, dtype=torch.float32, device="cuda")
-    run = lambda: _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, _lib.stream_ptr())
-    for _ in range(2):
-        run()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / reps
+    out = {}
+    for name, nt in (("plain", 0), ("non_temporal", 1)):
+        run = lambda: _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, nt, _lib.stream_ptr())
+        for _ in range(2):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = 12 * pairs * 8 / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9
     del src, dst
     torch.cuda.empty_cache()
-    return 12 * pairs * 8 / (ms * 1e-3) / 1e9
+    return out
 
 
 def side_metrics() -> dict:
@@ -351,10 +353,11 @@ def main() -> None:
                      "kernel": "cfr_iteration_kernel", "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes,
                      "flat_stream_same_mix_GBps": flat,
-                     "flat_stream_note": "p2hip_stream_probe: 5 arrays read + 7 written, 512 MiB each, measured by "
-                                         "this run after the timed region; the kernel's bytes (counted traffic where "
-                                         "a counter run exists, else algorithmic) over its time, as a share of it",
-                     "frac_of_flat_stream": moved / (kernel_ms * 1e-3) / 1e9 / flat},
+                     "flat_stream_note": "p2hip_stream_probe: 5 arrays read + 7 written, 512 MiB each, ordinary and "
+                                         "non-temporal accesses, measured by this run after the timed region; the "
+                                         "kernel's bytes (counted traffic where a counter run exists, else "
+                                         "algorithmic) over its time, as a share of the faster of the two",
+                     "frac_of_flat_stream": moved / (kernel_ms * 1e-3) / 1e9 / max(flat.values())},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.tree, args.seed)

@@ -407,9 +407,11 @@ int p2hip_upload_floats(float* dst, const float* host_values, int n, void* strea
 
 /* No counterpart in the reference and not on the search path: a structure-free element-wise stream over
  * n_read input and n_write output arrays of `pairs` float2 each (array k starts k * pairs float2 after the
- * base pointer), for (n_read, n_write) in {(5,7), (1,1), (2,0), (0,2)}.  bench.py times it to report what
- * HBM gives a kernel of the iteration kernel's read / write mix on the same machine. */
-int p2hip_stream_probe(const float* in, float* out, int64_t pairs, int n_read, int n_write, void* stream);
+ * base pointer), for (n_read, n_write) in {(5,7), (1,1), (2,0), (0,2)}; non_temporal != 0 marks every access
+ * non-temporal.  bench.py times it to report what HBM gives a kernel of the iteration kernel's read / write
+ * mix on the same machine. */
+int p2hip_stream_probe(const float* in, float* out, int64_t pairs, int n_read, int n_write, int non_temporal,
+                       void* stream);
 
 #ifdef __cplusplus
 }

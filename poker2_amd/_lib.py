@@ -72,7 +72,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_sample_snapshot": [_P, _P, _P, _P, _L, _P],
     "p2hip_cfr_iteration": [_P, _L, _I, _I, _P],
     "p2hip_write_scalars": [_P, _P, _P, _P, _P],
-    "p2hip_stream_probe": [_P, _P, _L, _I, _I, _P],
+    "p2hip_stream_probe": [_P, _P, _L, _I, _I, _I, _P],
 }
 _RESTYPE = {"p2hip_error_string": ctypes.c_char_p, "p2hip_showdown_table_bytes": _L,
             "p2hip_tree_node_columns": _L}

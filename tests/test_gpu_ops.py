@@ -375,16 +375,18 @@ def test_stream_probe_moves_what_it_says():
     rng = np.random.default_rng(3)
     src = torch.from_numpy(rng.random((5, pairs, 2)).astype(np.float32)).cuda()
     dst = torch.full((7, pairs, 2), -1.0, device="cuda")
-    _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, _lib.stream_ptr())
-    torch.cuda.synchronize()
     acc = torch.tensor([1.0, 2.0], device="cuda").expand(pairs, 2).clone()
     for k in range(5):
         acc = acc + src[k]
-    for k in range(7):
-        exp = acc.clone()
-        exp[:, 0] += float(k)
-        assert torch.equal(dst[k], exp)
-    code = _lib.load().p2hip_stream_probe(src.data_ptr(), dst.data_ptr(), pairs, 3, 3, _lib.stream_ptr())
+    for non_temporal in (0, 1):
+        dst.fill_(-1.0)
+        _lib.call("p2hip_stream_probe", src.data_ptr(), dst.data_ptr(), pairs, 5, 7, non_temporal, _lib.stream_ptr())
+        torch.cuda.synchronize()
+        for k in range(7):
+            exp = acc.clone()
+            exp[:, 0] += float(k)
+            assert torch.equal(dst[k], exp)
+    code = _lib.load().p2hip_stream_probe(src.data_ptr(), dst.data_ptr(), pairs, 3, 3, 0, _lib.stream_ptr())
     assert code != 0
 
 
