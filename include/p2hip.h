@@ -329,12 +329,14 @@ int p2hip_sample_snapshot(const float* policy_probs, float* policy_probs_sample,
 
 /* Device pointers of one subgame batch.  Tree arrays and state tensors are the evaluator's
  * own (row-major over all nodes of all roots); the rest is derived once per subgame:
- *   node_flags [total] bytes: bit0 = river showdown row, bit1 = terminal row
+ *   node_flags [total] bytes: bit0 = river showdown row, bit1 = terminal row, bit2 = the row has children,
+ *             bit3 = childless row whose ranges feed a leaf evaluation (a showdown row, or a row the caller's
+ *             leaf network is asked about); bits 2 and 3 are read by lean launches only
  *   root_parent_offsets [roots+1], root_parents: rows that have children, per root, ascending
  *   root_showdown_offsets [roots+1], root_showdown_nodes: river showdown rows per root
  *   tables [roots, p2hip_showdown_table_bytes()] (NULL when no row is a showdown)
  *   potential [total,2] float, scale [total] float: showdown pay-off factors per row
- *   scratch [total,H] float workspace
+ *   scratch [total,H] float workspace (may be NULL when reach_avg_prev is given)
  *   fscal[8]: t^alpha, t^beta, t^alpha+1, t^beta+1, mix_old, mix_new, mix_old+mix_new, 1/(mix_old+mix_new)
  *   iscal[8]: t, apply_dcfr, cfr_plus, average_policy_is_copied, enforce_zero_sum, update_average_values,
  *             cfr_avg (regret weights and showdown values from beliefs_avg), linear (regrets of player t mod 2
@@ -379,6 +381,13 @@ typedef struct P2HipIterArgs {
    * rewrites, so it runs everywhere first). */
   const int64_t* item_root;
   const uint8_t* item_top;
+  /* Optional, [total,2,H]: reach_avg as the PREVIOUS iteration left it, in a buffer of its own.  The
+   * average-policy mix (search/fused_sparse_cfr_evaluator.py:355-398) weighs the old average policy by the
+   * parent's reach_avg from before this iteration; with NULL the kernel saves that row in `scratch`
+   * before it overwrites reach_avg in place.  A caller that keeps two reach_avg buffers and swaps them
+   * from iteration to iteration passes the other one here and saves a row write and a row read per
+   * parent.  Root rows of both buffers hold the roots' reach (1); must differ from reach_avg. */
+  const float* reach_avg_prev;
 } P2HipIterArgs;
 
 /* One workgroup per root runs the whole iteration of FusedSparseCFREvaluator.cfr_iteration
@@ -386,7 +395,13 @@ typedef struct P2HipIterArgs {
  * cfr_avg = False: sample snapshot, instantaneous regrets, DCFR update, regret matching, reach,
  * beliefs, average policy, reach_avg, beliefs_avg (phases bit 0; bit 2 = the regret part alone, bit 3 = the
  * reach / belief / average-policy part alone); showdown leaf values, value backup, average values
- * (phases bit 1).  host_args is a HOST pointer to a struct of device
+ * (phases bit 1).  phases bit 4 (16) marks a LEAN iteration, for callers that run many iterations and
+ * look at the state only after the last (evaluate_cfr, search/cfr_evaluator.py:1497-1528): the reach /
+ * belief part then stores only rows that a later part of this iteration or the next iteration reads —
+ * reach and reach_avg of rows with children, beliefs of rows with children or a leaf evaluation
+ * (node_flags bits 2, 3), beliefs_avg only under cfr_avg or enforce_zero_sum.  The rows left out are
+ * functions of rows that are kept: one iteration without the bit afterwards leaves all eleven tensors
+ * bit-identical to a run that never set it.  host_args is a HOST pointer to a struct of device
  * pointers; n_items = workgroups to launch (= roots unless the work-item lists are given);
  * max_children = largest child count in the tree (<= 8). */
 int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max_children, int phases,

@@ -41,6 +41,8 @@ static_assert(IT_BLOCK == UB_BLOCK && IT_BLOCK == SD_BLOCK, "shared helpers assu
 
 constexpr uint8_t NODE_SHOWDOWN = 1;  // river showdown leaf: value from the showdown evaluator
 constexpr uint8_t NODE_DONE = 2;      // terminal node: excluded from the zero-sum shift
+constexpr uint8_t NODE_PARENT = 4;    // the row has children
+constexpr uint8_t NODE_LEAF_EVAL = 8; // childless row whose ranges feed a leaf evaluation (showdown, leaf network)
 // vectors card-summed per batch: what the LDS union holds next to the showdown buffers, and
 // never less than one family (parent + children)
 template <int MAXC>
@@ -75,6 +77,7 @@ struct IterArgs {
   float* latest;
   float* values_avg;
   float* scratch;                    // [total,H] workspace
+  const float* reach_avg_prev;       // [total,2,H] or null: reach_avg as the previous iteration left it (see PHASE_LEAN)
   // iteration-dependent scalars in device memory
   const float* fscal;    // t_alpha_num, t_beta_num, t_alpha_den, t_beta_den, mix_old, mix_new, mix_total, mix_inv_total
   const int64_t* iscal;  // t, apply_dcfr, cfr_plus, avg_policy_copy, enforce_zero_sum, update_avg_values, cfr_avg, linear
@@ -95,6 +98,19 @@ struct IterArgs {
 // simply follow each other (PHASE_12 | PHASE_3).  With a root split into work items it takes four
 // launches: every item sweep 1, tree tops sweep 2, subtrees sweeps 2 + 3, tree tops sweep 3.
 constexpr int PHASE_12 = 1, PHASE_3 = 2, PHASE_1 = 4, PHASE_2 = 8;
+// PHASE_LEAN: an iteration whose result nobody looks at before the next one runs.  Sweep 2 then stores
+// only the rows a later sweep or the next iteration reads: reach and reach_avg of rows that have
+// children (a family reads its parent's), beliefs of rows that have children or feed a leaf evaluation
+// (from beliefs_avg instead under cfr_avg), beliefs_avg only where cfr_avg or the zero-sum shift read
+// it.  Every skipped row is a pure function of rows that are kept, so one ordinary iteration afterwards
+// leaves all eleven tensors exactly as a run of ordinary iterations would.
+//
+// reach_avg_prev (independent of PHASE_LEAN): the average-policy mix of a family needs its parent's
+// reach_avg[actor] from BEFORE this iteration, which the family above has overwritten by then.  With
+// reach_avg_prev null, sweep 1 stashes that row in `scratch`; with two reach_avg buffers that the host
+// swaps from iteration to iteration, sweep 2 reads it from the buffer of the previous iteration
+// instead: one row read per parent in place of a read, a write and a re-read.
+constexpr int PHASE_LEAN = 16;
 
 constexpr int IT_VSTRIDE = P2_H + 2;  // floats between vectors staged in LDS
 constexpr int IT_RED = 20;            // block-reduction slots: 2 + 2 * 8 children, rounded up
@@ -245,9 +261,12 @@ __device__ __forceinline__ float2 mul2(float2 a, float2 b) { return make_float2(
 // row of its first child, the child count and who acts.  The kernel broadcasts an entry with a lane
 // read, so walking the tree costs no dependent global loads per family; every wave keeps its own copy.
 struct FamWin {
-  int p, first, ca;   // ca = child count | actor << 8
+  int p, first, ca;   // ca = child count | actor << 8 | kinds << 16
   int base;           // list position (relative to the item's first family) held by lane 0
 };
+// KINDS: also collect, per child k, bit 2k = the child has children, bit 2k + 1 = its ranges feed a
+// leaf evaluation (what a lean iteration decides its stores by).
+template <int MAXC, bool KINDS>
 __device__ __forceinline__ void fam_load(FamWin& F, const IterArgs& A, int64_t pp0, int nfam, int base) {
   const int l = base + (int)(threadIdx.x & 63);
   F.base = base;
@@ -256,12 +275,20 @@ __device__ __forceinline__ void fam_load(FamWin& F, const IterArgs& A, int64_t p
   F.ca = 0;
   if (l < nfam) {
     const int64_t p = A.root_parents[pp0 + l];
+    const int64_t first = A.child_offsets[p];
+    const int cnt = (int)A.child_count[p];
     F.p = (int)p;
-    F.first = (int)A.child_offsets[p];
-    F.ca = (int)A.child_count[p] | ((int)A.to_act[p] << 8);
+    F.first = (int)first;
+    int kinds = 0;
+    if (KINDS) {
+#pragma unroll
+      for (int k = 0; k < MAXC; ++k)
+        if (k < cnt) kinds |= (((int)A.node_flags[first + k] >> 2) & 3) << (2 * k);
+    }
+    F.ca = cnt | ((int)A.to_act[p] << 8) | (kinds << 16);
   }
 }
-struct Fam { int64_t p, first; int cnt, actor; };
+struct Fam { int64_t p, first; int cnt, actor, kinds; };
 __device__ __forceinline__ Fam fam_get(const FamWin& F, int i) {
   const int s = i - F.base;
   Fam f;
@@ -269,7 +296,8 @@ __device__ __forceinline__ Fam fam_get(const FamWin& F, int i) {
   f.first = __builtin_amdgcn_readlane(F.first, s);
   const int ca = __builtin_amdgcn_readlane(F.ca, s);
   f.cnt = ca & 0xFF;
-  f.actor = ca >> 8;
+  f.actor = (ca >> 8) & 0xFF;
+  f.kinds = (int)((unsigned)ca >> 16);
   return f;
 }
 
@@ -297,7 +325,7 @@ __device__ __forceinline__ float readlane_f(float v, int s) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), s));
 }
 
-template <int MAXC>
+template <int MAXC, bool LEAN, bool ALT>
 __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iteration_kernel(IterArgs A) {
   constexpr int IT_CHUNK = ItChunk<MAXC>::value;
   // how many rows are requested together: parents staged for the card sums, children of a family in
@@ -313,7 +341,8 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
   Lane ln;
   lane_init(ln);
   FamWin F;
-  fam_load(F, A, pp0, nfam, 0);
+  fam_load<MAXC, LEAN>(F, A, pp0, nfam, 0);
+  constexpr bool stash = !ALT;   // the pre-update reach_avg of a parent goes through `scratch`
 
   const float f_an = A.fscal[0], f_bn = A.fscal[1], f_ad = A.fscal[2], f_bd = A.fscal[3];
   const float mix_old = A.fscal[4], mix_new = A.fscal[5], mix_total = A.fscal[6], mix_inv = A.fscal[7];
@@ -351,7 +380,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
     }
     for (int i0 = 0; i0 < nfam; i0 += IT_CHUNK) {
       const int nch = (nfam - i0) < IT_CHUNK ? (nfam - i0) : IT_CHUNK;
-      if (i0 < F.base || i0 + nch > F.base + 64) fam_load(F, A, pp0, nfam, i0);
+      if (i0 < F.base || i0 + nch > F.base + 64) fam_load<MAXC, LEAN>(F, A, pp0, nfam, i0);
       // opponent beliefs of every parent of the chunk: requested together, staged together,
       // card-summed in one pass
       PROF_BEGIN(t_c1);
@@ -365,7 +394,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
             const int u = u0 + uu < nch ? u0 + uu : nch - 1;
             const Fam f = fam_get(F, i0 + u);
             ld(bo[uu], leaf_beliefs, f.p * 2 + (1 - f.actor), ln);
-            ld(ra[uu], A.reach_avg, f.p * 2 + f.actor, ln);  // the mix in sweep 2 needs the pre-update value
+            if (stash) ld(ra[uu], A.reach_avg, f.p * 2 + f.actor, ln);  // the mix in sweep 2 needs the pre-update value
           }
 #pragma unroll
           for (int uu = 0; uu < SB; ++uu) {
@@ -373,7 +402,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
             if (u < IT_CHUNK && u < nch) {
               const Fam f = fam_get(F, i0 + u);
               to_lds(L.u.vecs[u], bo[uu], ln);
-              st(A.scratch, f.p, ra[uu], ln);
+              if (stash) st(A.scratch, f.p, ra[uu], ln);
             }
           }
         }
@@ -477,12 +506,19 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
     // next to a family's children they wait there (in this lane's own slots: no barrier) instead of
     // occupying 24 registers through the whole sweep.
     constexpr bool ROOT_LDS = IT_CHUNK - MAXC >= 4;
+    // Which rows a lean iteration keeps (see PHASE_LEAN): beliefs_avg everywhere for the zero-sum shift
+    // of sweep 3, under cfr_avg where they take the place of beliefs, else nowhere.
+    const bool bavg_all = !LEAN || enforce_zs, bavg_any = bavg_all || cfr_avg;
     float2 rbk[2][IT_PPT], rbak[2][IT_PPT], ap[IT_PPT];
     uchar2 am[IT_PPT];
     ld(rbk[0], A.beliefs, r * 2, ln);
     ld(rbk[1], A.beliefs, r * 2 + 1, ln);
-    ld(rbak[0], A.beliefs_avg, r * 2, ln);
-    ld(rbak[1], A.beliefs_avg, r * 2 + 1, ln);
+    if (bavg_any) {
+      ld(rbak[0], A.beliefs_avg, r * 2, ln);
+      ld(rbak[1], A.beliefs_avg, r * 2 + 1, ln);
+    } else {
+      IT_FOR(j) rbak[0][j] = rbak[1][j] = make_float2(0.f, 0.f);
+    }
     ld(ap, A.allowed_prob, r, ln);
     {
       const uchar2* m2 = reinterpret_cast<const uchar2*>(A.allowed + r * P2_H);
@@ -496,17 +532,23 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
       to_lds(L.u.vecs[MAXC + 3], rbak[1], ln);
     }
     for (int i = 0; i < nfam; ++i) {
-      if (i < F.base || i >= F.base + 64) fam_load(F, A, pp0, nfam, i);
+      if (i < F.base || i >= F.base + 64) fam_load<MAXC, LEAN>(F, A, pp0, nfam, i);
       const Fam f = fam_get(F, i);
       const int64_t p = f.p, first = f.first;
       const int cnt = f.cnt, actor = f.actor;
+      // per child: does it have children (its reach rows are read by its own family), do its ranges feed
+      // a leaf evaluation; an ordinary iteration keeps every row
+      const int has_children = LEAN ? f.kinds & 0x5555 : 0x5555, leaf_eval = LEAN ? (f.kinds >> 1) & 0x5555 : 0x5555;
+      const int keep_b = cfr_avg ? has_children : (has_children | leaf_eval);
+      const int keep_ba = bavg_all ? 0x5555 : (cfr_avg ? (has_children | leaf_eval) : 0);
       float2 rn[2][IT_PPT], ran[2][IT_PPT], ra_old[IT_PPT];
       float2 cur[MAXC][IT_PPT], pav[MAXC][IT_PPT];
       ld(rn[0], A.reach, p * 2, ln);
       ld(rn[1], A.reach, p * 2 + 1, ln);
       ld(ran[0], A.reach_avg, p * 2, ln);
       ld(ran[1], A.reach_avg, p * 2 + 1, ln);
-      ld(ra_old, A.scratch, p, ln);
+      if (stash) ld(ra_old, A.scratch, p, ln);
+      else ld(ra_old, A.reach_avg_prev, p * 2 + actor, ln);
 #pragma unroll
       for (int k = 0; k < MAXC; ++k)
         if (k < cnt) ld(cur[k], A.policy, first + k, ln);
@@ -614,9 +656,14 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
           float2 xa[IT_PPT];
           from_lds(xa, L.u.vecs[k], ln);
           IT_FOR(j) {
-            const float2 vb = mul2(rb_act[j], xa[j]), vba = mul2(rba_act[j], pav[k][j]);
+            const float2 vb = mul2(rb_act[j], xa[j]);
             sums[2 + 2 * k] += vb.x + vb.y;
-            sums[3 + 2 * k] += vba.x + vba.y;
+          }
+          if (keep_ba) {
+            IT_FOR(j) {
+              const float2 vba = mul2(rba_act[j], pav[k][j]);
+              sums[3 + 2 * k] += vba.x + vba.y;
+            }
           }
         }
       }
@@ -627,7 +674,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
       // reach
 #pragma unroll
       for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
+        if (k < cnt && ((has_children >> (2 * k)) & 1)) {
           const int64_t c = first + k;
           float2 xa[IT_PPT];
           from_lds(xa, L.u.vecs[k], ln);
@@ -638,7 +685,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
       // reach_avg
 #pragma unroll
       for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
+        if (k < cnt && ((has_children >> (2 * k)) & 1)) {
           const int64_t c = first + k;
           if (actor == 0) { st(A.reach_avg, c * 2, pav[k], ln); st(A.reach_avg, c * 2 + 1, ran_opp, ln); }
           else { st(A.reach_avg, c * 2, ran_opp, ln); st(A.reach_avg, c * 2 + 1, pav[k], ln); }
@@ -653,7 +700,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
       }
 #pragma unroll
       for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
+        if (k < cnt && ((keep_b >> (2 * k)) & 1)) {
           const int64_t c = first + k;
           const float sa = sums[2 + 2 * k];
           float2 o[IT_PPT], xa[IT_PPT];
@@ -669,7 +716,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
       // beliefs_avg
 #pragma unroll
       for (int k = 0; k < MAXC; ++k) {
-        if (k < cnt) {
+        if (k < cnt && ((keep_ba >> (2 * k)) & 1)) {
           const int64_t c = first + k;
           const float saa = sums[3 + 2 * k];
           float2 oa[IT_PPT];
@@ -736,7 +783,7 @@ __global__ __launch_bounds__(IT_BLOCK, ItTune<MAXC>::min_waves) void cfr_iterati
 
     // ---------------- sweep 3b: backup, bottom-up ----------------
     for (int i = nfam - 1; i >= 0; --i) {
-      if (i < F.base || i >= F.base + 64) fam_load(F, A, pp0, nfam, i > 63 ? i - 63 : 0);
+      if (i < F.base || i >= F.base + 64) fam_load<MAXC, LEAN>(F, A, pp0, nfam, i > 63 ? i - 63 : 0);
       const Fam f = fam_get(F, i);
       const int64_t p = f.p, first = f.first;
       const int cnt = f.cnt, actor = f.actor;
@@ -934,8 +981,8 @@ int p2hip_upload_floats(float* dst, const float* host_values, int n, void* strea
 
 int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max_children, int phases,
                         void* stream) {
-  if (!host_args || n_items < 0 || n_items > 0x7FFFFFFF || max_children < 1 || max_children > 8 || (phases & ~15) ||
-      phases == 0)
+  if (!host_args || n_items < 0 || n_items > 0x7FFFFFFF || max_children < 1 || max_children > 8 || (phases & ~31) ||
+      (phases & 15) == 0)
     return P2_EINVAL;
   if (n_items == 0) return 0;
   const P2HipIterArgs& h = *host_args;
@@ -944,11 +991,15 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max
                             h.root_showdown_offsets,  // root_showdown_nodes is empty (null) without showdown rows
                             h.t_sample, h.allowed, h.allowed_prob, h.potential, h.scale, h.policy, h.policy_avg,
                             h.policy_sample, h.cum, h.wsum, h.beliefs, h.beliefs_avg, h.reach, h.reach_avg, h.latest,
-                            h.values_avg, h.scratch, h.fscal, h.iscal};
+                            h.values_avg, h.fscal, h.iscal};
   for (const void* p : required)
     if (!p) return P2_EINVAL;
+  // the pre-update reach_avg of a parent travels through `scratch` unless the previous iteration's buffer is given
+  if (!h.scratch && !h.reach_avg_prev) return P2_EINVAL;
+  if (h.reach_avg_prev == h.reach_avg) return P2_EINVAL;
   const void* rows[] = {h.allowed_prob, h.policy, h.policy_avg, h.policy_sample, h.cum, h.wsum, h.beliefs,
-                        h.beliefs_avg, h.reach, h.reach_avg, h.latest, h.values_avg, h.scratch, h.tables};
+                        h.beliefs_avg, h.reach, h.reach_avg, h.latest, h.values_avg, h.scratch, h.tables,
+                        h.reach_avg_prev};
   for (const void* p : rows)
     if (!p2_aligned8(p)) return P2_EINVAL;
   p2::IterArgs a;
@@ -961,12 +1012,24 @@ int p2hip_cfr_iteration(const P2HipIterArgs* host_args, int64_t n_items, int max
   a.beliefs_avg = h.beliefs_avg; a.reach = h.reach; a.reach_avg = h.reach_avg; a.latest = h.latest;
   a.values_avg = h.values_avg; a.scratch = h.scratch; a.fscal = h.fscal; a.iscal = h.iscal;
   a.item_root = h.item_root; a.item_top = h.item_top;
-  a.phases = phases;
+  a.reach_avg_prev = h.reach_avg_prev;
+  a.phases = phases & 15;
+  const bool lean = (phases & p2::PHASE_LEAN) != 0;
   const dim3 grid((unsigned)n_items), block(p2::IT_BLOCK);
-  if (max_children <= 5)
-    hipLaunchKernelGGL((p2::cfr_iteration_kernel<5>), grid, block, 0, (hipStream_t)stream, a);
-  else
-    hipLaunchKernelGGL((p2::cfr_iteration_kernel<8>), grid, block, 0, (hipStream_t)stream, a);
+  const bool alt = h.reach_avg_prev != nullptr;
+#define P2_ITER_LAUNCH(MAXC, LEAN, ALT) \
+  hipLaunchKernelGGL((p2::cfr_iteration_kernel<MAXC, LEAN, ALT>), grid, block, 0, (hipStream_t)stream, a)
+#define P2_ITER_MODES(MAXC)                                  \
+  do {                                                       \
+    if (lean && alt) P2_ITER_LAUNCH(MAXC, true, true);       \
+    else if (lean) P2_ITER_LAUNCH(MAXC, true, false);        \
+    else if (alt) P2_ITER_LAUNCH(MAXC, false, true);         \
+    else P2_ITER_LAUNCH(MAXC, false, false);                 \
+  } while (0)
+  if (max_children <= 5) P2_ITER_MODES(5);
+  else P2_ITER_MODES(8);
+#undef P2_ITER_MODES
+#undef P2_ITER_LAUNCH
   P2_LAUNCH_CHECK();
   return 0;
 }

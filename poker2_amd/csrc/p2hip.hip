@@ -14,7 +14,7 @@
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.
-int p2hip_abi_version(void) { return 3; }
+int p2hip_abi_version(void) { return 4; }
 // Number of visible HIP devices (0 when there is none); never throws.
 int p2hip_device_count(void) {
   int n = 0;

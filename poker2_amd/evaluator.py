@@ -50,7 +50,7 @@ STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumul
                "regret_weight_sums", "self_reach", "self_reach_avg", "beliefs", "beliefs_avg",
                "latest_values", "values_avg")
 
-_NODE_SHOWDOWN, _NODE_DONE = 1, 2
+_NODE_SHOWDOWN, _NODE_DONE, _NODE_PARENT, _NODE_LEAF_EVAL = 1, 2, 4, 8
 
 
 class _IterArgs(ctypes.Structure):
@@ -59,12 +59,15 @@ class _IterArgs(ctypes.Structure):
         "root_showdown_offsets", "root_showdown_nodes", "t_sample",
         "allowed", "allowed_prob", "tables", "potential", "scale", "policy", "policy_avg", "policy_sample", "cum",
         "wsum", "beliefs", "beliefs_avg", "reach", "reach_avg", "latest", "values_avg", "scratch", "fscal", "iscal",
-        "item_root", "item_top")]
+        "item_root", "item_top", "reach_avg_prev")]
 
 
 # Sweeps a launch of the iteration kernel runs (include/p2hip.h): 1 = regrets + reach/beliefs, 2 = values,
 # 4 = regrets alone, 8 = reach/beliefs alone.
 _PHASE_12, _PHASE_3, _PHASE_1, _PHASE_2 = 1, 2, 4, 8
+# Lean launch (include/p2hip.h): the reach / belief part stores only the rows that the rest of the
+# iteration or the next iteration reads.  ``evaluate_cfr`` runs every iteration but its last that way.
+_PHASE_LEAN = 16
 # One workgroup per root fills the chip (256 CUs x 3 resident workgroups) from 768 roots on.  Below
 # SPLIT_ROOTS_BELOW roots each root's tree is cut at level SPLIT_CUT_LEVEL into work items (the top of
 # the tree, and one subtree per node of that level) that get a workgroup each.  Measured on the
@@ -131,7 +134,7 @@ class HipSparseCFREvaluator:
     def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
                  compile_model: bool = True, fused_iteration: bool = True,
                  max_raises: int | None = None, tree_builder: str = "device",
-                 split_small_batches: bool | None = None) -> None:
+                 split_small_batches: bool | None = None, lean_search: bool = True) -> None:
         self.model = model
         self.device = torch.device(device)
         self.cfg = cfg
@@ -176,6 +179,10 @@ class HipSparseCFREvaluator:
         self.tree_builder = tree_builder     # both give identical trees; 'host' is the numpy builder
         # None: split each root into several workgroups when there are too few roots to fill the chip
         self.split_small_batches = split_small_batches
+        # evaluate_cfr runs every iteration but the last one lean (rows nobody reads before the next
+        # iteration are not stored) and lets reach_avg alternate between two buffers; the final state is
+        # bit-identical either way.  False: every iteration as ``cfr_iteration`` runs it.
+        self.lean_search = bool(lean_search)
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -191,9 +198,8 @@ class HipSparseCFREvaluator:
         self._iscal = torch.zeros(8, dtype=torch.int64, device=self.device)
         self._fscal_host = (ctypes.c_float * 8)()
         self._iscal_host = (ctypes.c_int64 * 8)()
-        self._iter_args = None
-        self._iter_args_tiers = None
-        self._iter_args_regret = None
+        self._iter_bundles: dict = {}
+        self._reach_avg_alt = None
         self._chance_helper = None
         self.subgame_serial = 0
 
@@ -309,6 +315,12 @@ class HipSparseCFREvaluator:
         flags = np.zeros(T, dtype=np.uint8)
         flags[tree.showdown_mask] |= _NODE_SHOWDOWN
         flags[st["done"]] |= _NODE_DONE
+        # what a lean iteration decides its stores by: rows with children, and childless rows whose ranges
+        # are read by a leaf evaluation (the showdown kernel, or the leaf network when there is one)
+        flags[tree.child_count > 0] |= _NODE_PARENT
+        flags[tree.showdown_mask & (tree.child_count == 0)] |= _NODE_LEAF_EVAL
+        if self.model is not None:
+            flags[model_mask & (tree.child_count == 0)] |= _NODE_LEAF_EVAL
         self._node_flags = self._t(flags)
         def per_root(mask):
             """Rows selected by ``mask`` grouped by root (ascending inside a root) + offsets [N+1]."""
@@ -323,9 +335,8 @@ class HipSparseCFREvaluator:
         self._root_showdown_nodes, self._root_showdown_offsets = per_root(tree.showdown_mask)
         self._max_children = int(tree.child_count.max()) if T else 1
         self._has_model_leaves = bool(model_mask.any())
-        self._iter_args = None
-        self._iter_args_tiers = None
-        self._iter_args_regret = None
+        self._iter_bundles = {}
+        self._reach_avg_alt = None
         split = self.split_small_batches
         if split is None:
             split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
@@ -670,7 +681,7 @@ class HipSparseCFREvaluator:
             self.latest_values[self.showdown_indices] = self._showdown_value_both(beliefs[self.showdown_indices])
 
     # ------------------------------------------------------------------ iteration
-    def _build_iter_args(self, items=None) -> _IterArgs:
+    def _build_iter_args(self, items=None, reach_avg=None, reach_avg_prev=None) -> _IterArgs:
         a = _IterArgs()
         p = _lib.ptr
         a.child_offsets, a.child_count, a.to_act = p(self.child_offsets), p(self.child_count), p(self.env.to_act)
@@ -683,7 +694,9 @@ class HipSparseCFREvaluator:
         a.policy, a.policy_avg, a.policy_sample = p(self.policy_probs), p(self.policy_probs_avg), p(self.policy_probs_sample)
         a.cum, a.wsum = p(self.cumulative_regrets), p(self.regret_weight_sums)
         a.beliefs, a.beliefs_avg = p(self.beliefs), p(self.beliefs_avg)
-        a.reach, a.reach_avg = p(self.self_reach), p(self.self_reach_avg)
+        a.reach = p(self.self_reach)
+        a.reach_avg = p(self.self_reach_avg if reach_avg is None else reach_avg)
+        a.reach_avg_prev = p(reach_avg_prev)
         a.latest, a.values_avg, a.scratch = p(self.latest_values), p(self.values_avg), p(self._scratch)
         a.fscal, a.iscal = p(self._fscal), p(self._iscal)
         it = items if items is not None else (self._items if self._items is not None else self._root_items)
@@ -700,47 +713,78 @@ class HipSparseCFREvaluator:
                                                _lib.stream_ptr())
         _lib.check(code, "p2hip_cfr_iteration")
 
-    def _launch_iteration(self, phases: int) -> None:
-        """``phases``: 1 = regrets, policy, reach, beliefs; 2 = leaf values and backup; 3 = both."""
-        if self._iter_args is None:
-            self._iter_args = self._build_iter_args()
-            if self._items is not None:
-                self._iter_args_regret = (self._build_iter_args(self._items_regret), sum(self._items_regret.tiers))
-                # one argument block per tier: the same lists entered behind the items of the tiers before
-                self._iter_args_tiers, first = [], 0
-                for count in self._items.tiers:
-                    tier = self._build_iter_args()
-                    tier.root_parent_offsets += 8 * first
-                    tier.root_showdown_offsets += 8 * first
-                    tier.item_root += 8 * first
-                    tier.item_top += first
-                    self._iter_args_tiers.append((tier, count))
-                    first += count
-        if self._items is None:
-            self._launch_items(self._iter_args, self.root_nodes, phases)
-            return
-        tiers = self._iter_args_tiers
-        if phases & _PHASE_12:
-            self._launch_items(*self._iter_args_regret, _PHASE_1)                 # regrets of every family, all items at once
-            for args, count in tiers[:-1]:
-                self._launch_items(args, count, _PHASE_2)                           # upper tiers, top-down
-        args, count = tiers[-1]
-        self._launch_items(args, count, (_PHASE_2 if phases & _PHASE_12 else 0) | (phases & _PHASE_3))
-        if phases & _PHASE_3:
-            for args, count in reversed(tiers[:-1]):
-                self._launch_items(args, count, _PHASE_3)                           # the upper tiers' backup comes last
+    def _other_reach_avg(self) -> torch.Tensor:
+        """The second reach_avg buffer of the alternating scheme (allocated on first use; root rows 1)."""
+        if self._reach_avg_alt is None or self._reach_avg_alt.shape != self.self_reach_avg.shape:
+            self._reach_avg_alt = torch.empty_like(self.self_reach_avg)
+            self._reach_avg_alt[:self.root_nodes] = 1.0
+        return self._reach_avg_alt
 
-    def cfr_iteration(self, t: int) -> None:
-        """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533)."""
+    def _iter_bundle(self, alternate: bool) -> SimpleNamespace:
+        """Argument blocks of the iteration kernel for the tensor ``self_reach_avg`` names right now:
+        updated in place (the old row saved in the scratch tensor), or — ``alternate`` — read as the
+        previous iteration's and the new one written to the other buffer."""
+        key = (self.self_reach_avg.data_ptr(), bool(alternate))
+        b = self._iter_bundles.get(key)
+        if b is not None:
+            return b
+        if alternate:
+            kw = dict(reach_avg=self._other_reach_avg(), reach_avg_prev=self.self_reach_avg)
+        else:
+            kw = {}
+        b = SimpleNamespace(main=self._build_iter_args(**kw), regret=None, tiers=None)
+        if self._items is not None:
+            b.regret = (self._build_iter_args(self._items_regret, **kw), sum(self._items_regret.tiers))
+            # one argument block per tier: the same lists entered behind the items of the tiers before
+            b.tiers, first = [], 0
+            for count in self._items.tiers:
+                tier = self._build_iter_args(**kw)
+                tier.root_parent_offsets += 8 * first
+                tier.root_showdown_offsets += 8 * first
+                tier.item_root += 8 * first
+                tier.item_top += first
+                b.tiers.append((tier, count))
+                first += count
+        self._iter_bundles[key] = b
+        return b
+
+    def _launch_iteration(self, phases: int, lean: bool = False, alternate: bool = False) -> None:
+        """``phases``: 1 = regrets, policy, reach, beliefs; 2 = leaf values and backup; 3 = both.
+        ``lean``: store only what is read again (include/p2hip.h).  ``alternate``: write reach_avg into
+        the other of two buffers; ``self_reach_avg`` names the new one when this returns."""
+        alternate = alternate and bool(phases & _PHASE_12)
+        b = self._iter_bundle(alternate)
+        mode = _PHASE_LEAN if lean else 0
+        if self._items is None:
+            self._launch_items(b.main, self.root_nodes, phases | mode)
+        else:
+            tiers = b.tiers
+            if phases & _PHASE_12:
+                self._launch_items(*b.regret, _PHASE_1 | mode)                      # regrets of every family, all items at once
+                for args, count in tiers[:-1]:
+                    self._launch_items(args, count, _PHASE_2 | mode)                # upper tiers, top-down
+            args, count = tiers[-1]
+            self._launch_items(args, count, (_PHASE_2 if phases & _PHASE_12 else 0) | (phases & _PHASE_3) | mode)
+            if phases & _PHASE_3:
+                for args, count in reversed(tiers[:-1]):
+                    self._launch_items(args, count, _PHASE_3 | mode)                # the upper tiers' backup comes last
+        if alternate:
+            self.self_reach_avg, self._reach_avg_alt = self._reach_avg_alt, self.self_reach_avg
+
+    def cfr_iteration(self, t: int, *, lean: bool = False, alternate_reach_avg: bool = False) -> None:
+        """One CFR iteration (fused_sparse_cfr_evaluator.py:478-533).  The two keywords are for
+        ``evaluate_cfr`` (one-kernel path only): ``lean`` leaves rows unwritten that nothing reads before
+        the next iteration rewrites them — the state is complete again after one ordinary iteration —
+        and ``alternate_reach_avg`` rebinds ``self_reach_avg`` to the other of two buffers."""
         if not self._skip_t_scalars_update:
             self.prepare_replay(t)
         if self.fused_iteration:
             if self._has_model_leaves and self.model is not None:
-                self._launch_iteration(1)
+                self._launch_iteration(1, lean, alternate_reach_avg)
                 self.set_leaf_values(t, showdown=False)
-                self._launch_iteration(2)
+                self._launch_iteration(2, lean)
             else:
-                self._launch_iteration(3)
+                self._launch_iteration(3, lean, alternate_reach_avg)
             return
         F.fused_sample_snapshot_(self.policy_probs_sample, self.policy_probs, self.t_sample, self._t_scalars.t_tensor)
         regrets = self.compute_instantaneous_regrets(self.latest_values)
@@ -850,11 +894,22 @@ class HipSparseCFREvaluator:
         """cfr_evaluator.py:1497-1528 (statistics recording left out): the search, then the
         leaves from which the next searches continue."""
         self.prepare_search()
-        for t in range(self.warm_start_iterations, self.cfr_iterations):
-            self.cfr_iteration(t)
+        self.run_search_iterations()
         if self.use_final_policy_values:
             self.update_average_values_final()
         return self.sample_leaves(training_mode)
+
+    def run_search_iterations(self) -> None:
+        """The loop of ``evaluate_cfr`` (cfr_evaluator.py:1516-1519).  Nobody looks at the state between
+        its iterations, so with ``lean_search`` all but the last run lean, and reach_avg alternates
+        between two buffers over an even number of iterations — it ends in the tensor it started in (an
+        odd first iteration updates it in place).  The state afterwards is bit-identical to a loop of
+        plain ``cfr_iteration`` calls."""
+        ts = range(self.warm_start_iterations, self.cfr_iterations)
+        lean = self.lean_search and self.fused_iteration
+        for k, t in enumerate(ts):
+            self.cfr_iteration(t, lean=lean and k + 1 < len(ts),
+                               alternate_reach_avg=lean and not (len(ts) % 2 == 1 and k == 0))
 
     def update_average_values_final(self) -> None:
         """cfr_evaluator.py:1276-1292."""

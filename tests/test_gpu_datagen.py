@@ -355,6 +355,11 @@ def test_policy_targets_kernel_matches_pull_back_on_a_deep_tree():
     rows = torch.from_numpy(rng.permutation(top)[: top // 2]).to(DEV)             # any rows, any order, leaves too
     got = ev._policy_targets(rows).cpu().numpy()
     assert np.array_equal(got, exp[rows.cpu().numpy()])                             # a gather: exact
+    # Childless rows of the last level: their child_offsets entry equals the row count, so a slot without
+    # a child must request a row of the table itself (the node's own), never `child_offsets[r]`.
+    last = torch.arange(ev.total_nodes - 3, ev.total_nodes, device=DEV)
+    assert int(ev.child_count[last].sum()) == 0 and int(ev.child_offsets[last].max()) >= ev.total_nodes - 1
+    assert not bool(ev._policy_targets(last).any())
     # the same into a buffer that is only 8-byte aligned (rows as float2 instead of whole 128-byte lines),
     # with guard floats on both sides
     from poker2_amd import _lib
