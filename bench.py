@@ -1,14 +1,22 @@
 """Headline benchmark: fused DCFR iteration on river subgames, one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--roots B] [--tree depth2|raise1|raise2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--roots B] [--tree raise3|raise1|raise2|depth2] [--mode search|plain]
 
 A step is ONE CFR iteration over a batch of B seeded synthetic river subgames (random
 5-card boards, Dirichlet(0.5) ranges with board-blocked combos removed, pot 200, stacks
-800/800, bet bins {0.5, 1.0}, discounted CFR alpha 1.5 / beta 0 / gamma 2).  All inputs are
-resident in HBM before the timed region.  Prints ONE JSON line:
+800/800 = stack/pot 4, bet bins {0.5, 1.0} + all-in, at most three raises: 105 nodes per root, every
+leaf a fold or a showdown; discounted CFR alpha 1.5 / beta 0 / gamma 2).  All inputs are
+resident in HBM before the timed region.  The steps run the way a search runs them
+(``HipSparseCFREvaluator.run_search_iterations``: every iteration but a search's last leaves rows
+unwritten that nothing reads before the next iteration rewrites them, and reach_avg alternates
+between two buffers; the final state of a search is bit-identical either way); ``--mode plain`` times
+the iteration that writes all eleven tensors in full, as ``cfr_iteration(t)`` does.  Both are in the line.
+Prints ONE JSON line:
   value        subgame-iterations per second (iterations/s x subgames)
-  roofline     algorithmic bytes of the iteration kernel / its mean launch time (HIP events
-               on the launch stream) against the 8 TB/s HBM peak
+  roofline     canonical algorithmic bytes of an iteration (29 vectors per node) / the mean time of
+               the iteration's launches (HIP events on the launch stream) against the 8 TB/s HBM
+               peak; `traffic` = HBM bytes the launches really move (rocprofv3 counters), with the
+               fraction of peak on those bytes beside it
   cpu_baseline the numpy oracle (a CPU restatement of the reference's torch path) timed on
                this box's host cores on a small sample of the same workload
   extra        showdown evaluations/s (B=4096 boards), 7-card hands ranked/s (2^20 hands), each with
@@ -39,9 +47,12 @@ TREES = {"depth2": (2, None), "raise1": (16, 1), "raise2": (16, 2), "raise3": (1
 # program: counters need the profiler, so these are constants taken from the summary file named
 # below, one per workload that has a counter run; None elsewhere.  (read bytes, written bytes)
 TRAFFIC_SOURCE = "profiles/cfr_iteration_kernel_river.hbm_counters.txt"
-MEASURED_TRAFFIC_BYTES = {("depth2", 4096): (5.873e9, 6.723e9), ("raise3", 4096): (33.58e9, 35.94e9),
-                          ("raise3", 1024): (8.395e9, 8.986e9),
-                          ("depth2", 1024): (1.455e9, 1.681e9)}
+MEASURED_TRAFFIC_BYTES = {("raise3", 4096, "plain"): (33.67e9, 35.77e9), ("raise3", 4096, "search"): (32.30e9, 23.12e9),
+                          ("depth2", 4096, "plain"): (5.87e9, 6.69e9), ("depth2", 4096, "search"): (5.68e9, 3.82e9),
+                          ("raise1", 4096, "plain"): (6.60e9, 7.02e9), ("raise1", 4096, "search"): (6.35e9, 4.61e9),
+                          ("raise3", 1024, "plain"): (8.42e9, 8.94e9), ("raise3", 1024, "search"): (8.08e9, 5.78e9)}
+# how the iterations of a search run (all but its last) / how cfr_iteration(t) runs one
+MODES = {"search": dict(lean=True, alternate_reach_avg=True), "plain": {}}
 
 
 def cpu_model() -> str:
@@ -149,7 +160,7 @@ def flat_stream_rate(pairs: int = 1 << 26, reps: int = 5) -> dict:
     return out
 
 
-def side_metrics() -> dict:
+def side_metrics(skip=()) -> dict:
     """Showdown evaluations/s (B=4096 public states) and hands ranked/s (2^20 hands)."""
     import torch
     from poker2_amd import rules_hip
@@ -193,34 +204,41 @@ def side_metrics() -> dict:
     # the batch the reference's own settings search at a time (num_envs: 192), on the three-raise tree: few roots
     # are cut into work items that get a workgroup each
     small, _, _ = make_evaluator(192, "raise3", 42, iterations=64)
-    for t in range(1, 6):
-        small.cfr_iteration(t)
-    ev0.record()
-    for t in range(6, 6 + reps):
-        small.cfr_iteration(t)
-    ev1.record()
-    torch.cuda.synchronize()
-    ms = ev0.elapsed_time(ev1) / reps
-    out["iteration_ms_B192_three_raise_tree"] = ms
-    out["subgame_iterations_per_s_B192"] = 192 / (ms * 1e-3)
-    out["algorithmic_GBps_B192"] = BYTES_PER_NODE_ITER * small.total_nodes / (ms * 1e-3) / 1e9
-    del small
-    # the same iteration kernel on the other river workloads (HIP events around 20 launches each)
-    others = []
-    for roots, tree in ((4096, "raise3"), (4096, "raise1"), (1024, "depth2"), (1024, "raise3")):
-        ev, _, _ = make_evaluator(roots, tree, 42, iterations=64)
-        for t in range(5):
-            ev.cfr_iteration(t)
-        torch.cuda.synchronize()
+    for mode, kw in MODES.items():
+        for t in range(1, 6):
+            small.cfr_iteration(t, **kw)
         ev0.record()
-        for t in range(5, 25):
-            ev.cfr_iteration(t)
+        for t in range(6, 6 + reps):
+            small.cfr_iteration(t, **kw)
         ev1.record()
         torch.cuda.synchronize()
-        ms = ev0.elapsed_time(ev1) / 20
-        gbs = BYTES_PER_NODE_ITER * ev.total_nodes / (ms * 1e-3) / 1e9
-        others.append({"roots": roots, "tree": tree, "nodes_per_root": ev.total_nodes // roots, "iteration_ms": ms,
-                       "algorithmic_GBps": gbs, "frac": gbs / HBM_PEAK_GBS})
+        ms = ev0.elapsed_time(ev1) / reps
+        tag = "" if mode == "search" else "_plain"
+        out["iteration_ms_B192_three_raise_tree" + tag] = ms
+        out["subgame_iterations_per_s_B192" + tag] = 192 / (ms * 1e-3)
+        out["algorithmic_GBps_B192" + tag] = BYTES_PER_NODE_ITER * small.total_nodes / (ms * 1e-3) / 1e9
+    del small
+    # the same iteration kernel on the other river workloads (HIP events around 20 iterations each), as a search
+    # runs them and in full
+    others = []
+    for roots, tree in ((4096, "depth2"), (4096, "raise1"), (1024, "depth2"), (1024, "raise3")):
+        if (roots, tree) == tuple(skip):
+            continue
+        ev, _, _ = make_evaluator(roots, tree, 42, iterations=64)
+        row = {"roots": roots, "tree": tree, "nodes_per_root": ev.total_nodes // roots}
+        for mode, kw in MODES.items():
+            for t in range(6):
+                ev.cfr_iteration(t, **kw)
+            torch.cuda.synchronize()
+            ev0.record()
+            for t in range(6, 26):
+                ev.cfr_iteration(t, **kw)
+            ev1.record()
+            torch.cuda.synchronize()
+            ms = ev0.elapsed_time(ev1) / 20
+            gbs = BYTES_PER_NODE_ITER * ev.total_nodes / (ms * 1e-3) / 1e9
+            row[mode] = {"iteration_ms": ms, "algorithmic_GBps": gbs, "frac": gbs / HBM_PEAK_GBS}
+        others.append(row)
         del ev
         torch.cuda.empty_cache()
     out["iteration_other_workloads"] = others
@@ -268,7 +286,9 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=60)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--roots", type=int, default=4096)
-    ap.add_argument("--tree", choices=sorted(TREES), default="depth2")
+    ap.add_argument("--tree", choices=sorted(TREES), default="raise3")
+    ap.add_argument("--mode", choices=sorted(MODES), default="search",
+                    help="search: the iterations as a search runs all but its last; plain: every tensor written in full")
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
@@ -294,30 +314,39 @@ def main() -> None:
         del src, dst
     ev, _, _ = make_evaluator(args.roots, args.tree, args.seed, iterations=args.warmup + args.steps + 1)
     nodes_per_root = ev.total_nodes // ev.root_nodes
-    t = 0
-    for _ in range(args.warmup):
-        ev.cfr_iteration(t)
-        t += 1
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ev._skip_t_scalars_update = True
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        ev.prepare_replay(t)          # tiny scalar-upload kernel, outside the kernel timing
-        starts[k].record()
-        ev.cfr_iteration(t)           # ONE launch of the iteration kernel (four with fewer than 400 roots)
-        ends[k].record()
-        t += 1
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = float(np.mean([s.elapsed_time(e) for s, e in zip(starts, ends)]))
-    ms_per_step = wall * 1e3 / args.steps
+    launches = 1 if ev._items is None else 2 * len(ev._items.tiers)
+
+    def timed(mode: str, steps: int, warmup: int, t: int):
+        """Mean time of an iteration's launches (HIP events on the launch stream) and the wall clock per step."""
+        kw = MODES[mode]
+        for _ in range(warmup):
+            ev.cfr_iteration(t, **kw)
+            t += 1
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+        ev._skip_t_scalars_update = True
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(steps):
+            ev.prepare_replay(t)          # tiny scalar-upload kernel, outside the kernel timing
+            starts[k].record()
+            ev.cfr_iteration(t, **kw)     # the iteration's launches: one per root-sized tree, four over work items
+            ends[k].record()
+            t += 1
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ev._skip_t_scalars_update = False
+        return float(np.mean([s.elapsed_time(e) for s, e in zip(starts, ends)])), wall * 1e3 / steps, t
+
+    kernel_ms, ms_per_step, t_next = timed(args.mode, args.steps, args.warmup, 0)
+    other_mode = "plain" if args.mode == "search" else "search"
+    other_kernel_ms, other_ms_per_step, _ = timed(other_mode, min(args.steps, 20), 3, t_next)
     value = args.roots / (ms_per_step * 1e-3)
     algo_bytes = BYTES_PER_NODE_ITER * ev.total_nodes
     achieved = algo_bytes / (kernel_ms * 1e-3) / 1e9
     assert torch.isfinite(ev.values_avg).all()
-    rw = MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots))
+    rw = MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots, args.mode))
+    rw_other = MEASURED_TRAFFIC_BYTES.get((args.tree, args.roots, other_mode))
     traffic = float(sum(rw)) if rw else None
     total_nodes = ev.total_nodes
     del ev
@@ -325,6 +354,9 @@ def main() -> None:
 
     flat = flat_stream_rate()
     moved = traffic if traffic else algo_bytes
+    mode_text = {"search": "iterations as a search runs all but its last (rows nothing reads before the next iteration "
+                           "rewrites them are not stored; reach_avg alternates between two buffers)",
+                 "plain": "every iteration writes all eleven tensors in full, as cfr_iteration(t) does"}
     result = {
         "metric": "river CFR iters/sec x subgames",
         "value": value,
@@ -339,9 +371,11 @@ def main() -> None:
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"fused DCFR iteration, river subgames, B={args.roots}, tree={args.tree} "
-                               f"({nodes_per_root} nodes/root, bins 0.5/1.0, pot 200, stacks 800)",
+                               f"({nodes_per_root} nodes/root, bins 0.5/1.0 + all-in, pot 200, stacks 800)",
                    "roots": args.roots, "nodes_per_root": nodes_per_root, "total_nodes": total_nodes,
-                   "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0"},
+                   "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0",
+                   "mode": args.mode, "mode_note": mode_text[args.mode],
+                   "launches_per_iteration": launches},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic,
@@ -352,6 +386,15 @@ def main() -> None:
                      "frac_of_peak_on_measured_traffic": (traffic / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if traffic else None,
                      "kernel": "cfr_iteration_kernel", "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": algo_bytes,
+                     "algorithmic_bytes_note": "29 vectors of 1326 floats per node and iteration (17 written, 12 read), "
+                                               "the canonical count of one iteration whatever the mode",
+                     "other_mode": {"mode": other_mode, "mode_note": mode_text[other_mode], "kernel_ms": other_kernel_ms,
+                                    "ms_per_step": other_ms_per_step,
+                                    "value": args.roots / (other_ms_per_step * 1e-3),
+                                    "frac": algo_bytes / (other_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                    "traffic": float(sum(rw_other)) if rw_other else None,
+                                    "frac_of_peak_on_measured_traffic":
+                                        (sum(rw_other) / (other_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if rw_other else None},
                      "flat_stream_same_mix_GBps": flat,
                      "flat_stream_note": "p2hip_stream_probe: 5 arrays read + 7 written, 512 MiB each, ordinary and "
                                          "non-temporal accesses, measured by this run after the timed region; the "
@@ -362,7 +405,7 @@ def main() -> None:
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.tree, args.seed)
     if not args.no_extra:
-        result["extra"] = side_metrics()
+        result["extra"] = side_metrics(skip=(args.roots, args.tree))
         if not args.no_cpu_baseline:
             result["extra"]["cpu"] = cpu_side_baselines()
     print(json.dumps(result))
