@@ -9,13 +9,15 @@
  *   - straight flush reports the HIGHEST window, straight the LOWEST;
  *   - window w (0..9) covers ranks w-1..w+3, ace doubling as rank -1.
  * Pinned by tests/golden/ranker_golden.npz (written by running the reference's
- * rules.py), the exhaustive C(52,7) category histogram and std_eval.c.
+ * rules.py), tests/golden/ranker_cards_golden.npz (written by running the reference's
+ * card-id kernel on hands that repeat a card), the exhaustive C(52,7) category
+ * histogram and std_eval.c.
  */
 #include <stdint.h>
 #include <string.h>
 
 typedef struct {
-    uint32_t suit[4];   /* 13-bit rank masks per suit (distinct cards only) */
+    uint32_t suit[4];   /* rank masks per suit; card-id input: the SUM of the cards' rank bits (a repeated card carries) */
     uint32_t quads, trips, pairs, singles; /* rank masks by multiplicity */
 } p2o_hand;
 
@@ -46,7 +48,7 @@ static inline int32_t pack6(int f0, int f1, int f2, int f3, int f4, int f5) {
 /* flush_first != 0: flush suit = first suit with >= 5 ranks (rules_triton.py);
  * flush_first == 0: suit with the most ranks, first on ties (rules.py:217-219) */
 static int32_t score(p2o_hand h, int flush_first) {
-    uint32_t rank_mask = h.suit[0] | h.suit[1] | h.suit[2] | h.suit[3];
+    uint32_t rank_mask = h.quads | h.trips | h.pairs | h.singles;
     uint32_t zeros = 0x1FFFu & ~(h.quads | h.trips | h.pairs | h.singles);
     int idx[5], cnt[5];
     for (int i = 0; i < 5; ++i) idx[i] = pop_top(&h, &zeros, &cnt[i]);
@@ -94,8 +96,9 @@ void p2o_rank_planes(const uint8_t *planes, int64_t n, int32_t *out) {
     }
 }
 
-/* cards: [n, k] int16 ids (negative = absent); semantics of rules_triton.py:
- * repeated ids count twice for multiplicities, once for suit masks */
+/* cards: [n, k] int16 ids (negative = absent); semantics of rules_triton.py:414-446: a repeated id
+ * counts again for the multiplicities, and a suit mask is the integer sum of its cards' rank bits
+ * (tl.sum, :421-425), so a repeated card carries into the next higher bit of its suit's mask */
 void p2o_rank_cards(const int16_t *cards, int64_t n, int k, int32_t *out) {
     for (int64_t i = 0; i < n; ++i) {
         p2o_hand h; memset(&h, 0, sizeof(h));
@@ -104,7 +107,7 @@ void p2o_rank_cards(const int16_t *cards, int64_t n, int k, int32_t *out) {
             int c = cards[i * k + j];
             if (c < 0) continue;
             uint32_t bit = 1u << (c % 13);
-            h.suit[c / 13] |= bit;
+            h.suit[c / 13] += bit;
             p4 |= p3 & bit; p3 |= p2 & bit; p2 |= seen & bit; seen |= bit;
         }
         h.quads = p4; h.trips = p3 & ~p4; h.pairs = p2 & ~p3; h.singles = seen & ~p2;

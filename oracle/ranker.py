@@ -7,8 +7,9 @@ Follows ``src/p2/env/rules.py``:
   rank_hands          <- rank_hands                 :66-133
 and ``src/p2/env/rules_triton.py``:
   rank_cards          <- _evaluate_cards_player     :414-581  (card-id input;
-                         a duplicated card id counts twice towards
-                         pairs/trips/quads but once towards flushes)
+                         a duplicated card id counts again towards
+                         pairs/trips/quads, and carries into the next bit of
+                         its suit's mask, which is a SUM of rank bits)
   rank_hands_cards    <- rank_hands_triton          :120-148
 
 Card encoding: card = suit*13 + rank, rank 0..12 = 2..A.
@@ -33,11 +34,12 @@ rank-order lists of the reference's ``tests/test_rules.py`` (restated as data in
 histogram equalling the textbook table; (4) agreement with an independent
 best-5-of-7 evaluator (``oracle/std_eval.c``) outside the quirk classes.
 
-PARITY UNPINNED: what ``rank_cards`` returns for a hand that repeats a card id.  That rule is read
-off ``_evaluate_cards_player``; the kernels of ``rules_triton.py`` hold PTX inline assembly
-(:364-385), so they run neither under Triton's CPU interpreter nor on this hardware, and
-``rules.py`` takes card planes, which cannot express a repeated card.  No caller on the search
-path passes one (boards and hole cards are distinct).
+(5) for hands that REPEAT a card id (which ``rules.py`` cannot express and ``rank_hands_triton``
+produces for every combo that holds a board card): ``tests/golden/ranker_cards_golden.npz`` -- scores
+written by running the reference's own card-id kernel under Triton's CPU interpreter on 316 such
+hands and on all 1326 combos of three boards (``tests/golden/gen_ranker_cards_golden.py``; its two
+PTX leaf helpers, highest set bit and population count, are replaced there by plain integer code of
+the same meaning).
 """
 from __future__ import annotations
 
@@ -151,10 +153,25 @@ def compare_planes(ab: np.ndarray) -> np.ndarray:
     return np.clip(packed[:, 0] - packed[:, 1], -1, 1).astype(np.int32)
 
 
+def _popcount(x: np.ndarray) -> np.ndarray:
+    x = x.astype(np.int64)
+    return sum((x >> k) & 1 for k in range(32)).astype(np.int32)
+
+
+def _highest_bit(x: np.ndarray) -> np.ndarray:
+    """Index of the most significant set bit, 0 for an empty mask (``_pop_highest_rank``,
+    rules_triton.py:364-375: ``bfind`` clamped at 0)."""
+    x = x.astype(np.int64)
+    return sum(((x >> k) != 0).astype(np.int32) for k in range(1, 32)).astype(np.int32)
+
+
 def rank_cards(cards: np.ndarray) -> np.ndarray:
-    """Packed int32 score from card ids [..., K] where a repeated id counts
-    twice towards rank multiplicities but once towards suit masks; the flush
-    suit is the first suit holding >= 5 distinct ranks."""
+    """Packed int32 score from card ids [..., K] as ``_evaluate_cards_player`` scores them
+    (rules_triton.py:414-581): a repeated id counts again towards the rank multiplicities
+    (:431-440), and each suit's mask is the integer SUM of its cards' rank bits (``tl.sum``,
+    :421-425), so a repeated card carries into the next higher bit of its suit's mask; straights
+    come from the ranks present; the flush suit is the first suit whose mask has >= 5 bits, its
+    five kickers the mask's highest bits; straight-flush windows look at bits 0..12 of the masks."""
     cards = np.asarray(cards, dtype=np.int64)
     lead = cards.shape[:-1]
     flat = cards.reshape(-1, cards.shape[-1])
@@ -163,10 +180,10 @@ def rank_cards(cards: np.ndarray) -> np.ndarray:
     ranks = flat % 13
     suits = flat // 13
     counts = np.zeros((n, 13), dtype=np.int32)
-    suit_planes = np.zeros((n, 4, 13), dtype=np.int32)
+    suit_mask = np.zeros((n, 4), dtype=np.int64)
     for j in range(flat.shape[1]):
         np.add.at(counts, (rows, ranks[:, j]), 1)
-        suit_planes[rows, suits[:, j], ranks[:, j]] = 1
+        np.add.at(suit_mask, (rows, suits[:, j]), np.int64(1) << ranks[:, j])
     counts = np.minimum(counts, 4)
 
     key = (counts << 8) | _RANKS
@@ -182,6 +199,7 @@ def rank_cards(cards: np.ndarray) -> np.ndarray:
             val = val | (np.asarray(x, dtype=np.int32) << (4 * (4 - i)))
         return val
 
+    suit_planes = ((suit_mask[:, :, None] >> _RANKS.astype(np.int64)) & 1).astype(np.int32)   # bits 0..12 of the masks
     ext = np.concatenate([suit_planes[..., 12:13], suit_planes], axis=-1)
     sf_win = _sliding5(ext).max(axis=-2) == 5
     has_sf = sf_win.any(axis=-1)
@@ -192,19 +210,15 @@ def rank_cards(cards: np.ndarray) -> np.ndarray:
     straight = conv.max(axis=-1) == 5
     low = conv.argmax(axis=-1)
 
-    suit_cnt = suit_planes.sum(axis=-1)
-    has5 = suit_cnt >= 5
+    has5 = _popcount(suit_mask) >= 5
     flush = has5.any(axis=-1)
     fsuit = np.where(flush, has5.argmax(axis=-1), 3)
-    suit_cards = suit_planes[rows, fsuit]
-    remaining = suit_cards.copy()
+    remaining = suit_mask[rows, fsuit]
     fl = []
     for _ in range(5):
-        # highest remaining rank of the flush suit, 0 once the suit is exhausted
-        any_left = remaining.any(axis=-1)
-        best = np.where(any_left, 12 - remaining[:, ::-1].argmax(axis=-1), 0)
-        fl.append(best.astype(np.int32))
-        remaining[rows[any_left], best[any_left]] = 0
+        best = _highest_bit(remaining)
+        fl.append(best)
+        remaining = remaining & ~(np.int64(1) << best.astype(np.int64))
 
     z = np.zeros(n, dtype=np.int32)
     w = np.where

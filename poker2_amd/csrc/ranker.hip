@@ -13,7 +13,8 @@
 namespace p2 {
 
 struct Hand {
-  uint32_t s0, s1, s2, s3;               // suit masks (distinct cards)
+  uint32_t s0, s1, s2, s3;               // suit masks: bit r = the suit holds rank r (card-id input: the SUM of the
+                                         // cards' rank bits, so a repeated card carries into the next bit)
   uint32_t quads, trips, pairs, singles;  // rank masks by multiplicity
 };
 
@@ -59,8 +60,11 @@ __host__ __device__ __forceinline__ Hand hand_from_suits(uint32_t s0, uint32_t s
   return h;
 }
 
-// Card-id insertion: a repeated id counts again towards the multiplicities but
-// not towards the suit masks (rules_triton.py:431-446).
+// Card-id insertion as the reference's card kernel does it: a repeated id counts again towards the
+// multiplicities (rules_triton.py:431-440), and a suit's mask is the integer SUM of its cards' rank
+// bits (:421-425), so the second copy of a card carries into the next higher bit instead of being
+// absorbed.  Hands of distinct cards — everything the search looks at — are not affected; the combos
+// that hold a board card in rank_hands_triton (:120-148) are, and score as the reference scores them.
 struct CardAcc {
   uint32_t s0 = 0, s1 = 0, s2 = 0, s3 = 0, seen = 0, p2 = 0, p3 = 0, p4 = 0;
   __host__ __device__ __forceinline__ void add(int card) {
@@ -69,10 +73,10 @@ struct CardAcc {
     const uint32_t suit = c / 13u;
     const uint32_t rank = c - suit * 13u;
     const uint32_t bit = 1u << rank;
-    s0 |= (suit == 0) ? bit : 0u;
-    s1 |= (suit == 1) ? bit : 0u;
-    s2 |= (suit == 2) ? bit : 0u;
-    s3 |= (suit == 3) ? bit : 0u;
+    s0 += (suit == 0) ? bit : 0u;
+    s1 += (suit == 1) ? bit : 0u;
+    s2 += (suit == 2) ? bit : 0u;
+    s3 += (suit == 3) ? bit : 0u;
     p4 |= p3 & bit;
     p3 |= p2 & bit;
     p2 |= seen & bit;
@@ -98,7 +102,7 @@ __host__ __device__ __forceinline__ int32_t imax(int32_t a, int32_t b) { return 
 // otherwise the suit with the most ranks, first on ties (rules.py:215-219).
 // The two agree whenever at most 9 cards are present.
 __host__ __device__ __forceinline__ int32_t score_hand(Hand h, bool flush_first) {
-  const uint32_t rank_mask = h.s0 | h.s1 | h.s2 | h.s3;
+  const uint32_t rank_mask = h.quads | h.trips | h.pairs | h.singles;   // ranks present, whatever the suit masks carry
   uint32_t q = h.quads, t = h.trips, p = h.pairs, s = h.singles;
   uint32_t z = 0x1FFFu & ~(q | t | p | s);
   int idx[5], cnt[5];

@@ -135,8 +135,13 @@ class HipSparseCFREvaluator:
                  compile_model: bool = True, fused_iteration: bool = True,
                  max_raises: int | None = None, tree_builder: str = "device",
                  split_small_batches: bool | None = None, lean_search: bool = True) -> None:
-        self.model = model
         self.device = torch.device(device)
+        if model is not None and not hasattr(model, "leaf_values"):
+            # the reference hands its network over as is (cfr_evaluator.py:306-322, 1025-1047): its
+            # leaf rule and initial policy are NetworkLeafModel's
+            from .leaf_models import NetworkLeafModel
+            model = NetworkLeafModel(model, self.device)
+        self.model = model
         self.cfg = cfg
         if self.device.type != "cuda":
             raise ValueError("HipSparseCFREvaluator requires a GPU device.")

@@ -63,20 +63,56 @@ class RangeBoardMLP(torch.nn.Module):
         return SimpleNamespace(hand_values=x.view(-1, 2, NUM_HANDS))
 
 
+def _accepts_keyword(fn, name: str) -> bool:
+    """Whether ``fn`` can be called with the keyword ``name``."""
+    import inspect
+    try:
+        params = inspect.signature(fn).parameters.values()
+    except (TypeError, ValueError):
+        return False
+    return any(p.name == name or p.kind is inspect.Parameter.VAR_KEYWORD for p in params)
+
+
 class NetworkLeafModel:
     """The reference's own leaf rule (src/p2/search/cfr_evaluator.py:1024-1040): the network sees
     the encoded features of every leaf that is not terminal; a leaf that closed a betting round
     is encoded with the board before the next deal, so the network itself stands for the chance
-    node."""
+    node.  The initial policy comes from the same network's ``policy_logits`` (:305-329), uniform over
+    the legal actions if it has none.  ``HipSparseCFREvaluator`` wraps a bare network — anything
+    without ``leaf_values`` — in this class itself, so the reference's constructor call
+    ``Evaluator(model, device, cfg)`` (src/p2/rl/cfr_trainer.py:194-207) carries over unchanged."""
 
-    def __init__(self, net, device, *, enforce_zero_sum: bool = False,
+    def __init__(self, net, device, *, enforce_zero_sum: bool | None = None,
                  autocast_dtype: torch.dtype | None = None) -> None:
         self.net = net
         self.device = torch.device(device)
-        self.enforce_zero_sum = enforce_zero_sum
+        # the reference reads the flag off the network (cfr_evaluator.py:970)
+        self.enforce_zero_sum = bool(getattr(net, "enforce_zero_sum", False)) if enforce_zero_sum is None \
+            else bool(enforce_zero_sum)
         self.autocast_dtype = autocast_dtype
         self._cached_for = None
         self._cached = None
+        call = net.forward if isinstance(net, torch.nn.Module) else net
+        self._policy_keyword = _accepts_keyword(call, "include_policy")
+
+    def _run(self, feats, include_policy: bool):
+        if hasattr(self.net, "eval"):
+            self.net.eval()
+        kw = {"include_policy": include_policy} if self._policy_keyword else {}
+        if self.autocast_dtype is not None:
+            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                return self.net(feats, **kw)
+        return self.net(feats, **kw)
+
+    @torch.no_grad()
+    def policy_logits(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
+        """[K, 1326, actions] logits of the network at node rows ``rows`` (cfr_evaluator.py:305-319);
+        zeros — a uniform policy over the legal actions — for a network without a policy head."""
+        feats = ev.feature_encoder.encode(beliefs, indices=rows)
+        logits = getattr(self._run(feats, True), "policy_logits", None) if self._policy_keyword else None
+        if logits is None:
+            return torch.zeros(rows.numel(), NUM_HANDS, ev.num_actions, dtype=torch.float32, device=self.device)
+        return logits.reshape(rows.numel(), NUM_HANDS, ev.num_actions)
 
     @torch.no_grad()
     def leaf_values(self, beliefs: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:
@@ -90,15 +126,7 @@ class NetworkLeafModel:
         c = self._cached
         feats = MLPFeatures(context=c.context, street=c.street, to_act=c.to_act, board=c.board,
                             beliefs=beliefs.reshape(beliefs.shape[0], -1))
-        if hasattr(self.net, "eval"):
-            self.net.eval()
-        if self.autocast_dtype is not None:
-            with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
-                hv = self.net(feats).hand_values
-        else:
-            hv = self.net(feats).hand_values
-        return hv
-
+        return self._run(feats, False).hand_values
 
     @torch.no_grad()
     def leaf_values_from_nodes(self, table: torch.Tensor, rows: torch.Tensor, ev) -> torch.Tensor:

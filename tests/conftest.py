@@ -15,3 +15,18 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """What the element-wise comparisons of tests/parity.py measured in this session (exempt shares and
+    worst entries per tensor): printed, and kept in gpurun_out/ when that folder exists."""
+    from tests import parity
+    if not parity.MEASURED:
+        return
+    text = parity.measured_report()
+    terminalreporter.write_sep("-", "parity: measured over this session")
+    terminalreporter.write_line(text)
+    out = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out):
+        with open(os.path.join(out, "parity_measured.txt"), "w") as f:
+            f.write(text + "\n")

@@ -267,12 +267,12 @@ def test_turn_subgame_with_chance_leaves_matches_oracle(K, fused, streets):
     # measured on the oracle (tests/parity.py: twins that start a few roundings away); every other
     # entry is held to NETWORK_FACTOR x (1e-5 relative + parity.ATOL).
     pack = PAR.OracleWithTwins(orc, seed=12, n_twins=2, amp=3e-7)
-    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what="after the preparation step: ")
+    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, kind="free running, network at the leaves", what="after the preparation step: ")
     assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3     # the network's values are not trivial
     for t in range(iters):
         ev.cfr_iteration(t)
         pack.cfr_iteration(t)
-        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what=f"t={t}: ")
+        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, kind="free running, network at the leaves", what=f"t={t}: ")
         print(f"t={t}: worst determined entry {PAR.worst_of(rep):.2f} tolerances, largest exempt share "
               f"{max(r['exempt'] for r in rep.values()):.1e}")
 
@@ -532,12 +532,12 @@ def test_preflop_subgame_with_flop_leaves_matches_oracle(K):
                          t_sample_roots=np.full(n, -1, dtype=np.int64), fused_variant=True)
     orc.prepare()
     pack = PAR.OracleWithTwins(orc, seed=14, n_twins=2, amp=3e-7)      # as in the turn test above
-    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what="after the preparation step: ")
+    PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, kind="free running, network at the leaves", what="after the preparation step: ")
     assert np.abs(orc.latest_values[orc.model_indices]).max() > 1e-3
     for t in range(iters):
         ev.cfr_iteration(t)
         pack.cfr_iteration(t)
-        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, max_exempt=0.35, what=f"t={t}: ")
+        rep = PAR.compare_free(PAR.state_of(ev), pack, factor=NETWORK_FACTOR, kind="free running, network at the leaves", what=f"t={t}: ")
         print(f"t={t}: worst determined entry {PAR.worst_of(rep):.2f} tolerances, largest exempt share "
               f"{max(r['exempt'] for r in rep.values()):.1e}")
 

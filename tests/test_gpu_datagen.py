@@ -737,3 +737,71 @@ class _WithoutNodes:
 
     def leaf_values(self, beliefs, rows, ev):
         return self.inner.leaf_values(beliefs, rows, ev)
+
+
+def test_evaluator_takes_a_bare_network_like_the_reference():
+    """``Evaluator(model, device, cfg)`` with the network itself, as the reference's trainer builds it
+    (src/p2/rl/cfr_trainer.py:194-207): the constructor wraps it in NetworkLeafModel — same search as with
+    the explicit wrapper, ``enforce_zero_sum`` read off the network (cfr_evaluator.py:970) — and a network
+    with a policy head, called as the reference calls it (``model(features, include_policy=True)``,
+    :305-329), sets the initial policy."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.leaf_models import NetworkLeafModel, RangeBoardMLP
+    from poker2_amd.tree import RootStates
+    from tests.helpers import random_boards, random_ranges
+    rng = np.random.default_rng(18)
+    n = 4
+    boards = random_boards(rng, n, 5)
+    boards[:2, 4] = -1
+    beliefs = torch.from_numpy(random_ranges(rng, boards))
+    roots = RootStates.at_round_start(np.where(boards[:, 4] < 0, 2, 3), np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards)
+
+    def search(model):
+        ev = HipSparseCFREvaluator(model, torch.device(DEV), river_dcfr_config(n, iterations=4, depth=16), max_raises=1)
+        ev.initialize_subgame(roots, np.arange(n), beliefs)
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
+        first_policy = ev.policy_probs.clone()
+        ev.run_search_iterations()
+        return ev, first_policy
+
+    net = RangeBoardMLP(hidden=64, layers=2, seed=3).to(DEV)
+    bare, _ = search(net)
+    wrapped, _ = search(NetworkLeafModel(net, DEV))
+    assert isinstance(bare.model, NetworkLeafModel) and bare.model.net is net and not bare.enforce_zero_sum
+    assert bare.model_indices.numel() > 0
+    for k in OCFR.OracleCFR.STATE_NAMES:
+        assert torch.equal(getattr(bare, k), getattr(wrapped, k)), k
+
+    class PolicyNet(torch.nn.Module):
+        enforce_zero_sum = True
+
+        def __init__(self, actions):
+            super().__init__()
+            self.actions = actions
+            self.calls = []
+
+        def forward(self, f, include_policy=True):
+            self.calls.append(include_policy)
+            k = f.beliefs.shape[0]
+            hv = 0.01 * (f.beliefs.view(k, 2, H).flip(1) * H - 1.0)
+            logits = None
+            if include_policy:
+                hand = torch.arange(H, device=f.beliefs.device, dtype=torch.float32)
+                act = torch.arange(self.actions, device=f.beliefs.device, dtype=torch.float32)
+                logits = torch.sin(0.01 * hand[None, :, None] * (1.0 + act[None, None, :])) + f.context[:, 1, None, None]
+            return SimpleNamespace(hand_values=hv, policy_logits=logits)
+
+    pnet = PolicyNet(5)
+    ev, first_policy = search(pnet)
+    assert ev.enforce_zero_sum and True in pnet.calls and False in pnet.calls
+    # root level by hand: softmax over the legal actions of the network's logits, one child row per action
+    hand = torch.arange(H, device=DEV, dtype=torch.float32)
+    act = torch.arange(5, device=DEV, dtype=torch.float32)
+    feats = ev.feature_encoder.encode(ev.beliefs, indices=torch.arange(n, device=DEV))
+    logits = torch.sin(0.01 * hand[None, :, None] * (1.0 + act[None, None, :])) + feats.context[:, 1, None, None]
+    probs = torch.softmax(logits.masked_fill(~ev.legal_mask[:n, None, :], float("-inf")), dim=-1)
+    lo, hi = ev.depth_offsets[1], ev.depth_offsets[2]
+    want = probs[ev.parent_index[lo:hi], :, ev.action_from_parent[lo:hi]]
+    assert torch.allclose(first_policy[lo:hi], want, rtol=1e-6, atol=1e-7)
+    assert float((first_policy[lo:hi] - 1.0 / ev.child_count[ev.parent_index[lo:hi]][:, None]).abs().max()) > 0.05

@@ -68,7 +68,7 @@ def make_pair(n_roots, depth, max_raises, seed, fused, iters, cfr_type="discount
 # — a quotient of differences of nearly equal values — amplifies them; that the iteration ITSELF
 # is right to well within the tolerance is what the one-step comparison shows.
 FREE_FACTOR_FIRST, FREE_FACTOR_LATER = 3.0, 5.0
-P999_FACTOR = 15.0        # largest seen: 9.9 (depth-3 tree, sixth iteration)
+P999_FACTOR = 14.0        # largest seen: 9.9 (depth-3 tree, sixth iteration)
 
 
 class Lockstep:
@@ -464,7 +464,7 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
                                select=lambda s, arr: arr[..., cols],
                                also_exempt=None if blocked is None else
                                (lambda s: blocked if got[s].ndim == 2 else blocked[:, None, :]),
-                               max_exempt=1.0 if blocked is not None else 0.25, what=f"{name} {tag}: ")
+                               what=f"{name} {tag}: ", kind=f"reference fixture, {fixture} class")
         worst[tag] = max(r["worst_over_tol"] for r in rep.values())
         # and over EVERY compared entry, exempt or not: all but one in a thousand within P999_FACTOR tolerances
         p999[tag] = max(r["p999_over_tol"] for r in rep.values())
@@ -492,12 +492,14 @@ def test_product_matches_reference_vectors(golden_dir, name, fused, fixture):
 def test_one_kernel_and_per_op_paths_agree_on_random_subgames(seed):
     """Seeded sweep over tree shapes the other tests do not reach: random chips (including short
     stacks that remove bets and leave one- and two-child families), one to five bet fractions (up
-    to 8 children), depths 1-5, raise caps, CFR variants.  The two product paths share no kernel
-    for the iteration itself, so their agreement checks each against the other."""
+    to 6 children: the kernel instantiation for more than five), depths 1-5, raise caps, CFR variants.
+    Each of the two product paths — they share no kernel for the iteration itself — is held to the
+    oracle, every iteration one step from the path's own state, at 1 x the tolerance of tests/parity.py."""
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.fused_cfr_hip import CFRType
     from poker2_amd.tree import RootStates
+    from oracle.ranker import rank_hands_cards
     rng = np.random.default_rng(1000 + seed)
     n = int(rng.integers(1, 6))
     all_bins = [0.25, 0.5, 0.75, 1.0, 2.0]
@@ -510,11 +512,11 @@ def test_one_kernel_and_per_op_paths_agree_on_random_subgames(seed):
     pot = rng.integers(40, 900, n)
     stacks = rng.integers(30, 2500, (n, 2))
     roots = RootStates.at_round_start(3, pot, stacks, boards, button=rng.integers(0, 2, n), bb=int(rng.choice([10, 100])))
-    evs = []
+    delay = int(rng.integers(0, 3))
+    what = f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type}"
+    t_sample_roots = np.full(n, 1, dtype=np.int64)
     for fused in (True, False):
-        cfg = river_dcfr_config(n, iterations=20, depth=depth, dcfr_delay=int(rng.integers(0, 3)) if fused else 0)
-        if not fused:
-            cfg.search.dcfr_plus_delay = evs[0].dcfr_delay
+        cfg = river_dcfr_config(n, iterations=20, depth=depth, dcfr_delay=delay)
         cfg.search.cfr_type = CFRType[cfr_type]
         cfg.search.cfr_plus = bool(seed % 2)
         cfg.search.cfr_avg = bool((seed // 2) % 2)
@@ -523,17 +525,17 @@ def test_one_kernel_and_per_op_paths_agree_on_random_subgames(seed):
                                    tree_builder="device" if fused else "host")
         ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
         ev.prepare_search(t_sample=torch.full((ev.total_nodes,), 1, dtype=torch.long))
-        evs.append(ev)
-    a, b = evs
-    assert a.total_nodes == b.total_nodes
-    for t in range(4):
-        a.cfr_iteration(t)
-        b.cfr_iteration(t)
-    for name in OCFR.OracleCFR.STATE_NAMES:
-        x, y = getattr(a, name), getattr(b, name)
-        bad = ((x - y).abs() > 2e-5 + 2e-4 * y.abs()).float().mean().item()
-        assert bad <= 1e-3, f"seed {seed} bins {bins} depth {depth} raises {max_raises} {cfr_type}: {name} {bad:.2e} " \
-                            f"max {float((x - y).abs().max()):.3e}"
+        orc = OCFR.OracleCFR(tree_as_dict(ev.tree), boards, beliefs, cfr_type=cfr_type, dcfr_alpha=1.5, dcfr_beta=0.0,
+                             dcfr_gamma=2.0, dcfr_delay=delay, cfr_plus=cfg.search.cfr_plus, cfr_avg=cfg.search.cfr_avg,
+                             cfr_iterations=20, t_sample_roots=t_sample_roots, ranker=rank_hands_cards,
+                             fused_variant=True)
+        orc.prepare()
+        for t in range(4):
+            PAR.set_state(orc, PAR.state_of(ev))
+            ev.cfr_iteration(t)
+            orc.cfr_iteration(t)
+            PAR.compare_step(PAR.state_of(ev), orc,
+                             what=f"{what}, {'one kernel' if fused else 'per operation'}, t={t}: ")
 
 
 # ---- full benchmark sizes: properties that do not depend on the size -------------------------

@@ -140,3 +140,23 @@ def test_comparison_vector_and_scalar_compare(K, golden_dir):
     t, s, cs = stats.slice_for_player(torch.tensor([0, 1, 1, 0, 1], device="cuda"))
     assert t.shape == (5, 1326) and s.shape == (5,) and cs.shape == (5, 52)
     torch.testing.assert_close(cs.sum(-1), 2 * s, rtol=1e-5, atol=1e-5)
+
+
+def test_repeated_card_ids_score_like_the_reference_kernel(K, golden_dir):
+    """Hands that repeat a card id, scored by the reference's own card-id kernel run under Triton's CPU
+    interpreter (tests/golden/gen_ranker_cards_golden.py): the repeat counts again towards pairs / trips /
+    quads and carries into the next bit of its suit's mask (rules_triton.py:421-440).  Every input dtype,
+    the comparison entry point, and ``rank_hands_triton`` on three boards — where every combo that holds a
+    board card is such a hand — bit for bit."""
+    g = np.load(os.path.join(golden_dir, "ranker_cards_golden.npz"))
+    hands, scores = g["hands"], g["scores"]
+    assert int((np.sort(hands, axis=1)[:, 1:] == np.sort(hands, axis=1)[:, :-1]).any(axis=1).sum()) >= 300
+    for dt in (torch.int8, torch.int16, torch.int32, torch.int64):
+        out = K.rank_7_cards_single_batch_triton(torch.from_numpy(hands.astype(np.int64)).to(dt).cuda())
+        assert np.array_equal(out.cpu().numpy(), scores), dt
+    pairs = np.stack([hands[:-1], hands[1:]], axis=1).astype(np.int16)
+    exp = np.sign(scores[:-1].astype(np.int64) - scores[1:]).astype(np.int32)
+    assert np.array_equal(K.compare_7_cards_single_batch_triton(torch.from_numpy(pairs).cuda()).cpu().numpy(), exp)
+    for dt in (torch.int8, torch.int64):
+        p, o = K.rank_hands_triton(torch.from_numpy(g["boards"]).to(dt).cuda())
+        assert np.array_equal(p.cpu().numpy(), g["hand_ranks"]) and np.array_equal(o.cpu().numpy(), g["sorted_indices"])

@@ -138,3 +138,18 @@ def test_numpy_and_c_oracles_agree_on_random_and_short_hands():
     short = cards.copy()
     short[:, 4:] = -1
     assert np.array_equal(R.rank_planes(R.cards_to_planes(short)), RC.rank_cards(short))
+
+
+def test_repeated_card_ids_match_the_reference_kernel(golden_dir):
+    """tests/golden/ranker_cards_golden.npz: scores of the reference's own card-id kernel (run under
+    Triton's CPU interpreter) for 316 hands that repeat a card id, 64 that do not, and all 1326 combos of
+    three boards through the card assembly of rank_hands_triton.  Both oracles, bit for bit."""
+    g = np.load(os.path.join(golden_dir, "ranker_cards_golden.npz"))
+    hands, scores = g["hands"], g["scores"]
+    assert np.array_equal(R.rank_cards(hands.astype(np.int64)), scores)
+    assert np.array_equal(RC.rank_cards(hands), scores)
+    packed, order = R.rank_hands_cards(g["boards"])
+    assert np.array_equal(packed, g["hand_ranks"]) and np.array_equal(order, g["sorted_indices"])
+    # the carry is what the fixture is about: with the suit masks OR-ed instead of summed a third of the hands differ
+    sorted_h = np.sort(hands, axis=1)
+    assert int((sorted_h[:, 1:] == sorted_h[:, :-1]).any(axis=1).sum()) == 316

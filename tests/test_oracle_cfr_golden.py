@@ -72,7 +72,8 @@ def check(pack, golden, name, tag, factor):
     got = {s: getattr(o, s) for s in names}
     expected = {s: golden[f"{name}/{tag}/{s}"] for s in names}
     return PAR.compare_free(got, pack, factor=factor, names=names, expected=expected,
-                            select=lambda s, arr: arr[..., cols], what=f"{name} {tag}: ")
+                            select=lambda s, arr: arr[..., cols], what=f"{name} {tag}: ",
+                            kind="oracle against the reference fixtures")
 
 
 @pytest.mark.parametrize("name", ["discounted_d2", "dplus_d3", "linear_avg_d2", "linear_noplus_d2", "standard_d2",
