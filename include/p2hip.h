@@ -86,12 +86,25 @@ int p2hip_showdown_both(const float* beliefs, const uint8_t* tables, const int64
  * sample_offsets [n+1] int64 (device) = prefix sums of 52 - cards on board.  source_rows = rows of
  * pre_beliefs / board, total_samples = rows the three outputs hold: a state whose row index lies
  * outside 0..source_rows-1 is skipped and no sample at or beyond total_samples is written, so
- * offsets that disagree with the boards cannot make the kernel leave its buffers.  Replaces the
+ * offsets that disagree with the boards cannot make the kernel leave its buffers; where a state
+ * yields fewer samples than its share [sample_offsets[i], sample_offsets[i+1]) of the outputs (more
+ * cards on its board than the offsets assume, no empty slot, a skipped row) the rest of the share is
+ * filled with zeros and root_lookup with i, so no output row is left uninitialised.  Replaces the
  * expansion half of ChanceNodeHelper.single_card_chance_values,
  * search/chance_node_helper.py:394-443. */
 int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
                         const int64_t* sample_offsets, int64_t source_rows, int64_t total_samples,
                         float* post_beliefs, int64_t* board_samples, int64_t* root_lookup, void* stream);
+
+/* The same expansion written as rows of a value network's INPUT MATRIX: input_rows [total_samples, 2704]
+ * in element type dtype (0 float32, 1 bfloat16, 2 float16), row s = the sample's 2 x 1326 ranges followed
+ * by the 52-entry one-hot of its board (the state's cards and the dealt one) — what the reference builds
+ * with a concatenation and a cast in front of its network (models/mlp/rebel_ffn.py forward; the ranges
+ * are the `beliefs` of the MLPFeatures that search/chance_node_helper.py:445-456 assembles).
+ * input_rows and pre_beliefs must be 16-byte aligned; board_samples may be NULL. */
+int p2hip_chance_expand_input(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
+                              const int64_t* sample_offsets, int64_t source_rows, int64_t total_samples,
+                              void* input_rows, int dtype, int64_t* board_samples, int64_t* root_lookup, void* stream);
 
 /* expected[i] = mean of hand_values [S,2,H] over samples sample_offsets[i] .. sample_offsets[i+1]
  * (index_add_ + divide of search/chance_node_helper.py:467-477). */

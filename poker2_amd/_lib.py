@@ -39,6 +39,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_tree_legal": [_P, _L, _P, _I, _I, _I, _I, _P, _P, _P],
     "p2hip_tree_step": [_P, _L, _L, _P, _I, _I, _L, _I, _P, _P, _P],
     "p2hip_chance_expand": [_P, _P, _P, _L, _P, _L, _L, _P, _P, _P, _P],
+    "p2hip_chance_expand_input": [_P, _P, _P, _L, _P, _L, _L, _P, _I, _P, _P, _P],
     "p2hip_flop_expand": [_P, _P, _L, _P, _L, _P, _P],
     "p2hip_perm_mean": [_P, _L, _L, _P, _I, _P, _I, _P, _P, _I, _P],
     "p2hip_chance_mean": [_P, _P, _L, _P, _P],

@@ -2,7 +2,7 @@
 not on its board (blocked hands removed, ranges renormalised), a value network answers for the
 samples, and the answers are averaged per leaf.
 
-    python -m poker2_amd.bench_turn [--roots 512] [--max-raises 1] [--iterations 100] [--json]
+    python -m poker2_amd.bench_turn [--roots 512] [--max-raises 3] [--iterations 100] [--json]
 
 Roots: random 4-card boards, Gamma(0.5) ranges with board-blocked hands removed, pot 200, stacks 800
 each, bet bins {0.5, 1} pot.  Network: 2 x 1326 ranges + board one-hot -> 3 x 1536 ReLU -> 2 x 1326,
@@ -45,7 +45,7 @@ def make_roots(b: int, seed: int):
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--roots", type=int, default=512)
-    ap.add_argument("--max-raises", type=int, default=1)
+    ap.add_argument("--max-raises", type=int, default=3)
     ap.add_argument("--iterations", type=int, default=100)
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--json", action="store_true")
@@ -63,12 +63,13 @@ def main() -> None:
     ev = HipSparseCFREvaluator(model, dev, cfg, fused_iteration=True, max_raises=args.max_raises)
     ev.initialize_subgame(roots, np.arange(b), bel)
     ev.prepare_search()
+    lean = dict(lean=True, alternate_reach_avg=True)       # as evaluate_cfr runs every iteration but its last
     for t in range(2):                       # first iterations: allocator, GEMM heuristics
-        ev.cfr_iteration(t)
+        ev.cfr_iteration(t, **lean)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     for t in range(2, args.iterations):
-        ev.cfr_iteration(t)
+        ev.cfr_iteration(t, **(lean if t + 1 < args.iterations else {}))
     torch.cuda.synchronize()
     t2 = time.perf_counter()
     reps = 5

@@ -73,9 +73,18 @@ def _rows_out_of_range(rows: torch.Tensor, n: int) -> bool:
     return bool(rows.numel()) and bool(((rows < 0) | (rows >= n)).any())
 
 
+INPUT_ROW_WIDTH = 2 * NUM_HANDS + 52       # [ranges of both players | one-hot of the board]
+_INPUT_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
 def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, board_pre: torch.Tensor,
-                  cards_on_board: int | None = None, check_rows: bool = True):
+                  cards_on_board: int | None = None, check_rows: bool = True, input_dtype: torch.dtype | None = None):
     """Every (state, next card) sample of a single-card chance node.
+
+    ``input_dtype`` (float32 / bfloat16 / float16): the samples are written as rows of a value network's
+    input matrix instead — first return value [S, 2704] in that dtype, each row the sample's ranges
+    followed by the 52-entry one-hot of its board — for networks whose input is exactly that
+    (``RangeBoardMLP``): no concatenation and no cast in front of the network.
 
     pre_chance_beliefs [R,2,1326] fp32, board_pre [R,5] int64 (-1 = empty), root_indices [B].
     Returns (post_beliefs [S,2,1326], board_samples [S,5], root_lookup [S], sample_offsets [B+1])
@@ -111,11 +120,23 @@ def chance_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, 
         per_state = 52 - cards_on_board
         total = b * per_state
         offsets = torch.arange(0, total + 1, per_state, dtype=torch.int64, device=dev)   # one launch, no board read
-    post = torch.empty(total, 2, NUM_HANDS, dtype=torch.float32, device=dev)
-    board_samples = torch.empty(total, 5, dtype=torch.int64, device=dev)
-    root_lookup = torch.empty(total, dtype=torch.int64, device=dev)
     # With ``cards_on_board`` given the sample count is taken on trust; the kernel gets the buffers'
-    # size and writes nothing beyond it if a board holds fewer cards than claimed.
+    # size and writes nothing beyond it if a board holds fewer cards than claimed.  Where a state has
+    # fewer samples than its share of the buffers (a board with MORE cards than claimed, no empty slot,
+    # or a row outside the table with check_rows=False) the kernel fills the rest of the share with zeros
+    # (root_lookup = the state): what a wrong claim leaves behind is defined, never uninitialised memory.
+    alloc = torch.empty
+    board_samples = alloc(total, 5, dtype=torch.int64, device=dev)
+    root_lookup = alloc(total, dtype=torch.int64, device=dev)
+    if input_dtype is not None:
+        _req(input_dtype in _INPUT_DTYPES, "input_dtype: float32, bfloat16 or float16")
+        rows = alloc(total, INPUT_ROW_WIDTH, dtype=input_dtype, device=dev)
+        _req(pre.data_ptr() % 16 == 0 and rows.data_ptr() % 16 == 0, "16-byte aligned ranges and input matrix")
+        _lib.call("p2hip_chance_expand_input", _lib.ptr(pre), _lib.ptr(roots), _lib.ptr(board), b, _lib.ptr(offsets),
+                  source_rows, total, _lib.ptr(rows), _INPUT_DTYPES[input_dtype], _lib.ptr(board_samples),
+                  _lib.ptr(root_lookup), _lib.stream_ptr())
+        return rows, board_samples, root_lookup, offsets
+    post = alloc(total, 2, NUM_HANDS, dtype=torch.float32, device=dev)
     _lib.call("p2hip_chance_expand", _lib.ptr(pre), _lib.ptr(roots), _lib.ptr(board), b, _lib.ptr(offsets),
               source_rows, total, _lib.ptr(post), _lib.ptr(board_samples), _lib.ptr(root_lookup),
               _lib.stream_ptr())
@@ -405,6 +426,25 @@ class ChanceNodeHelper:
         if root_indices.numel() == 0:
             return torch.zeros(0, self.num_players, NUM_HANDS, device=self.device, dtype=self.float_dtype)
         root_indices = root_indices.to(self.device)
+        model = self.model
+        if getattr(model, "input_layout", None) == "ranges|board_onehot" and hasattr(model, "forward_input") \
+                and pre_chance_beliefs.dtype == torch.float32 and pre_chance_beliefs.is_contiguous() \
+                and pre_chance_beliefs.data_ptr() % 16 == 0:
+            # the network reads nothing but the ranges and the board: the expansion writes its input matrix
+            in_dtype = self.autocast_dtype if self.autocast_dtype in _INPUT_DTYPES else torch.float32
+            rows, _, _, offsets = chance_expand(pre_chance_beliefs, root_indices, board_pre, cards_on_board,
+                                                check_rows, input_dtype=in_dtype)
+            if rows.shape[0] == 0:
+                return torch.zeros(root_indices.numel(), self.num_players, NUM_HANDS, device=self.device,
+                                   dtype=self.float_dtype)
+            if hasattr(model, "eval"):
+                model.eval()
+            if self.autocast_dtype is not None:
+                with torch.autocast(device_type="cuda", dtype=self.autocast_dtype):
+                    hv = model.forward_input(rows).hand_values
+            else:
+                hv = model.forward_input(rows).hand_values
+            return chance_mean(hv.to(torch.float32), offsets).to(self.float_dtype)
         post, board_samples, root_lookup, offsets = chance_expand(pre_chance_beliefs, root_indices, board_pre,
                                                                   cards_on_board, check_rows)
         if post.shape[0] == 0:

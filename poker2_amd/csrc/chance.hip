@@ -69,6 +69,26 @@ __device__ __forceinline__ bool chance_work(int64_t n, int parts, int group_size
   return true;
 }
 
+// A state's share of the output buffers is samples [sample_offsets[i], sample_offsets[i + 1]).  When the
+// state yields fewer samples than that (`have`: its board holds more cards than the caller's offsets
+// assume, has no empty slot, or its row lies outside the table) the rest of the share is filled with
+// zeros, root_lookup with the state, so that no row of the outputs is left uninitialised.  Called by the
+// workgroup of the state's last part; `row_bytes` is a multiple of 8 and `rows` 8-byte aligned.
+__device__ __forceinline__ void chance_fill_rest(const int64_t* __restrict__ sample_offsets, int64_t i, int have,
+                                                 int64_t total_samples, void* rows, int64_t row_bytes,
+                                                 int64_t* board_samples, int64_t* root_lookup) {
+  const int64_t s0 = sample_offsets[i] + have;
+  int64_t s1 = sample_offsets[i + 1];
+  if (s1 > total_samples) s1 = total_samples;
+  if (s0 < 0 || s0 >= s1) return;
+  uint2* dst = reinterpret_cast<uint2*>(reinterpret_cast<char*>(rows) + s0 * row_bytes);
+  const int64_t words = (s1 - s0) * (row_bytes / 8);
+  for (int64_t k = threadIdx.x; k < words; k += blockDim.x) dst[k] = make_uint2(0u, 0u);
+  for (int64_t k = threadIdx.x; k < (s1 - s0) * 5; k += blockDim.x)
+    if (board_samples) board_samples[s0 * 5 + k] = 0;
+  for (int64_t k = threadIdx.x; k < s1 - s0; k += blockDim.x) root_lookup[s0 + k] = i;
+}
+
 static inline unsigned chance_grid(int64_t n, int parts, int group_size) {
   return (unsigned)(((n + group_size - 1) / group_size) * group_size * parts);
 }
@@ -87,10 +107,14 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_kernel(const float* __
   int part;
   if (!chance_work(n, CH_SPLIT, CH_GROUP_ROWS, i, part)) return;
   const int64_t root = root_indices ? root_indices[i] : i;
-  if (root < 0 || root >= source_rows) return;   // uniform per workgroup: nothing to read, nothing written
+  const bool in_table = root >= 0 && root < source_rows;
   int bcards[5];
-  uint64_t bits;
-  const int ncards = chance_board(board + root * 5, bcards, bits);
+  uint64_t bits = 0;
+  const int ncards = in_table ? chance_board(board + root * 5, bcards, bits) : 5;
+  if (part == CH_SPLIT - 1)
+    chance_fill_rest(sample_offsets, i, ncards < 5 ? P2_CARDS - ncards : 0, total_samples, post_beliefs,
+                     2 * P2_H * (int64_t)sizeof(float), board_samples, root_lookup);
+  if (!in_table) return;   // uniform per workgroup: nothing to read
 
   // this lane's hands: pairs k -> hands 2*idx, 2*idx+1 with idx = tid + k*256
   float v[2][CH_PPT][2];
@@ -185,28 +209,45 @@ struct ChanceSample {   // what a float4 needs to know about its sample
   int pad;
 };
 
+// What a sample's output row looks like.  INPUT_ROWS = false: the 2 x 1326 ranges as float32, samples back to
+// back (`post_beliefs` [S, 2, 1326]).  INPUT_ROWS = true: a row of a value network's input matrix
+// [S, CH_INPUT_WIDTH] in element type DT (0 float32, 1 bfloat16, 2 float16) — the ranges followed by the
+// 52-entry one-hot of the sample's board (the state's cards and the dealt one) — so the network needs
+// neither a concatenation nor a cast.  Either way a row is a whole number of 16-byte units and the
+// samples of a workgroup are one contiguous run of units.
+constexpr int CH_INPUT_WIDTH = 2 * P2_H + P2_CARDS;   // 2704
+constexpr int CH_LDS_PAD = 8;                          // the unit that straddles the end of the ranges reads on
+static_assert((CH_INPUT_WIDTH * 2) % 16 == 0 && (CH_INPUT_WIDTH * 4) % 16 == 0, "input rows are whole 16-byte units");
+
+template <int DT, bool INPUT_ROWS>
 __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const float* __restrict__ pre_beliefs,
                                                                         const int64_t* __restrict__ root_indices,
                                                                         const int64_t* __restrict__ board,
                                                                         const int64_t* __restrict__ sample_offsets,
                                                                         int64_t source_rows, int64_t total_samples,
-                                                                        float* __restrict__ post_beliefs,
+                                                                        void* __restrict__ post_beliefs,
                                                                         int64_t* __restrict__ board_samples,
                                                                         int64_t* __restrict__ root_lookup, int64_t n,
                                                                         int parts) {
-  __shared__ __align__(16) float t[2 * P2_H];            // the state's ranges without the board's hands
-  __shared__ __align__(16) uint16_t cards_of[2 * P2_H];  // a | b << 8 of the hand behind every float of t
+  static_assert(INPUT_ROWS || DT == 0, "plain ranges are float32");
+  constexpr int UNIT = DT == 0 ? 4 : 8;                                        // elements per 16-byte unit
+  constexpr int ROW_UNITS = (INPUT_ROWS ? CH_INPUT_WIDTH : 2 * P2_H) / UNIT;   // 663, 676 or 338
+  __shared__ __align__(16) float t[2 * P2_H + CH_LDS_PAD];            // the state's ranges without the board's hands
+  __shared__ __align__(16) uint16_t cards_of[2 * P2_H + CH_LDS_PAD];  // a | b << 8 of the hand behind every float of t
   __shared__ double cs[2 * P2_CARDS];
   __shared__ __align__(16) ChanceSample sample[CH_MAX_RUN];
   int64_t i;
   int part;
   if (!chance_work(n, parts, CH_GROUP_LINES, i, part)) return;
   const int64_t root = root_indices ? root_indices[i] : i;
-  if (root < 0 || root >= source_rows) return;   // uniform per workgroup
+  const bool in_table = root >= 0 && root < source_rows;
   int bcards[5];
-  uint64_t bits;
-  const int ncards = chance_board(board + root * 5, bcards, bits);
-  if (ncards >= 5) return;                       // no empty slot: nothing to expand
+  uint64_t bits = 0;
+  const int ncards = in_table ? chance_board(board + root * 5, bcards, bits) : 5;
+  if (part == parts - 1)
+    chance_fill_rest(sample_offsets, i, ncards < 5 ? P2_CARDS - ncards : 0, total_samples, post_beliefs,
+                     ROW_UNITS * 16ll, board_samples, root_lookup);
+  if (ncards >= 5) return;                       // outside the table, or no empty slot: nothing to expand
 
   const float4* src = reinterpret_cast<const float4*>(pre_beliefs + root * (2 * P2_H));
 #pragma unroll
@@ -228,6 +269,10 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
     reinterpret_cast<float4*>(t)[j] = make_float4(y[0], y[1], y[2], y[3]);
     reinterpret_cast<uint2*>(cards_of)[j] = make_uint2((uint32_t)packed[0] | ((uint32_t)packed[1] << 16),
                                                        (uint32_t)packed[2] | ((uint32_t)packed[3] << 16));
+  }
+  if (threadIdx.x < CH_LDS_PAD) {
+    t[2 * P2_H + threadIdx.x] = 0.f;
+    cards_of[2 * P2_H + threadIdx.x] = 0;
   }
   p2_sync_lds();
   card_sums_multi(t, P2_H, 2, cs);
@@ -269,7 +314,7 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
 #pragma unroll
         for (int q = 1; q < 5; ++q) card = slot == q ? (int64_t)bcards[q] : card;
         if (slot == ncards) card = sample[m].card;
-        board_samples[(s_first + m) * 5 + slot] = card;
+        if (board_samples) board_samples[(s_first + m) * 5 + slot] = card;
       } else if (slot == 5) {
         root_lookup[s_first + m] = i;
       }
@@ -278,27 +323,48 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
 
   const int remaining = P2_CARDS - ncards - 1;          // cards left for the hands of a sample
   const float uniform = 1.0f / fmaxf((float)(remaining * (remaining - 1) / 2), 1.0f);
-  float4* out = reinterpret_cast<float4*>(post_beliefs);
-  const int64_t g0 = s_first * CH_QUADS, g1 = g0 + (int64_t)count * CH_QUADS;   // float4 range of the workgroup
+  uint4* out = reinterpret_cast<uint4*>(post_beliefs);
+  const int64_t g0 = s_first * ROW_UNITS, g1 = g0 + (int64_t)count * ROW_UNITS;   // 16-byte units of the workgroup
   for (int64_t g = (g0 & ~7ll) + threadIdx.x; g < g1; g += CH_BLOCK) {
     if (g < g0) continue;
     const uint32_t local = (uint32_t)(g - g0);
-    const uint32_t m = local / CH_QUADS, j = local - m * CH_QUADS;
+    const uint32_t m = local / ROW_UNITS, j = local - m * ROW_UNITS;
     const ChanceSample sm = sample[m];
-    const float4 x = reinterpret_cast<const float4*>(t)[j];
-    const uint2 pk = reinterpret_cast<const uint2*>(cards_of)[j];
-    const float xs[4] = {x.x, x.y, x.z, x.w};
-    const uint32_t cd[4] = {pk.x & 0xFFFFu, pk.x >> 16, pk.y & 0xFFFFu, pk.y >> 16};
-    float r[4];
+    float xs[UNIT];
+    uint32_t cd[UNIT];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float inv = (4 * j + q >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
+    for (int u = 0; u < UNIT / 4; ++u) {
+      // a unit behind the ranges (board one-hot only) reads the last padded quad: its values are not used
+      const uint32_t quad = min(j * (UNIT / 4) + u, (uint32_t)(2 * P2_H + CH_LDS_PAD) / 4 - 1);
+      const float4 x = reinterpret_cast<const float4*>(t)[quad];
+      const uint2 pk = reinterpret_cast<const uint2*>(cards_of)[quad];
+      xs[4 * u] = x.x; xs[4 * u + 1] = x.y; xs[4 * u + 2] = x.z; xs[4 * u + 3] = x.w;
+      cd[4 * u] = pk.x & 0xFFFFu; cd[4 * u + 1] = pk.x >> 16; cd[4 * u + 2] = pk.y & 0xFFFFu; cd[4 * u + 3] = pk.y >> 16;
+    }
+    const uint64_t dealt = bits | (1ull << sm.card);   // the sample's board as a card set
+    float r[UNIT];
+#pragma unroll
+    for (int q = 0; q < UNIT; ++q) {
+      const uint32_t e = UNIT * j + q;                  // element of the row
+      const float inv = (e >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
       const uint32_t a = cd[q] & 0xFFu, b = cd[q] >> 8;
       float val = xs[q] * inv;
       if (inv == 0.f) val = (((bits >> a) | (bits >> b)) & 1ull) ? 0.f : uniform;   // no mass left: uniform
       r[q] = (a == (uint32_t)sm.card || b == (uint32_t)sm.card) ? 0.f : val;
+      if (INPUT_ROWS && e >= (uint32_t)(2 * P2_H)) r[q] = ((dealt >> (e - 2 * P2_H)) & 1ull) ? 1.f : 0.f;
     }
-    out[g] = make_float4(r[0], r[1], r[2], r[3]);
+    uint4 w;
+    if (DT == 0) {
+      w = make_uint4(__builtin_bit_cast(uint32_t, r[0]), __builtin_bit_cast(uint32_t, r[1]),
+                     __builtin_bit_cast(uint32_t, r[2]), __builtin_bit_cast(uint32_t, r[3]));
+    } else if (DT == 1) {
+      w = make_uint4(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]), pack_bf16(r[4 % UNIT], r[5 % UNIT]),
+                     pack_bf16(r[6 % UNIT], r[7 % UNIT]));
+    } else {
+      w = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4 % UNIT], r[5 % UNIT]),
+                     pack_f16(r[6 % UNIT], r[7 % UNIT]));
+    }
+    out[g] = w;
   }
 }
 
@@ -821,15 +887,37 @@ int p2hip_chance_expand(const float* pre_beliefs, const int64_t* root_indices, c
     // runs of 13 cards = 4 workgroups per state (3584 states: 375 us, in runs of 4 cards 465 us; 333 states:
     // 37 and 42 us); runs of 4 cards only where there would be fewer workgroups than the chip takes at once
     const int parts = n >= 256 ? 4 : p2::CH_SPLIT;
-    hipLaunchKernelGGL(p2::chance_expand_lines_kernel, dim3(p2::chance_grid(n, parts, p2::CH_GROUP_LINES)), dim3(p2::CH_BLOCK), 0,
-                       (hipStream_t)stream, pre_beliefs, root_indices, board, sample_offsets, source_rows,
-                       total_samples, post_beliefs, board_samples, root_lookup, n, parts);
+    hipLaunchKernelGGL((p2::chance_expand_lines_kernel<0, false>), dim3(p2::chance_grid(n, parts, p2::CH_GROUP_LINES)),
+                       dim3(p2::CH_BLOCK), 0, (hipStream_t)stream, pre_beliefs, root_indices, board, sample_offsets,
+                       source_rows, total_samples, (void*)post_beliefs, board_samples, root_lookup, n, parts);
     P2_LAUNCH_CHECK();
     return 0;
   }
   hipLaunchKernelGGL(p2::chance_expand_kernel, dim3(p2::chance_grid(n, p2::CH_SPLIT, p2::CH_GROUP_ROWS)), dim3(p2::CH_BLOCK), 0,
                      (hipStream_t)stream, pre_beliefs, root_indices, board, sample_offsets, source_rows,
                      total_samples, post_beliefs, board_samples, root_lookup, n);
+  P2_LAUNCH_CHECK();
+  return 0;
+}
+
+int p2hip_chance_expand_input(const float* pre_beliefs, const int64_t* root_indices, const int64_t* board, int64_t n,
+                              const int64_t* sample_offsets, int64_t source_rows, int64_t total_samples,
+                              void* input_rows, int dtype, int64_t* board_samples, int64_t* root_lookup, void* stream) {
+  if (n < 0 || source_rows < 0 || total_samples < 0 || dtype < 0 || dtype > 2) return P2_EINVAL;
+  if (n == 0) return 0;
+  if (!pre_beliefs || !board || !sample_offsets || !input_rows || !root_lookup) return P2_EINVAL;
+  if (((reinterpret_cast<uintptr_t>(pre_beliefs) | reinterpret_cast<uintptr_t>(input_rows)) & 15u) != 0) return P2_EINVAL;
+  if (n > 0x7FFFFFFF / p2::CH_SPLIT - p2::CH_GROUP_ROWS) return P2_EINVAL;
+  const int parts = n >= 256 ? 4 : p2::CH_SPLIT;
+  const dim3 grid(p2::chance_grid(n, parts, p2::CH_GROUP_LINES)), block(p2::CH_BLOCK);
+#define P2_EXPAND_INPUT(DT)                                                                                      \
+  hipLaunchKernelGGL((p2::chance_expand_lines_kernel<DT, true>), grid, block, 0, (hipStream_t)stream, pre_beliefs, \
+                     root_indices, board, sample_offsets, source_rows, total_samples, input_rows, board_samples,  \
+                     root_lookup, n, parts)
+  if (dtype == 0) P2_EXPAND_INPUT(0);
+  else if (dtype == 1) P2_EXPAND_INPUT(1);
+  else P2_EXPAND_INPUT(2);
+#undef P2_EXPAND_INPUT
   P2_LAUNCH_CHECK();
   return 0;
 }

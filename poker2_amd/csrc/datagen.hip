@@ -163,19 +163,6 @@ __global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* _
 constexpr int LEAF_ROW = 2 * P2_H;            // 2652 floats
 constexpr int LEAF_CHUNKS = LEAF_ROW / 4;     // 663
 
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {   // round to nearest even, like torch
-  auto one = [](float x) -> uint32_t {
-    uint32_t u = __builtin_bit_cast(uint32_t, x);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;          // NaN stays NaN
-    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-  };
-  return one(a) | (one(b) << 16);
-}
-__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
-  const _Float16 x = (_Float16)a, y = (_Float16)b;
-  return (uint32_t)__builtin_bit_cast(uint16_t, x) | ((uint32_t)__builtin_bit_cast(uint16_t, y) << 16);
-}
-
 // dst[i, 0:2652] = src[rows[i]] converted to DT (0 float32, 1 bfloat16, 2 float16); dst rows are
 // dst_stride elements apart (columns behind 2652 are left alone).
 template <int DT>

@@ -46,6 +46,9 @@ class RangeBoardMLP(torch.nn.Module):
     # 2652 columns (HipSparseCFREvaluator.gather_leaf_rows does that in the matrix's dtype) and call
     # forward_input: no concatenation and no separate cast per call.
     input_width = 2 * NUM_HANDS + 52
+    # context, street and player to act are not read: a caller that can produce [ranges | board one-hot]
+    # rows itself (the chance-node expansion does) may skip the feature bundle altogether
+    input_layout = "ranges|board_onehot"
 
     def static_input_columns(self, features: MLPFeatures, dtype: torch.dtype) -> torch.Tensor:
         """[N, input_width] with the columns that do not depend on the ranges filled in."""

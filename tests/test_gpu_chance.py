@@ -563,3 +563,91 @@ def test_orbit_mean_equals_the_mean_over_all_24_permutations(K):
         base = torch.from_numpy(rng.standard_normal((b, 2, H)).astype(np.float32)).cuda()
         again = K.orbit_mean(t_hv, t_w, out=base.clone())
         np.testing.assert_allclose(again.cpu().numpy(), base.cpu().numpy() + exp, rtol=1e-5, atol=4e-6)
+
+
+# ---- the expansion written straight into the network's input matrix ---------------------------
+@pytest.mark.parametrize("n", [6, 300])
+def test_expansion_as_input_rows_equals_concatenation_and_cast(K, n):
+    """``chance_expand(..., input_dtype=...)``: rows [ranges | one-hot of the sample's board] in float32 /
+    bfloat16 / float16 against what the network's own ``forward`` builds from the plain expansion
+    (scatter one-hot, concatenate, cast): bit for bit — the values are those of the plain expansion,
+    which the oracle pins, and the casts round like torch's."""
+    rng = np.random.default_rng(70 + n)
+    boards, pre = inputs(rng, n, [4, 3, 4, 0, 4])
+    pre[1, 0] = 0.0
+    roots = torch.from_numpy(rng.permutation(n)[: max(n - 2, 1)]).cuda()
+    tp, tb = torch.from_numpy(pre).cuda(), torch.from_numpy(boards).cuda()
+    post, bs, lookup, offsets = K.chance_expand(tp, roots, tb)
+    onehot = torch.zeros(bs.shape[0], 53, device="cuda")
+    onehot.scatter_(1, torch.where(bs >= 0, bs, torch.full_like(bs, 52)), 1.0)
+    want = torch.cat([post.reshape(post.shape[0], -1), onehot[:, :52]], dim=1)
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        rows, bs2, lookup2, offsets2 = K.chance_expand(tp, roots, tb, input_dtype=dt)
+        assert rows.dtype == dt and rows.shape == (post.shape[0], K.INPUT_ROW_WIDTH)
+        assert torch.equal(rows, want.to(dt)), dt
+        assert torch.equal(bs2, bs) and torch.equal(lookup2, lookup) and torch.equal(offsets2, offsets)
+
+
+@pytest.mark.parametrize("autocast", [None, torch.bfloat16])
+def test_helper_feeds_a_ranges_and_board_network_without_concatenation(K, autocast):
+    """``single_card_chance_values`` with a network that declares its input as [ranges | board one-hot]
+    (RangeBoardMLP): the expansion writes the input matrix, ``forward_input`` runs on it; same answer as the
+    feature-bundle path (``forward``: scatter, concatenate, cast under autocast) — the same numbers reach the
+    same GEMMs."""
+    from poker2_amd.leaf_models import RangeBoardMLP
+    rng = np.random.default_rng(77)
+    n = 40
+    boards, pre = inputs(rng, n, [4])
+    dev = torch.device("cuda")
+    net = RangeBoardMLP(hidden=64, layers=2, seed=5).to(dev)
+
+    class Plain(torch.nn.Module):                      # the same network without the declaration
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, f):
+            return self.inner(f)
+    roots = torch.arange(n, device=dev)
+    feats = K.MLPFeatures(context=torch.zeros(n, 4, device=dev), street=torch.full((n,), 2, device=dev),
+                          to_act=torch.zeros(n, dtype=torch.long, device=dev), board=torch.from_numpy(boards).to(dev),
+                          beliefs=torch.from_numpy(pre).to(dev).reshape(n, -1))
+    tp, tb = torch.from_numpy(pre).to(dev), torch.from_numpy(boards).to(dev)
+    direct = K.ChanceNodeHelper(dev, torch.float32, 2, net, autocast_dtype=autocast)
+    bundle = K.ChanceNodeHelper(dev, torch.float32, 2, Plain(net), autocast_dtype=autocast)
+    a = direct.single_card_chance_values(roots, feats, tp, tb)
+    b = bundle.single_card_chance_values(roots, feats, tp, tb)
+    c = direct.single_card_chance_values(roots, feats, tp, tb, cards_on_board=4, check_rows=False)
+    assert torch.equal(a, b) and torch.equal(a, c)
+    assert float(a.abs().max()) > 0
+
+
+def test_a_wrong_card_count_claim_leaves_defined_rows(K):
+    """With ``cards_on_board`` claimed and ``check_rows=False`` the outputs are sized on trust.  A board that
+    holds more cards than claimed, a board without an empty slot and a row outside the table yield fewer
+    samples than their share of the buffers: the rest of the share is zeros with ``root_lookup`` = the state,
+    in every form of the expansion, so nothing uninitialised reaches the network."""
+    rng = np.random.default_rng(78)
+    boards, pre = inputs(rng, 5, [3])
+    boards[1, 3] = 40 if 40 not in boards[1] else 41            # four cards where three are claimed
+    boards[2] = np.array([0, 1, 2, 3, 4])                       # no empty slot
+    roots = torch.tensor([0, 1, 2, 7, 4]).cuda()                # 7: outside the table
+    tp, tb = torch.from_numpy(pre).cuda(), torch.from_numpy(boards).cuda()
+    for kw in ({}, {"input_dtype": torch.float32}, {"input_dtype": torch.bfloat16}):
+        for poison in (float("nan"), 3.0):
+            # the caching allocator hands the poisoned block back to the call below
+            width = 2 * H if not kw else K.INPUT_ROW_WIDTH
+            junk = torch.full((5 * 49, width), poison, dtype=kw.get("input_dtype", torch.float32), device="cuda")
+            del junk
+            out, bs, lookup, offsets = K.chance_expand(tp, roots, tb, cards_on_board=3, check_rows=False, **kw)
+            torch.cuda.synchronize()
+            rows = out.reshape(5, 49, -1).float()
+            assert bool(torch.isfinite(rows).all())
+            assert float(rows[1, 48].abs().max()) == 0 and float(rows[1, :48, :2 * H].sum()) > 0     # 48 samples + one zero row
+            assert float(rows[2].abs().max()) == 0 and float(rows[3].abs().max()) == 0                # nothing to expand
+            assert lookup.view(5, 49).eq(torch.arange(5, device="cuda")[:, None]).all()
+            assert float(rows[0, :, :2 * H].sum()) > 0 and float(rows[4, :, :2 * H].sum()) > 0
+    # the row-wise kernel (8-byte aligned output) through the C ABI: the same
+    g = _expand_through_abi(tp, roots, tb, 2, claimed_cards=3)
+    assert bool(torch.isfinite(g[0]).all()) and float(g[0].view(5, 49, -1)[2].abs().max()) == 0
+    assert g[2].view(5, 49).eq(torch.arange(5, device="cuda")[:, None]).all()

@@ -82,16 +82,16 @@ def test_turn_subgames_with_chance_leaves_B512():
     def run(n, iters=iters):
         roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards[:n],
                                           button=np.arange(n) % 2)
+        # the configuration's own bet tree: bins {0.5, 1} pot + all-in, at most three raises
         ev = HipSparseCFREvaluator(ChanceLeafModel(net, dev), dev, river_dcfr_config(n, iterations=iters, depth=16,
-                                                                                     dcfr_delay=0), max_raises=1)
+                                                                                     dcfr_delay=0), max_raises=3)
         ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs[:n]))
         ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
-        for t in range(iters):
-            ev.cfr_iteration(t)
+        ev.run_search_iterations()
         return ev
     # the configuration's own length: 100 iterations at the full batch, checked by what every state must satisfy
     ev = run(b, 100)
-    assert ev.total_nodes == 21 * b and ev.model_indices.numel() == 7 * b        # 7 street-end leaves per root
+    assert ev.total_nodes == 105 * b and ev.model_indices.numel() == 35 * b      # 35 street-end leaves per root
     assert float(ev.latest_values[ev.model_indices].abs().max()) > 1e-3          # the network matters
     check_distributions(ev, rng)
     stats = ev._compute_exploitability()
