@@ -142,7 +142,11 @@ int p2hip_orbit_mean(const float* hand_values, int64_t n, int64_t n_flops, const
  * call allocates and frees nothing.  shares * n * 2 * 1326 floats must fit it: a larger request
  * returns 2 (hipErrorOutOfMemory) before anything is launched.  Same results, bit for bit, as
  * p2hip_orbit_mean with the same `shares`.  Every call on one GPU uses that GPU's array: calls
- * that overlap on one GPU (different streams, threads) race; calls on one stream do not. */
+ * that overlap on one GPU (different streams, threads) race; calls on one stream do not.
+ * The array's address on a device is resolved by the first call made with that device current
+ * (hipGetSymbolAddress, which may load the code object): make that call OUTSIDE graph capture — a call
+ * with n = 0 does the resolution and nothing else (null pointers allowed).  Later calls on the device
+ * neither allocate nor resolve anything. */
 #define P2HIP_ORBIT_SCRATCH_FLOATS (4 * 1024 * 1024)
 int p2hip_orbit_mean_static(const float* hand_values, int64_t n, int64_t n_flops, const float* weight,
                             int accumulate, float* out, int shares, void* stream);

@@ -252,7 +252,8 @@ def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tenso
     ``static_scratch=True`` (needs ``out``) takes the entry point that allocates nothing
     (``p2hip_orbit_mean_static``): partial sums go to a 16 MiB array inside the library, so the
     call can sit under graph capture; it refuses inputs whose partial sums do not fit and must
-    not overlap with another such call on the same GPU."""
+    not overlap with another such call on the same GPU.  The first such call on a device resolves the
+    array's address there and must itself run outside capture: ``orbit_scratch_init()`` is that call."""
     if not _lib.hip_is_available():
         raise RuntimeError("orbit_mean needs libp2hip.so and a GPU (no CPU fallback exists).")
     _lib.require_gpu(hand_values, "orbit_mean")
@@ -286,6 +287,12 @@ def orbit_mean(hand_values: torch.Tensor, weight: torch.Tensor, out: torch.Tenso
     _lib.call("p2hip_orbit_mean", _lib.ptr(hv), b, k, _lib.ptr(w), int(accumulate), _lib.ptr(out),
               _lib.ptr(workspace), shares, _lib.stream_ptr())
     return out
+
+
+def orbit_scratch_init() -> None:
+    """Resolve the static scratch array of ``p2hip_orbit_mean_static`` on the current device (once per device,
+    outside graph capture); launches nothing."""
+    _lib.call("p2hip_orbit_mean_static", None, 0, 0, None, 0, None, 1, _lib.stream_ptr())
 
 
 def canonical_flops():

@@ -1059,7 +1059,12 @@ static int orbit_scratch_address(float** out) {
 int p2hip_orbit_mean_static(const float* hand_values, int64_t n, int64_t n_flops, const float* weight,
                             int accumulate, float* out, int shares, void* stream) {
   if (n < 0 || n_flops < 0 || shares < 1) return P2_EINVAL;
-  if (n == 0) return 0;
+  if (n == 0) {
+    // Set-up call: resolves this device's address of the array (the first resolution on a device may load
+    // the code object and is not something to do under graph capture) and launches nothing.
+    float* scratch = nullptr;
+    return p2::orbit_scratch_address(&scratch);
+  }
   if (!hand_values || !weight || !out || !p2_aligned8(hand_values) || !p2_aligned8(out)) return P2_EINVAL;
   if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
   const int64_t per_share = (n_flops + shares - 1) / shares;

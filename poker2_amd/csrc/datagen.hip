@@ -90,9 +90,9 @@ __global__ __launch_bounds__(DG_BLOCK) void policy_targets_kernel(const float* _
 #pragma unroll
   for (int j = 0; j < A; ++j) {
     const bool have = j < n_children;
-    // a slot without a child requests the node's own row (always inside the table; a childless node's
-    // child_offsets entry may equal the row count) and drops what it read
-    const int64_t row = have ? first + j : r;
+    // a slot without a child repeats the first child's row (a cache hit) and drops what it read; a node
+    // without any child requests its own row instead: its child_offsets entry may equal the row count
+    const int64_t row = have ? first + j : (n_children > 0 ? first : r);
     const int a = have ? (int)action_from_parent[row] : -1;
     act[j] = (a >= 0 && a < A) ? a : -1;
     const float2* src = p2_row2(policy_avg, row);

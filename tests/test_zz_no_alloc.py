@@ -20,7 +20,10 @@ def test_static_variant_refuses_what_does_not_fit_without_touching_a_gpu():
     assert lib.p2hip_orbit_mean_static(None, 4, 8, None, 0, None, 2, None) == 1
     assert lib.p2hip_orbit_mean_static(fake, -1, 8, fake, 0, fake, 2, None) == 1
     assert lib.p2hip_orbit_mean_static(fake, 4, 8, fake, 0, fake, 0, None) == 1
-    assert lib.p2hip_orbit_mean_static(fake, 0, 8, fake, 0, fake, 2, None) == 0      # nothing to do
+    # n = 0 is the set-up call: it resolves the array's address on the current device and launches nothing;
+    # without a device it reports the HIP error instead of resolving anything
+    rc = lib.p2hip_orbit_mean_static(None, 0, 0, None, 0, None, 1, None)
+    assert (rc == 0) == torch.cuda.is_available()
     n, shares = 800, 2                            # 2 * 800 * 2652 = 4 243 200 floats > 4 194 304
     assert shares * n * 2 * H > SCRATCH_FLOATS
     assert lib.p2hip_orbit_mean_static(fake, n, 8, fake, 0, fake, shares, None) == 2  # hipErrorOutOfMemory
@@ -56,6 +59,9 @@ def test_static_variant_equals_the_workspace_variant_on_two_calls_in_a_row():
         assert torch.isfinite(got).all()
         return got
 
+    from poker2_amd import chance_node_helper as K
+    K.orbit_scratch_init()                                  # the per-device set-up call (n = 0), twice: idempotent
+    K.orbit_scratch_init()
     first = both(n=24, k=40, shares=16, accumulate=0)       # 16 * 24 * 2652 floats = 1.0 M of the 4 M array
     second = both(n=5, k=7, shares=3, accumulate=1)         # smaller, other share layout, on top of `out`
     assert first.shape == (24, 2, H) and second.shape == (5, 2, H)
@@ -67,7 +73,6 @@ def test_static_variant_equals_the_workspace_variant_on_two_calls_in_a_row():
     fake = first.data_ptr()
     assert lib.p2hip_orbit_mean_static(fake, n_max + 1, 2, fake, 0, fake, 2, stream) == 2
     # the Python wrapper's switch reaches the same entry point
-    from poker2_amd import chance_node_helper as K
     hv = torch.randn(6, 300, 2, H, generator=gen).to(dev)
     w = torch.rand(300, generator=gen).to(dev)
     a = K.orbit_mean(hv, w)
