@@ -1,7 +1,7 @@
 """Where a workgroup of the iteration kernel spends its time: the sweeps' shares, from the tuning build.
 
     python -m poker2_amd.build --sweep-timers          (once, beside the library; needs no GPU)
-    python -m poker2_amd.bench_sweeps [--roots 4096] [--max-raises 3] [--depth 16] [--iterations 10] [--one-workgroup-per-root]
+    python -m poker2_amd.bench_sweeps [--roots 4096] [--max-raises 3] [--depth 16] [--iterations 10] [--one-workgroup-per-root] [--plain]
 
 The tuning build of the library (``-DP2_ITER_PROFILE``) adds the ticks of the 100 MHz wall clock that
 each workgroup spends inside each sweep of ``cfr_iteration_kernel`` into a table in device memory; this
@@ -43,7 +43,11 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--one-workgroup-per-root", action="store_true",
                     help="no work items: every root's tree walked by one workgroup")
+    ap.add_argument("--plain", action="store_true",
+                    help="iterations that store every row, reach_avg in place (cfr_iteration(t)); default: as a search "
+                         "runs them (rows nothing reads left unwritten, reach_avg alternating between two buffers)")
     args = ap.parse_args()
+    how = {} if args.plain else dict(lean=True, alternate_reach_avg=True)
     if not torch.cuda.is_available():
         raise SystemExit("bench_sweeps needs a GPU")
     if not os.path.exists(SWEEP_TIMER_LIB_PATH):
@@ -65,13 +69,13 @@ def main() -> None:
     ev.prepare_search()
     table = np.zeros((8192, 8), dtype=np.int64)
     for t in range(5):
-        ev.cfr_iteration(t)
+        ev.cfr_iteration(t, **how)
     torch.cuda.synchronize()
     _lib.check(read(table.ctypes.data, 1), "p2hip_iter_prof_read")
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for t in range(5, 5 + args.iterations):
-        ev.cfr_iteration(t)
+        ev.cfr_iteration(t, **how)
     stop.record()
     torch.cuda.synchronize()
     _lib.check(read(table.ctypes.data, 1), "p2hip_iter_prof_read")
@@ -80,7 +84,8 @@ def main() -> None:
     total = us[0] + us[1] + us[2]
     items = "one workgroup per root" if ev._items is None else f"work items in tiers of {list(ev._items.tiers)}"
     print(f"{n} river roots, {int(ev.total_nodes)} nodes ({ev.total_nodes // n} per root), {items}; "
-          f"{args.iterations} iterations, {start.elapsed_time(stop) / args.iterations:.3f} ms each with the timers")
+          f"{args.iterations} {'plain' if args.plain else 'search'} iterations, "
+          f"{start.elapsed_time(stop) / args.iterations:.3f} ms each with the timers")
     print(f"{'':58s} {'us / root-iteration':>20s} {'share':>7s}")
     for slot, label, parent in SLOTS:
         print(f"{label:58s} {us[slot]:20.1f} {100 * us[slot] / total:6.1f}%")

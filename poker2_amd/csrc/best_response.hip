@@ -125,7 +125,10 @@ __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const double v = total_b - cs[nc * P2_CARDS + (ab[k][q] & 0xFFu)] - cs[nc * P2_CARDS + (ab[k][q] >> 8)] + (double)b[k][q];
-      ub[k][q] = fmaxf((float)v, 0.f);
+      // one reciprocal per hand instead of a division per hand and child (0 where the opponent has no
+      // compatible mass: the projected probability is then 0, cfr_evaluator.py:700-703)
+      const float u0 = fmaxf((float)v, 0.f);
+      ub[k][q] = u0 > 1e-5f ? 1.0f / u0 : 0.f;
       ov[k][q] = 0.f;
     }
   for (int g0 = 0; g0 < nc; g0 += BR_GRP) {
@@ -146,8 +149,7 @@ __global__ __launch_bounds__(BR_BLOCK) void best_response_level_kernel(
         for (int q = 0; q < 2; ++q) {
           const double u = total_c - csc[ab[k][q] & 0xFFu] - csc[ab[k][q] >> 8] + (double)mm[q];
           const float uc = fmaxf((float)u, 0.f);
-          const float prob = ub[k][q] > 1e-5f ? uc / ub[k][q] : 0.f;
-          ov[k][q] += prob * vv[q];
+          ov[k][q] += (uc * ub[k][q]) * vv[q];
         }
       }
     }

@@ -99,37 +99,46 @@ class RebelDataGenerator:
                              device=self.device)
         return PublicBeliefState(env=self.env_proto.reset(target_batch_size), beliefs=beliefs)
 
-    def _extend_pbs(self, pbs, desired_size: int) -> PublicBeliefState:
-        """Freshly dealt hands behind the states that are still being played (:42-50)."""
-        current = pbs.env.n
-        new_pbs = self._new_pbs(desired_size)
-        _overwrite_rows(new_pbs.env, pbs.env, current)
-        new_pbs.beliefs[:current] = pbs.beliefs
-        return new_pbs
+    def _top_up(self) -> PublicBeliefState:
+        """The states the next search starts from: the hands still being played first, freshly dealt
+        ones behind them until the evaluator's batch is full (:42-50, :60-66)."""
+        want = self.evaluator.root_nodes
+        playing = self.current_pbs
+        if playing is not None and playing.env.n >= want:
+            return playing
+        fresh = self._new_pbs(want)
+        if playing is not None:
+            kept = playing.env.n
+            _overwrite_rows(fresh.env, playing.env, kept)
+            fresh.beliefs[:kept] = playing.beliefs
+        return fresh
+
+    def search_pass(self) -> tuple[RebelBatch, RebelBatch, RebelBatch]:
+        """One search over a full batch of public states.  Its three training batches — values at the
+        roots, values of the states before the deal, policies — go to the buffers in the reference's
+        order (policy, value, pre-deal value: :70-77); the sampled leaves become the states that are
+        still being played."""
+        start = self._top_up()
+        ev = self.evaluator
+        ev.initialize_subgame(start.env, np.arange(start.env.n), start.beliefs)
+        self.current_pbs = ev.evaluate_cfr()
+        value, pre_deal_value, policy = ev.training_data()
+        for buffer, batch in ((self.policy_buffer, policy), (self.value_buffer, value),
+                              (self.value_buffer, pre_deal_value)):
+            buffer.add_batch(batch)
+        return value, pre_deal_value, policy
 
     def generate_data(self, value_sample_count: int) -> tuple[RebelBatch | None, RebelBatch | None]:
-        """Searches until ``value_sample_count`` value samples have been collected (:52-95).
-        Returns (value batch, policy batch) of this call; both also went to the buffers."""
-        N = self.evaluator.root_nodes
-        root_indices = np.arange(N)
-        collected = self.last_extra
-        value_batches, policy_batches = [], []
-        while collected < value_sample_count:
-            if self.current_pbs is None:
-                self.current_pbs = self._new_pbs(N)
-            elif self.current_pbs.env.n < N:
-                self.current_pbs = self._extend_pbs(self.current_pbs, N)
-            self.evaluator.initialize_subgame(self.current_pbs.env, root_indices, self.current_pbs.beliefs)
-            self.current_pbs = self.evaluator.evaluate_cfr()
-            value_batch, augmented_value_batch, policy_batch = self.evaluator.training_data()
-            self.policy_buffer.add_batch(policy_batch)
-            self.value_buffer.add_batch(value_batch)
-            self.value_buffer.add_batch(augmented_value_batch)
-            policy_batches.append(policy_batch)
-            value_batches.append(value_batch)
-            value_batches.append(augmented_value_batch)
-            collected += len(value_batch)
-        self.last_extra = collected - value_sample_count
-        fresh_value_batch = RebelBatch.cat(value_batches) if value_batches else None
-        fresh_policy_batch = RebelBatch.cat(policy_batches) if policy_batches else None
-        return fresh_value_batch, fresh_policy_batch
+        """Runs search passes until ``value_sample_count`` root value samples exist, counting what the
+        previous call produced beyond its own request (:52-95).  Returns (value batch, policy batch)
+        of this call — the same batches that went to the buffers — or None where no pass ran."""
+        have = self.last_extra
+        values: list[RebelBatch] = []
+        policies: list[RebelBatch] = []
+        while have < value_sample_count:
+            value, pre_deal_value, policy = self.search_pass()
+            values += [value, pre_deal_value]
+            policies.append(policy)
+            have += len(value)
+        self.last_extra = have - value_sample_count
+        return (RebelBatch.cat(values) if values else None), (RebelBatch.cat(policies) if policies else None)

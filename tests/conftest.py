@@ -19,14 +19,15 @@ def golden_dir():
 
 def pytest_terminal_summary(terminalreporter):
     """What the element-wise comparisons of tests/parity.py measured in this session (exempt shares and
-    worst entries per tensor): printed, and kept in gpurun_out/ when that folder exists."""
+    worst entries per tensor): printed, and also written to the file that the environment variable
+    P2_PARITY_REPORT names, if it is set."""
     from tests import parity
     if not parity.MEASURED:
         return
     text = parity.measured_report()
     terminalreporter.write_sep("-", "parity: measured over this session")
     terminalreporter.write_line(text)
-    out = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out):
-        with open(os.path.join(out, "parity_measured.txt"), "w") as f:
+    out = os.environ.get("P2_PARITY_REPORT")
+    if out:
+        with open(out, "w") as f:
             f.write(text + "\n")

@@ -57,6 +57,25 @@ def same_but_few(big, ref, name, rtol=1e-3, atol=2e-4):
         f"{name}: {n_over} of {diff.numel()} over tolerance, max abs diff {float(diff.max()):.3e}"
 
 
+class RowWiseNetwork:
+    """A stand-in for the value network whose answer for a sample depends on that sample alone and has no
+    sum in it (the opponent's range, scaled by the board's ranks): no GEMM tiling, so a root's search
+    must give the same bits whatever batch it is part of."""
+
+    def eval(self):
+        pass
+
+    def __call__(self, f, include_policy=False):
+        from types import SimpleNamespace
+        b = f.beliefs.view(-1, 2, H).float()
+        ranks = torch.where(f.board >= 0, (f.board % 13).float(), torch.zeros_like(f.board, dtype=torch.float32))
+        return SimpleNamespace(hand_values=torch.flip(b, dims=[1]) * (40.0 + ranks.sum(dim=1))[:, None, None] - 0.01)
+
+
+STATE_TENSORS = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets", "regret_weight_sums",
+                 "self_reach", "self_reach_avg", "beliefs", "beliefs_avg", "latest_values", "values_avg")
+
+
 def rows_of_first_roots(ev, k):
     """Node rows that belong to roots 0..k-1, in row order (= the row order of a tree built from
     those roots alone: rows are level-major, parent-major)."""
@@ -79,12 +98,12 @@ def test_turn_subgames_with_chance_leaves_B512():
         for lin in net.linears:
             lin.weight.mul_(2.0)
 
-    def run(n, iters=iters):
+    def run(n, iters=iters, network=net):
         roots = RootStates.at_round_start(2, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards[:n],
                                           button=np.arange(n) % 2)
         # the configuration's own bet tree: bins {0.5, 1} pot + all-in, at most three raises
-        ev = HipSparseCFREvaluator(ChanceLeafModel(net, dev), dev, river_dcfr_config(n, iterations=iters, depth=16,
-                                                                                     dcfr_delay=0), max_raises=3)
+        ev = HipSparseCFREvaluator(ChanceLeafModel(network, dev), dev, river_dcfr_config(n, iterations=iters, depth=16,
+                                                                                         dcfr_delay=0), max_raises=3)
         ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs[:n]))
         ev.prepare_search(t_sample=torch.full((ev.total_nodes,), -1, dtype=torch.long))
         ev.run_search_iterations()
@@ -106,6 +125,14 @@ def test_turn_subgames_with_chance_leaves_B512():
     rows = torch.from_numpy(rows).to(DEV)
     for name in ("policy_probs_avg", "beliefs_avg", "values_avg"):
         same_but_few(getattr(ev, name)[rows], getattr(ref, name), name)
+    del ev, ref
+    # the same with a network that has no GEMM in it: every tensor of the first roots bit for bit, so the tolerance
+    # above is the network's and not the library's (expansion, mean and iteration do not depend on the batch)
+    ev = run(b, 6, RowWiseNetwork())
+    ref = run(small, 6, RowWiseNetwork())
+    assert float(ev.latest_values[ev.model_indices].abs().max()) > 1e-3
+    for name in STATE_TENSORS:
+        assert torch.equal(getattr(ev, name)[rows], getattr(ref, name)), name
 
 
 def test_data_generation_step_B16384():
@@ -122,10 +149,10 @@ def test_data_generation_step_B16384():
         for lin in net.linears:
             lin.weight.mul_(2.0)
 
-    def run(n, autocast, iters=iters):
+    def run(n, autocast, iters=iters, network=net):
         gen = torch.Generator(device=dev)
         gen.manual_seed(1)
-        model = NetworkLeafModel(net, dev, autocast_dtype=autocast)
+        model = NetworkLeafModel(network, dev, autocast_dtype=autocast)
         ev = HipSparseCFREvaluator(model, dev, river_dcfr_config(n, iterations=iters, depth=64), generator=gen,
                                    max_raises=3)
         ev.initialize_subgame(roots.select(np.arange(n)), np.arange(n), bel[:n])
@@ -157,6 +184,16 @@ def test_data_generation_step_B16384():
     rows = torch.from_numpy(rows).to(DEV)
     for name in ("policy_probs_avg", "beliefs_avg", "values_avg"):
         same_but_few(getattr(big, name)[rows], getattr(ref, name), name)
+    del big, ref
+    torch.cuda.empty_cache()
+    # and bit for bit with a network that has no GEMM in it (see the turn test above); the sampled policy is a
+    # snapshot at an iteration drawn per root from the generator, whose draws depend on the batch
+    big, _ = run(b, None, 6, RowWiseNetwork())
+    ref, _ = run(small, None, 6, RowWiseNetwork())
+    for name in STATE_TENSORS:
+        if name == "policy_probs_sample":
+            continue
+        assert torch.equal(getattr(big, name)[rows], getattr(ref, name)), name
 
 
 def test_generator_with_the_reference_production_settings():
