@@ -430,6 +430,12 @@ class HipSparseCFREvaluator:
         return rules_hip.showdown_value_both(beliefs, self.hand_rank_data, self._showdown_potential_f,
                                              self._showdown_scale, table_row=self._showdown_rows)
 
+    def _showdown_value(self, beliefs: torch.Tensor, hero: int) -> torch.Tensor:
+        """[M,H] showdown values of player ``hero`` at the showdown rows (cfr_evaluator.py:492-601); one
+        launch computes both players, so callers that want both use ``_showdown_value_both``."""
+        _req(hero in (0, 1), "hero in (0, 1)")
+        return self._showdown_value_both(beliefs)[:, hero]
+
     # ------------------------------------------------------------------ host-side scalars
     def _get_mixing_weights(self, t: int):
         """cfr_evaluator.py:285-303."""

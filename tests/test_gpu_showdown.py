@@ -174,3 +174,75 @@ def test_ev_from_strength_sorted_inputs_matches_oracle_and_refuses_bad_rows():
     with pytest.raises(NotImplementedError):
         F.showdown_ev_triton(b_sorted, c1, c2, dev(hrd.L_idx), dev(hrd.R_idx), eps=1e-6)
     torch.cuda.synchronize()
+
+
+# --- the remaining scenarios of the reference's showdown tests (tests/test_rebel_cfr_evaluator.py:1327-1472),
+# restated as data: board "Ac Kd Qh Js 9c", chips 100 each in a pot of 200 over a scale of 1000
+BROADWAY_BOARD = NAMED_BOARDS[6:7]
+
+
+def _scenario(K, villain_range):
+    from oracle import ranker as ORK
+    boards = BROADWAY_BOARD
+    allowed, prob = OC.allowed_hands_for_boards(boards)
+    bel = np.stack([prob, prob], axis=1).astype(np.float32)
+    bel[0, 1] = villain_range
+    pot = np.array([[100.0, 100.0]], dtype=np.float32)
+    scale = np.array([1000.0], dtype=np.float32)
+    out = run_hip(K, boards, bel, pot, scale)
+    np.testing.assert_allclose(out, oracle_both(boards, bel, pot, scale), rtol=RTOL, atol=ATOL)
+    combos = OC.hand_combos()
+    cards7 = np.concatenate([np.tile(boards[0], (H, 1)), combos], axis=1)
+    strength = ORK.rank_cards(cards7)          # board-blocked hands repeat a card; they are masked below
+    return out[0], strength, allowed[0]
+
+
+@pytest.mark.parametrize("villain", [(C(12, 0), C(11, 1)), (C(10, 2), C(9, 3)), (C(8, 0), C(7, 0)), (C(6, 1), C(5, 1))])
+def test_villain_holds_one_known_hand(K, villain):
+    """:1376-1437 — every compatible hero hand that beats the villain's wins the whole potential, every weaker
+    one loses it, equal ones and the villain's own hand get nothing."""
+    v = OC.combo_index(*villain)
+    rng = np.zeros(H, dtype=np.float32)
+    rng[v] = 1.0
+    ev, strength, allowed = _scenario(K, rng)
+    ok = allowed & OC.mask_conflicting(list(villain))
+    better, worse, ties = ok & (strength > strength[v]), ok & (strength < strength[v]), ok & (strength == strength[v])
+    assert better.any() or worse.any()
+    np.testing.assert_allclose(ev[0][better], 0.1, rtol=1e-6)
+    np.testing.assert_allclose(ev[0][worse], -0.1, rtol=1e-6)
+    assert np.all(ev[0][ties] == 0) and ev[0][v] == 0 and np.all(ev[0][~ok] == 0)
+
+
+def test_villain_holds_one_of_two_hands(K):
+    """:1440-1472 — half the mass on As Kh (aces and kings), half on Qd Jc (queens and jacks): a hand that beats
+    both wins the potential, one between them breaks even, one below both loses it."""
+    h1, h2 = OC.combo_index(C(12, 0), C(11, 1)), OC.combo_index(C(10, 2), C(9, 3))
+    rng = np.zeros(H, dtype=np.float32)
+    rng[h1] = rng[h2] = 0.5
+    ev, strength, allowed = _scenario(K, rng)
+    winner = OC.combo_index(C(8, 0), C(0, 1))      # Ts 2h: the ten completes the broadway straight
+    splitter = OC.combo_index(C(11, 0), C(10, 3))  # Ks Qc: beats QJ, loses to AK
+    loser = OC.combo_index(C(2, 0), C(0, 2))       # 4s 2d: loses to both
+    assert strength[winner] > max(strength[h1], strength[h2])
+    assert strength[h2] < strength[splitter] < strength[h1]
+    assert strength[loser] < min(strength[h1], strength[h2])
+    np.testing.assert_allclose(ev[0][[winner, splitter, loser]], [0.1, 0.0, -0.1], rtol=1e-6, atol=1e-9)
+
+
+def test_evaluator_answers_per_player_like_the_reference(K):
+    """`_showdown_value(beliefs, hero)` (cfr_evaluator.py:492) is the hero's half of `_showdown_value_both`."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(5)
+    boards = NAMED_BOARDS[[0, 3, 6]]
+    bel = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(3, np.full(3, 200), np.tile([[800, 800]], (3, 1)), boards)
+    ev = HipSparseCFREvaluator(None, torch.device("cuda"), river_dcfr_config(3, iterations=2, depth=2))
+    ev.initialize_subgame(roots, np.arange(3), torch.from_numpy(bel))
+    ev.prepare_search()
+    b = ev.beliefs[ev.showdown_indices]
+    both = ev._showdown_value_both(b)
+    assert both.shape == (ev.showdown_indices.numel(), 2, H) and float(both.abs().max()) > 0
+    for hero in (0, 1):
+        assert torch.equal(ev._showdown_value(b, hero), both[:, hero])
