@@ -237,14 +237,19 @@ def cases(repeats: int):
     del bel3, posr, den, uni, outc, vals3, vavg, regrets, actor_v, src_w, pavg, pol, reach_avg3, hv, last, outm
 
     # --- local best response, one tree level of the same search: the 16 384 parents of level 1, four
-    # children each (per parent: the actor's range, per child its policy row and both value rows in,
-    # both value rows of the parent out)
+    # children each.  Per parent: the actor's range in, both value rows out; per child both value rows in and,
+    # where the parent's actor is not the deviating player, its policy row (a deviating actor takes the maximum
+    # over its children and reads no policy).  A search asks for both players' best responses, so every parent
+    # is in either case once: here every second parent deviates.
     from . import _lib
     base, end = int(ev.depth_offsets[1]), int(ev.depth_offsets[2])
     n_par, n_ch = end - base, int(ev.child_count[base:end].sum())
-    deviator = torch.zeros(ev.total_nodes, dtype=torch.int64, device=dev)
+    deviator = ev.env.to_act.clone()
+    deviator[base + 1:end:2] = 1 - deviator[base + 1:end:2]
+    follows = deviator[base:end] != ev.env.to_act[base:end]
+    n_policy_rows = int(ev.child_count[base:end][follows].sum())
     vals = torch.rand(ev.total_nodes, 2, H, device=dev)
-    yield (f"best_response_level parents={n_par}", (3 * n_par + 3 * n_ch) * H * 4,
+    yield (f"best_response_level parents={n_par}", (3 * n_par + 2 * n_ch + n_policy_rows) * H * 4,
            lambda: _lib.call("p2hip_best_response_level", _lib.ptr(vals), _lib.ptr(ev.policy_probs_avg),
                              _lib.ptr(ev.beliefs), _lib.ptr(ev.env.to_act), _lib.ptr(deviator),
                              _lib.ptr(ev.child_offsets), _lib.ptr(ev.child_count), base, n_par,

@@ -183,11 +183,13 @@ def flop_expand(pre_chance_beliefs: torch.Tensor, root_indices: torch.Tensor, fl
     return post
 
 
-# Workgroups wanted from the (state, player) x share split of the flop means.  perm_mean keeps six
-# workgroups per CU resident, so 2048 leave a second, quarter-full round (1024 states x 256 flops:
-# 812 us with one share, 688 us with two, 670 us with three); orbit_mean is lighter per row and fastest
-# with the fewest shares that fill the chip once (470 us against 494 us with two).
-PERM_MEAN_TARGET_WORKGROUPS = 4096
+# Workgroups wanted from the (state, player) x share split of the flop means.  perm_mean is a pure read stream
+# (the permutations are applied once per workgroup, to the summed rows) and fastest with few, long workgroups:
+# 64 states x 256 flops 48.6 us with one share (128 workgroups), 30.5 us with three (384), 32.3 us with eight,
+# 44.2 us with 32; 1024 states 475 us with one share, 505 us with two.  orbit_mean goes through LDS per row and
+# wants the chip filled once (1024 states x 256 flops: 470 us with one share against 494 us with two; 64
+# states: 32.8 us with eight shares).
+PERM_MEAN_TARGET_WORKGROUPS = 384
 ORBIT_MEAN_TARGET_WORKGROUPS = 2048   # 256 CUs x 8
 
 

@@ -138,12 +138,13 @@ __global__ __launch_bounds__(FLAT_BLOCK) void regret_matching_divide_kernel(
   }
 }
 
-// K4 -- fused_cfr_triton.py:409-435; grid (M, 2)
+// K4 -- fused_cfr_triton.py:409-435; two workgroups per row, neighbours in the grid: together they read and write the
+// row's two players as one contiguous run
 __global__ __launch_bounds__(OPS_BLOCK) void weight_child_values_kernel(
     const float* __restrict__ values, const int64_t* __restrict__ prev_actor, const float* __restrict__ pol_hero,
     const float* __restrict__ pol_opp, float* __restrict__ out) {
-  const int64_t m = blockIdx.x;
-  const int p = blockIdx.y;
+  const int64_t m = blockIdx.x >> 1;
+  const int p = blockIdx.x & 1;
   const bool hero = (int64_t)p == prev_actor[m];
   const float2* v2 = p2_row2(values, m * 2 + p);
   const float2* w2 = p2_row2(hero ? pol_hero : pol_opp, m);
@@ -380,13 +381,13 @@ __global__ __launch_bounds__(OPS_BLOCK) void model_values_mix_zs_kernel(
   }
 }
 
-// K14 -- fused_cfr_triton.py:1787-1835; grid (parents, 2)
+// K14 -- fused_cfr_triton.py:1787-1835; two workgroups per parent (one per player), neighbours in the grid
 __global__ __launch_bounds__(OPS_BLOCK) void weighted_parent_sum_kernel(
     float* __restrict__ values, const int64_t* __restrict__ prev_actor, const float* __restrict__ pol_hero,
     const float* __restrict__ pol_opp, const int64_t* __restrict__ child_offsets,
     const int64_t* __restrict__ child_count, int64_t parent_base) {
-  const int64_t p = blockIdx.x;
-  const int player = blockIdx.y;
+  const int64_t p = blockIdx.x >> 1;
+  const int player = blockIdx.x & 1;
   const int64_t first = child_offsets[p];
   const int count = (int)child_count[p];
   if (count == 0) return;  // leaf at an intermediate depth keeps its value
@@ -576,7 +577,8 @@ int p2hip_weight_child_values(const float* values, const int64_t* prev_actor, co
   if (m == 0) return 0;
   P2_REQ(values && prev_actor && policy_hero && policy_opp && out);
   P2_REQ(p2_aligned8(values) && p2_aligned8(policy_hero) && p2_aligned8(policy_opp) && p2_aligned8(out));
-  hipLaunchKernelGGL(p2::weight_child_values_kernel, dim3((unsigned)m, 2), dim3(p2::OPS_BLOCK), 0, P2_ST, values,
+  P2_REQ(m <= 0x3FFFFFFF);
+  hipLaunchKernelGGL(p2::weight_child_values_kernel, dim3((unsigned)(2 * m)), dim3(p2::OPS_BLOCK), 0, P2_ST, values,
                      prev_actor, policy_hero, policy_opp, out);
   P2_LAUNCH_CHECK();
   return 0;
@@ -704,7 +706,8 @@ int p2hip_weighted_parent_sum(float* values, const int64_t* prev_actor, const fl
   if (num_parents == 0) return 0;
   P2_REQ(values && prev_actor && policy_hero && policy_opp && child_offsets && child_count);
   P2_REQ(p2_aligned8(values) && p2_aligned8(policy_hero) && p2_aligned8(policy_opp));
-  hipLaunchKernelGGL(p2::weighted_parent_sum_kernel, dim3((unsigned)num_parents, 2), dim3(p2::OPS_BLOCK), 0, P2_ST,
+  P2_REQ(num_parents <= 0x3FFFFFFF);
+  hipLaunchKernelGGL(p2::weighted_parent_sum_kernel, dim3((unsigned)(2 * num_parents)), dim3(p2::OPS_BLOCK), 0, P2_ST,
                      values, prev_actor, policy_hero, policy_opp, child_offsets, child_count, parent_base);
   P2_LAUNCH_CHECK();
   return 0;

@@ -368,14 +368,14 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
   }
 }
 
-// expected[i][p][h] = mean over the samples of state i.  blockIdx.y picks the player: a workgroup walks the
+// expected[i][p][h] = mean over the samples of state i.  The low bit of blockIdx.x picks the player: a workgroup walks the
 // whole 5304-byte rows of one player through all samples of its state (three pairs per lane), four
 // samples' rows in flight at a time.
 __global__ __launch_bounds__(CH_BLOCK) void chance_mean_kernel(const float* __restrict__ hand_values,
                                                                 const int64_t* __restrict__ sample_offsets,
                                                                 float* __restrict__ expected) {
-  const int64_t i = blockIdx.x;
-  const int p = blockIdx.y;
+  const int64_t i = blockIdx.x >> 1;
+  const int p = blockIdx.x & 1;
   const int64_t s0 = sample_offsets[i], s1 = sample_offsets[i + 1];
   float2 acc[CH_PPT];
 #pragma unroll
@@ -614,155 +614,82 @@ __global__ __launch_bounds__(CH_BLOCK) void flop_expand_lines_kernel(const float
 
 // out[i][p][h] (+)= sum_f weight[f] * mean_q hand_values[i][f][p][perms[q][h]]
 // (the suit-orbit mean of _avg_over_perms, chance_node_helper.py:18-28, and the weighted sum over
-// flops, :352-357).  A workgroup takes one (state, player) and one contiguous share of the flops:
-// each row goes through LDS once (the next one is already in flight in registers while the current
-// one is gathered), the permutation table is packed two hands per dword - in registers for up to
-// CH_REG_PERMS permutations, in LDS beyond - and the sums run in fp64.  With more than one share
-// the workgroups write partial sums that perm_reduce_kernel adds in a fixed order.
+// flops, :352-357).  The permutations of a call are the same for all of its flops (the reference draws
+// them once per chunk of flops, chance_node_helper.py:318-329), and the gather is linear, so
+//   sum_f w[f] * mean_q hv[f][perm_q[h]]  =  mean_q Y[perm_q[h]]   with   Y[j] = sum_f w[f] * hv[f][j]:
+// a workgroup takes one (state, player) and one contiguous share of the flops, adds the weighted rows of its
+// share hand by hand in fp64 registers - a pure read stream, CH_ROWS rows in flight per lane - and applies the
+// permutations ONCE, to the sums staged in LDS, instead of once per row.  With more than one share the
+// workgroups write partial results that perm_reduce_kernel adds in a fixed order.
 constexpr int CH_MAX_PERMS = 24;
-constexpr int CH_REG_PERMS = 8;
+constexpr int CH_ROWS = 4;   // rows requested together
 __global__ __launch_bounds__(CH_BLOCK) void perm_mean_kernel(const float* __restrict__ hand_values,
                                                               const int16_t* __restrict__ perms, int n_perms,
                                                               const float* __restrict__ weight, int64_t n_flops,
                                                               int64_t flops_per_share, int accumulate,
                                                               float* __restrict__ dst, int64_t dst_share_stride) {
-  extern __shared__ __align__(16) unsigned char lds_raw[];
-  float* rows = reinterpret_cast<float*>(lds_raw);                                  // [2][H + 2]
-  uint32_t* ptab = reinterpret_cast<uint32_t*>(lds_raw + 2 * (P2_H + 2) * 4);       // [n_perms][HPAIRS]
+  __shared__ double y[P2_H + 2];
   const int64_t i = blockIdx.x >> 1;
   const int p = blockIdx.x & 1;
   const int64_t f0 = (int64_t)blockIdx.y * flops_per_share;
   const int64_t f1 = f0 + flops_per_share < n_flops ? f0 + flops_per_share : n_flops;
-  const bool in_regs = n_perms <= CH_REG_PERMS;
-  uint32_t preg[CH_REG_PERMS][CH_PPT];
-#pragma unroll
-  for (int q = 0; q < CH_REG_PERMS; ++q)
-#pragma unroll
-    for (int k = 0; k < CH_PPT; ++k) {
-      const int idx = threadIdx.x + k * CH_BLOCK;
-      preg[q][k] = (in_regs && q < n_perms && idx < P2_HPAIRS)
-                       ? reinterpret_cast<const uint32_t*>(perms + (int64_t)q * P2_H)[idx] : 0u;
-    }
-  if (!in_regs)
-    for (int e = threadIdx.x; e < n_perms * P2_HPAIRS; e += CH_BLOCK) {
-      const int q = e / P2_HPAIRS, idx = e - q * P2_HPAIRS;
-      ptab[e] = reinterpret_cast<const uint32_t*>(perms + (int64_t)q * P2_H)[idx];
-    }
   double acc[CH_PPT][2];
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) acc[k][0] = acc[k][1] = 0.0;
-  const float inv_perms = 1.0f / (float)n_perms;
-  if (in_regs) {
-    // Two rows per step, interleaved hand by hand in LDS: one 64-bit gather serves both rows (the gathers
-    // keep the LDS pipe busy most of the time; this halves their number) and six row pieces are in flight
-    // per lane instead of three.  A share with an odd number of rows repeats its last row with weight 0.
-    float2* pairs = reinterpret_cast<float2*>(lds_raw);            // [2][H + 2] of (row f, row f + 1)
-    float2 na[CH_PPT], nb[CH_PPT];
-    auto fetch2 = [&](int64_t f) {
-      const float2* a = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
-      const float2* b = p2_row2(hand_values, ((int64_t)i * n_flops + (f + 1 < f1 ? f + 1 : f)) * 2 + p);
+  // rows beyond the share's end repeat its last row with weight 0: straight-line loads, no branch per row
+  float2 cur[CH_ROWS][CH_PPT], nxt[CH_ROWS][CH_PPT];
+  auto fetch = [&](int64_t f, float2 (&r)[CH_ROWS][CH_PPT]) {
+#pragma unroll
+    for (int j = 0; j < CH_ROWS; ++j) {
+      const int64_t fj = f + j < f1 ? f + j : f1 - 1;
+      const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + fj) * 2 + p);
 #pragma unroll
       for (int k = 0; k < CH_PPT; ++k) {
         const int idx = threadIdx.x + k * CH_BLOCK;
-        na[k] = a[idx < P2_HPAIRS ? idx : 0];
-        nb[k] = b[idx < P2_HPAIRS ? idx : 0];
+        r[j][k] = src[idx < P2_HPAIRS ? idx : 0];
       }
-    };
-    if (f0 < f1) fetch2(f0);
-    int buf = 0;
-    for (int64_t f = f0; f < f1; f += 2, buf ^= 1) {
-      float2* row = pairs + buf * (P2_H + 2);
-#pragma unroll
-      for (int k = 0; k < CH_PPT; ++k) {
-        const int idx = threadIdx.x + k * CH_BLOCK;
-        if (idx < P2_HPAIRS)
-          reinterpret_cast<float4*>(row)[idx] = make_float4(na[k].x, nb[k].x, na[k].y, nb[k].y);
-      }
-      if (f + 2 < f1) fetch2(f + 2);
-      p2_sync_lds();   // rows f, f+1 are complete; the other buffer was consumed before this barrier
-      const float wa = weight[f] * inv_perms;
-      const float wb = f + 1 < f1 ? weight[f + 1] * inv_perms : 0.f;
-#pragma unroll
-      for (int k = 0; k < CH_PPT; ++k) {
-        const int idx = threadIdx.x + k * CH_BLOCK;
-        if (idx >= P2_HPAIRS) continue;
-        float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
-#pragma unroll
-        for (int q = 0; q < CH_REG_PERMS; ++q)
-          if (q < n_perms) {
-            const float2 u = row[preg[q][k] & 0xFFFFu], v = row[preg[q][k] >> 16];
-            a0 += u.x; b0 += u.y;
-            a1 += v.x; b1 += v.y;
-          }
-        acc[k][0] += (double)(wa * a0);
-        acc[k][1] += (double)(wa * a1);
-        if (f + 1 < f1) {
-          acc[k][0] += (double)(wb * b0);
-          acc[k][1] += (double)(wb * b1);
-        }
-      }
-    }
-    float2* o = p2_row2(dst + (int64_t)blockIdx.y * dst_share_stride, i * 2 + p);
-#pragma unroll
-    for (int k = 0; k < CH_PPT; ++k) {
-      const int idx = threadIdx.x + k * CH_BLOCK;
-      if (idx >= P2_HPAIRS) continue;
-      const float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
-      o[idx] = make_float2(prev.x + (float)acc[k][0], prev.y + (float)acc[k][1]);
-    }
-    return;
-  }
-  float2 next[CH_PPT];
-  auto fetch = [&](int64_t f) {
-    const float2* src = p2_row2(hand_values, ((int64_t)i * n_flops + f) * 2 + p);
-#pragma unroll
-    for (int k = 0; k < CH_PPT; ++k) {
-      const int idx = threadIdx.x + k * CH_BLOCK;
-      next[k] = idx < P2_HPAIRS ? src[idx] : make_float2(0.f, 0.f);
     }
   };
-  if (f0 < f1) fetch(f0);
-  int buf = 0;
-  for (int64_t f = f0; f < f1; ++f, buf ^= 1) {
-    float* row = rows + buf * (P2_H + 2);
+  if (f0 < f1) fetch(f0, cur);
+  for (int64_t f = f0; f < f1; f += CH_ROWS) {
+    if (f + CH_ROWS < f1) fetch(f + CH_ROWS, nxt);
 #pragma unroll
-    for (int k = 0; k < CH_PPT; ++k) {
-      const int idx = threadIdx.x + k * CH_BLOCK;
-      if (idx < P2_HPAIRS) reinterpret_cast<float2*>(row)[idx] = next[k];
-    }
-    if (f + 1 < f1) fetch(f + 1);
-    p2_sync_lds();   // row f is complete; the other buffer (row f-1) was consumed before this barrier
-    const float w = weight[f] * inv_perms;
+    for (int j = 0; j < CH_ROWS; ++j) {
+      const double w = f + j < f1 ? (double)weight[f + j] : 0.0;
 #pragma unroll
-    for (int k = 0; k < CH_PPT; ++k) {
-      const int idx = threadIdx.x + k * CH_BLOCK;
-      if (idx >= P2_HPAIRS) continue;
-      float s0 = 0.f, s1 = 0.f;
-      if (in_regs) {
-#pragma unroll
-        for (int q = 0; q < CH_REG_PERMS; ++q)
-          if (q < n_perms) {
-            s0 += row[preg[q][k] & 0xFFFFu];
-            s1 += row[preg[q][k] >> 16];
-          }
-      } else {
-        for (int q = 0; q < n_perms; ++q) {
-          const uint32_t e = ptab[q * P2_HPAIRS + idx];
-          s0 += row[e & 0xFFFFu];
-          s1 += row[e >> 16];
-        }
+      for (int k = 0; k < CH_PPT; ++k) {
+        acc[k][0] += w * (double)cur[j][k].x;   // the product of two floats is exact in fp64
+        acc[k][1] += w * (double)cur[j][k].y;
       }
-      acc[k][0] += (double)(w * s0);
-      acc[k][1] += (double)(w * s1);
+    }
+#pragma unroll
+    for (int j = 0; j < CH_ROWS; ++j)
+#pragma unroll
+      for (int k = 0; k < CH_PPT; ++k) cur[j][k] = nxt[j][k];
+  }
+#pragma unroll
+  for (int k = 0; k < CH_PPT; ++k) {
+    const int idx = threadIdx.x + k * CH_BLOCK;
+    if (idx < P2_HPAIRS) {
+      y[2 * idx] = acc[k][0];
+      y[2 * idx + 1] = acc[k][1];
     }
   }
+  p2_sync_lds();
+  const double inv_perms = 1.0 / (double)n_perms;
   float2* o = p2_row2(dst + (int64_t)blockIdx.y * dst_share_stride, i * 2 + p);
 #pragma unroll
   for (int k = 0; k < CH_PPT; ++k) {
     const int idx = threadIdx.x + k * CH_BLOCK;
     if (idx >= P2_HPAIRS) continue;
+    double s0 = 0.0, s1 = 0.0;
+    for (int q = 0; q < n_perms; ++q) {
+      const uint32_t e = reinterpret_cast<const uint32_t*>(perms + (int64_t)q * P2_H)[idx];   // two hands per dword
+      s0 += y[e & 0xFFFFu];
+      s1 += y[e >> 16];
+    }
     const float2 prev = accumulate ? o[idx] : make_float2(0.f, 0.f);
-    o[idx] = make_float2(prev.x + (float)acc[k][0], prev.y + (float)acc[k][1]);
+    o[idx] = make_float2(prev.x + (float)(s0 * inv_perms), prev.y + (float)(s1 * inv_perms));
   }
 }
 
@@ -928,7 +855,10 @@ int p2hip_chance_mean(const float* hand_values, const int64_t* sample_offsets, i
   if (n == 0) return 0;
   if (!hand_values || !sample_offsets || !expected) return P2_EINVAL;
   if (!p2_aligned8(hand_values) || !p2_aligned8(expected)) return P2_EINVAL;
-  hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)n, 2), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
+  if (n > 0x3FFFFFFF) return P2_EINVAL;
+  // the two players of a state on neighbouring workgroups: together they read the state's samples as one
+  // contiguous run (3584 turn states: 345 -> 328 us against all of player 0's workgroups before player 1's)
+  hipLaunchKernelGGL(p2::chance_mean_kernel, dim3((unsigned)(2 * n)), dim3(p2::CH_BLOCK), 0, (hipStream_t)stream,
                      hand_values, sample_offsets, expected);
   P2_LAUNCH_CHECK();
   return 0;
@@ -973,13 +903,7 @@ int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const 
   if (((uintptr_t)perms & 3) != 0) return P2_EINVAL;
   if (n > 0x3FFFFFFF || shares > 65535) return P2_EINVAL;
   if (shares > 1 && (!workspace || !p2_aligned8(workspace))) return P2_EINVAL;
-  const size_t lds = n_perms > p2::CH_REG_PERMS ? (size_t)2 * (P2_H + 2) * 4 + (size_t)n_perms * P2_HPAIRS * 4
-                                                : (size_t)2 * (P2_H + 2) * 8;   // 74 KB with all 24, or 21 KB
-  if (lds > 64 * 1024) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(p2::perm_mean_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-  }
+  const size_t lds = 0;
   const int64_t per_share = (n_flops + shares - 1) / shares;
   const int64_t npairs = n * 2 * P2_HPAIRS;
   if (shares == 1) {
