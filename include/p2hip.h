@@ -120,9 +120,11 @@ int p2hip_flop_expand(const float* pre_beliefs, const int64_t* root_indices, int
 
 /* out [n,2,H] (+= if accumulate) sum_f weight[f] * mean_q hand_values[i][f][p][perms[q][h]]:
  * hand_values [n, n_flops, 2, H], perms int16 [n_perms <= 24, H] hand permutations, 4-byte aligned
- * (the suit-orbit mean of _avg_over_perms, :18-28, and the weighted flop sum, :352-357).
+ * (the suit-orbit mean of _avg_over_perms, :18-28, and the weighted flop sum, :352-357).  Evaluated as
+ * mean_q Y[perms[q][h]] with Y = sum_f weight[f] * hand_values[i][f][p] summed in float64 - the same
+ * number, since the permutations do not depend on the flop: a read stream and one permutation pass.
  * shares >= 1 splits the flops over that many workgroups per (state, player) - use it when
- * 2 * n alone does not fill the GPU; shares > 1 needs workspace [shares, n, 2, H] float32, whose
+ * 2 * n alone leaves most of the GPU idle (a few hundred workgroups are enough); shares > 1 needs workspace [shares, n, 2, H] float32, whose
  * partial sums are added in ascending order (results do not depend on scheduling). */
 int p2hip_perm_mean(const float* hand_values, int64_t n, int64_t n_flops, const int16_t* perms, int n_perms,
                     const float* weight, int accumulate, float* out, float* workspace, int shares, void* stream);
