@@ -126,6 +126,10 @@ def cases(repeats: int):
     post, _, _, offsets = CH.chance_expand(pre, roots, tb, cards_on_board=4)
     yield ("chance_expand states=3584 x48", k * (2 + 2 * 48) * H * 4,
            lambda: CH.chance_expand(pre, roots, tb, cards_on_board=4, check_rows=False))
+    # the same expansion written as rows of a value network's input matrix: [ranges | board one-hot], 2704 elements
+    for name, dt, size in (("float32", torch.float32, 4), ("bfloat16", torch.bfloat16, 2)):
+        yield (f"chance_expand -> input rows {name}", k * (2 * H * 4 + 48 * 2704 * size),
+               lambda dt=dt: CH.chance_expand(pre, roots, tb, cards_on_board=4, check_rows=False, input_dtype=dt))
     yield ("chance_mean states=3584 x48", k * (2 * 48 + 2) * H * 4, lambda: CH.chance_mean(post, offsets))
     del post
 

@@ -324,34 +324,62 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
   const int remaining = P2_CARDS - ncards - 1;          // cards left for the hands of a sample
   const float uniform = 1.0f / fmaxf((float)(remaining * (remaining - 1) / 2), 1.0f);
   uint4* out = reinterpret_cast<uint4*>(post_beliefs);
-  const int64_t g0 = s_first * ROW_UNITS, g1 = g0 + (int64_t)count * ROW_UNITS;   // 16-byte units of the workgroup
-  for (int64_t g = (g0 & ~7ll) + threadIdx.x; g < g1; g += CH_BLOCK) {
-    if (g < g0) continue;
-    const uint32_t local = (uint32_t)(g - g0);
-    const uint32_t m = local / ROW_UNITS, j = local - m * ROW_UNITS;
+  const int64_t g0 = s_first * ROW_UNITS;                // first 16-byte unit of the workgroup
+  const uint32_t units = (uint32_t)count * ROW_UNITS;    // at most 13 x 676
+  // Lanes sit on absolute 128-byte lines (8 units): lane l takes units l - lead, l - lead + 256, ... of the
+  // workgroup's run.  The sample m and the unit j inside its row follow by one division and then by increments
+  // (a row has more than 256 units).
+  static_assert(ROW_UNITS > CH_BLOCK, "one row boundary per step at most");
+  const uint32_t lead = (uint32_t)(g0 & 7);
+  uint32_t local = threadIdx.x >= lead ? threadIdx.x - lead : threadIdx.x - lead + CH_BLOCK;
+  uint32_t m = local / ROW_UNITS, j = local - m * ROW_UNITS;
+  for (; local < units; local += CH_BLOCK, j += CH_BLOCK) {
+    if (j >= (uint32_t)ROW_UNITS) { j -= ROW_UNITS; ++m; }
     const ChanceSample sm = sample[m];
     float xs[UNIT];
-    uint32_t cd[UNIT];
+    uint32_t pk[UNIT / 2];                               // a | b << 8 of two hands per word
 #pragma unroll
     for (int u = 0; u < UNIT / 4; ++u) {
       // a unit behind the ranges (board one-hot only) reads the last padded quad: its values are not used
       const uint32_t quad = min(j * (UNIT / 4) + u, (uint32_t)(2 * P2_H + CH_LDS_PAD) / 4 - 1);
       const float4 x = reinterpret_cast<const float4*>(t)[quad];
-      const uint2 pk = reinterpret_cast<const uint2*>(cards_of)[quad];
+      const uint2 c2 = reinterpret_cast<const uint2*>(cards_of)[quad];
       xs[4 * u] = x.x; xs[4 * u + 1] = x.y; xs[4 * u + 2] = x.z; xs[4 * u + 3] = x.w;
-      cd[4 * u] = pk.x & 0xFFFFu; cd[4 * u + 1] = pk.x >> 16; cd[4 * u + 2] = pk.y & 0xFFFFu; cd[4 * u + 3] = pk.y >> 16;
+      pk[2 * u] = c2.x; pk[2 * u + 1] = c2.y;
     }
-    const uint64_t dealt = bits | (1ull << sm.card);   // the sample's board as a card set
+    const uint32_t e0 = UNIT * j;                        // first element of the unit in its row
     float r[UNIT];
+    if (sm.inv0 != 0.f && sm.inv1 != 0.f) {
+      // both players have mass left: value x 1 / mass, zero for a hand that holds the dealt card.  Two hands per
+      // word: a byte of (cards ^ dealt card in every byte) is zero exactly where a card equals the dealt one.
+      // Cards are below 64, so with bit 7 of every byte set first, subtracting 1 from every byte borrows from
+      // no neighbour and clears bit 7 exactly in the bytes that were zero.
+      const uint32_t rep = (uint32_t)sm.card * 0x01010101u;
 #pragma unroll
-    for (int q = 0; q < UNIT; ++q) {
-      const uint32_t e = UNIT * j + q;                  // element of the row
-      const float inv = (e >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
-      const uint32_t a = cd[q] & 0xFFu, b = cd[q] >> 8;
-      float val = xs[q] * inv;
-      if (inv == 0.f) val = (((bits >> a) | (bits >> b)) & 1ull) ? 0.f : uniform;   // no mass left: uniform
-      r[q] = (a == (uint32_t)sm.card || b == (uint32_t)sm.card) ? 0.f : val;
-      if (INPUT_ROWS && e >= (uint32_t)(2 * P2_H)) r[q] = ((dealt >> (e - 2 * P2_H)) & 1ull) ? 1.f : 0.f;
+      for (int w = 0; w < UNIT / 2; ++w) {
+        // ranges end at an even element and units start at multiples of 4: both hands of a word are one player's
+        const float inv = (e0 + 2 * w >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
+        const uint32_t x = pk[w] ^ rep;
+        const uint32_t z = ~((x | 0x80808080u) - 0x01010101u) & 0x80808080u;
+        r[2 * w] = (z & 0x00008080u) ? 0.f : xs[2 * w] * inv;
+        r[2 * w + 1] = (z & 0x80800000u) ? 0.f : xs[2 * w + 1] * inv;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < UNIT; ++q) {
+        const float inv = (e0 + q >= (uint32_t)P2_H) ? sm.inv1 : sm.inv0;
+        const uint32_t cd = (pk[q / 2] >> (16 * (q & 1))) & 0xFFFFu;
+        const uint32_t a = cd & 0xFFu, b = cd >> 8;
+        float val = xs[q] * inv;
+        if (inv == 0.f) val = (((bits >> a) | (bits >> b)) & 1ull) ? 0.f : uniform;   // no mass left: uniform
+        r[q] = (a == (uint32_t)sm.card || b == (uint32_t)sm.card) ? 0.f : val;
+      }
+    }
+    if (INPUT_ROWS && e0 + UNIT > (uint32_t)(2 * P2_H)) {
+      const uint64_t dealt = bits | (1ull << sm.card);   // the sample's board as a card set
+#pragma unroll
+      for (int q = 0; q < UNIT; ++q)
+        if (e0 + q >= (uint32_t)(2 * P2_H)) r[q] = ((dealt >> (e0 + q - 2 * P2_H)) & 1ull) ? 1.f : 0.f;
     }
     uint4 w;
     if (DT == 0) {
@@ -364,7 +392,7 @@ __global__ __launch_bounds__(CH_BLOCK) void chance_expand_lines_kernel(const flo
       w = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4 % UNIT], r[5 % UNIT]),
                      pack_f16(r[6 % UNIT], r[7 % UNIT]));
     }
-    out[g] = w;
+    out[g0 + local] = w;
   }
 }
 
