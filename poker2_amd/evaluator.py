@@ -43,7 +43,7 @@ from .chance_node_helper import ChanceNodeHelper
 from .rebel_batch import RebelBatch
 from .rebel_feature_encoder import RebelFeatureEncoder
 from .tree import (CARDS_ON_STREET, RootStates, SparseTree, build_sparse_tree, build_sparse_tree_device,
-                   split_work_items)
+                   launch_order, split_work_items)
 from ._guards import require as _req
 
 STATE_NAMES = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
@@ -83,9 +83,10 @@ SPLIT_CUT_LEVEL = 2
 # families another (six launches per iteration instead of four).
 SPLIT_MID_LEVEL = 1
 # Trees with raises (57 and 105 nodes per root against 21) gain from the cut at every batch size: their
-# subtrees differ in size and the items are started largest first (three raises: 1024 roots 3.96 -> 3.73 ms,
-# 4096 roots 14.75 -> 14.41 ms; two raises: 1024 roots 2.15 -> 2.07 ms, 4096 roots 7.93 -> 7.76 ms; the
-# 21-node trees lose 3-7 % above 400 roots).
+# subtrees differ in size, so whole roots leave long tails (three raises: 1024 roots 3.96 -> 3.73 ms,
+# 4096 roots 14.75 -> 14.41 ms with all items started largest first, -> 12.8 ms with the items in row order
+# and only the last rounds' items by size; two raises: 1024 roots 2.15 -> 2.07 ms, 4096 roots 7.93 -> 7.76 ms;
+# the 21-node trees lose 3-7 % above 400 roots).
 SPLIT_NODES_PER_ROOT = 50
 
 
@@ -147,6 +148,9 @@ class HipSparseCFREvaluator:
             raise ValueError("HipSparseCFREvaluator requires a GPU device.")
         if not F.triton_is_available():
             raise RuntimeError("libp2hip.so or a GPU is not available; HipSparseCFREvaluator has no other backend.")
+        # work items of the last three rounds of a launch start largest first (tree.launch_order): the
+        # iteration kernel keeps three workgroups per compute unit resident
+        self._sorted_tail = 3 * 3 * int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         if getattr(cfg.env, "flop_showdown", False):
             raise NotImplementedError("the env's flop_showdown game variant (showdown right after the preflop round, "
                                       "hunl_tensor_env.py:900) is not built; the tree builders follow the full game")
@@ -352,11 +356,13 @@ class HipSparseCFREvaluator:
                               else self._items)
         self._root_items = None
         if self._items is None and T:
-            # Roots of unequal size (mixed streets, stacks, pots): one work item per root, largest tree
-            # first, so that the launch does not end on a long root that started last.
+            # Roots of unequal size (mixed streets, stacks, pots): one work item per root, largest tree first, so
+            # that the launch does not end on a long root that started last.  (Row order with only the last
+            # rounds by size, which wins for the work items of equal trees, loses here: 16 384 mixed roots 23.2 ms
+            # per iteration against 22.3 ms.)
             size = np.bincount(tree.root_index, minlength=N)
             if size.min() != size.max():
-                order = np.argsort(-size, kind="stable").astype(np.int64)
+                order = launch_order(size, N)
 
                 def per_item(mask):
                     rows = np.nonzero(mask)[0]
@@ -373,7 +379,10 @@ class HipSparseCFREvaluator:
 
     def _split_items(self, tree: SparseTree, mid_level: int | None = None):
         """``tree.split_work_items`` with the arrays on the device (None if the tree is too shallow to cut)."""
-        it = split_work_items(tree, self.root_nodes, SPLIT_CUT_LEVEL, mid_level)
+        # equal trees: items in row order, the last rounds' items by size; roots of unequal size: all by size
+        sizes = np.bincount(tree.root_index, minlength=self.root_nodes)
+        tail = self._sorted_tail if sizes.min() == sizes.max() else tree.total
+        it = split_work_items(tree, self.root_nodes, SPLIT_CUT_LEVEL, mid_level, sorted_tail=tail)
         if it is None:
             return None
         for name in ("parents", "parent_offsets", "showdown", "showdown_offsets", "item_root", "item_top"):

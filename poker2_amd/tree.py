@@ -339,7 +339,29 @@ def build_sparse_tree(roots: RootStates, bet_bins: list[float], depth: int,
                       reward=reward, state=state, board=np.array(roots.board))
 
 
-def split_work_items(tree: "SparseTree", n_roots: int, cut_level: int, mid_level: int | None = None):
+# Items that start in the last rounds of a launch are started largest first; three rounds of the 768
+# workgroups an MI355X holds at a time (3 per compute unit x 256).
+SORTED_TAIL_ITEMS = 3 * 768
+
+
+def launch_order(size: np.ndarray, sorted_tail: int = SORTED_TAIL_ITEMS) -> np.ndarray:
+    """Order in which work items of the given sizes are handed to the compute units: ascending index —
+    items that run at the same time then work on neighbouring rows of every tensor, which the memory
+    system rewards (4096 three-raise roots: 11.2 ms per iteration with all items sorted by size, 10.3 ms
+    this way) — except that the last ``sorted_tail`` items come largest first: a launch lasts until its last
+    item ends, so the long ones must not be the ones that start last.  A launch of fewer items than that is
+    sorted by size as a whole."""
+    n = len(size)
+    order = np.arange(n)
+    w = min(int(sorted_tail), n)
+    if w > 0:
+        tail = order[n - w:]
+        order = np.concatenate([order[:n - w], tail[np.argsort(-np.asarray(size)[tail], kind="stable")]])
+    return order.astype(np.int64)
+
+
+def split_work_items(tree: "SparseTree", n_roots: int, cut_level: int, mid_level: int | None = None,
+                     sorted_tail: int = SORTED_TAIL_ITEMS):
     """Work items for the iteration kernel when a root gets several workgroups (include/p2hip.h), in
     tiers: tier 0 holds one item per root, the top of its tree above the first cut level; every further
     tier one item per node of its cut level that has children, with the families from that level down
@@ -391,12 +413,10 @@ def split_work_items(tree: "SparseTree", n_roots: int, cut_level: int, mid_level
         sd_rows = sd_rows[tree.showdown_mask[sd_rows]]
         sd_rows = sd_rows[np.isin(anchor[sd_rows], heads)]
         ts, tso = grouped(sd_rows, anchor[sd_rows], heads)
-        # Largest items first: a launch lasts until its last work item ends, and items are handed to
-        # the compute units in index order, so the long ones must not be the ones that start last.
         below = np.arange(offs[lo], offs[hi + 1] if hi < n_levels else T)
         below = below[np.isin(anchor[below], heads)]
         size = np.bincount(np.searchsorted(heads, anchor[below]), minlength=len(heads))
-        order = np.argsort(-size, kind="stable")
+        order = launch_order(size, sorted_tail)
         lists_p.append(reordered(tp, tpo, order))
         lists_s.append(reordered(ts, tso, order))
         heads = heads[order]

@@ -120,8 +120,9 @@ def test_roots_of_the_flop_showdown_variant_are_refused():
 def test_work_items_partition_the_tree(seed):
     """split_work_items on random trees and cut levels: every family and every showdown row belongs to
     exactly one item; an item's rows lie under its head (tier 0: under its root) and inside its tier's
-    levels; a showdown row sits in the item that owns its parent's family; inside a tier the items come
-    largest first; the tiers' counts add up."""
+    levels; a showdown row sits in the item that owns its parent's family; inside a tier the items come in
+    row order except for a tail of stated length that comes largest first (the whole tier when it is
+    shorter than that); the tiers' counts add up."""
     from poker2_amd.tree import split_work_items
     rng = np.random.default_rng(900 + seed)
     n = int(rng.integers(1, 6))
@@ -134,7 +135,8 @@ def test_work_items_partition_the_tree(seed):
     level = np.searchsorted(offs, np.arange(tree.total), side="right") - 1
     has_children = tree.child_count > 0
     for cut, mid in ((1, None), (2, None), (2, 1), (9, None), (9, 1), (9, 2)):
-        it = split_work_items(tree, n, cut, mid)
+        tail = [10 ** 6, 3, 0][(seed + cut) % 3]        # longer than any tier / a few items / none
+        it = split_work_items(tree, n, cut, mid, sorted_tail=tail)
         if it is None:
             assert len(offs) - 1 < 3 or not has_children[offs[1]:].any()
             continue
@@ -161,7 +163,7 @@ def test_work_items_partition_the_tree(seed):
                         up[deeper] = tree.parent_index[up[deeper]]
                     assert (up == heads[0]).all()
                 owner[rows] = w
-            if tier > 0:                       # largest first, by the rows from the head down to the next cut
+            if tier > 0:                       # order of the items, by the rows from the head down to the next cut
                 hi_level = min(bounds[tier + 1], len(offs) - 2)
                 below = np.arange(offs[bounds[tier]], offs[hi_level + 1])
                 top = below.copy()
@@ -170,7 +172,19 @@ def test_work_items_partition_the_tree(seed):
                     top[deeper] = tree.parent_index[top[deeper]]
                 head_of = [it.parents[it.parent_offsets[w]] for w in range(first_item[tier], first_item[tier + 1])]
                 rows_under = [int((top == h).sum()) for h in head_of]
-                assert all(a >= b for a, b in zip(rows_under, rows_under[1:]))
+                k = max(0, len(head_of) - tail)                                            # items before the tail
+                assert all(a < b for a, b in zip(head_of[:k], head_of[1:k]))                # in row order
+                assert all(a >= b for a, b in zip(rows_under[k:], rows_under[k + 1:]))      # then largest first
+                assert sorted(head_of[k:]) == sorted(head_of)[k:]                          # the tail holds the last heads
         for w in range(len(it.item_root)):
             sd = it.showdown[it.showdown_offsets[w]:it.showdown_offsets[w + 1]]
             assert (owner[tree.parent_index[sd]] == w).all()                               # with its parent's family
+
+
+def test_launch_order_keeps_row_order_and_sorts_the_tail():
+    from poker2_amd.tree import launch_order
+    size = np.array([5, 1, 9, 3, 3, 7, 2, 8])
+    assert launch_order(size, 0).tolist() == list(range(8))
+    assert launch_order(size, 3).tolist() == [0, 1, 2, 3, 4, 7, 5, 6]                     # 7, 2, 8 -> 8, 7, 2
+    assert launch_order(size, 100).tolist() == [2, 7, 5, 0, 3, 4, 6, 1]                   # all by size, ties in row order
+    assert launch_order(np.zeros(0, dtype=np.int64)).tolist() == []
