@@ -397,7 +397,8 @@ typedef struct P2HipIterArgs {
    * children (item_top = 0); every family and showdown row belongs to exactly one item.  An iteration
    * is then four launches: all items with phases 4, top items with 8, subtree items with 8|2, top items
    * with 2 (the regret part of a family reads rows that the reach / belief part of the family above
-   * rewrites, so it runs everywhere first). */
+   * rewrites, so it runs everywhere first).  The tops may be cut again the same way (tiers of items:
+   * reach / belief parts tier by tier downwards, value parts upwards; two launches more per cut). */
   const int64_t* item_root;
   const uint8_t* item_top;
   /* Optional, [total,2,H]: reach_avg as the PREVIOUS iteration left it, in a buffer of its own.  The

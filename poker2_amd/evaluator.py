@@ -78,9 +78,11 @@ _PHASE_LEAN = 16
 # half the tree, deeper cuts put more of the tree into the few top items.
 SPLIT_ROOTS_BELOW = 400
 SPLIT_CUT_LEVEL = 2
-# With few roots the tree tops (one workgroup per root, five families in a row) are themselves too few and
-# too long: a second cut right under the root makes the root's family one item and each of its children's
-# families another (six launches per iteration instead of four).
+# The tree tops (one workgroup per root, five families in a row) are few and long: a second cut right under
+# the root makes the root's family one item and each of its children's families another (six launches per
+# iteration instead of four).  First made for few roots (192 roots: 0.80 -> 0.77 ms), it pays at every batch
+# size: 4096 three-raise roots 10.84 -> 10.41 ms per search iteration, 13.79 -> 12.75 ms per plain one; 2048
+# roots 5.52 -> 5.28 ms; 1024 roots unchanged (2.86 ms); 512 roots 1.46 -> 1.40 ms.
 SPLIT_MID_LEVEL = 1
 # Trees with raises (57 and 105 nodes per root against 21) gain from the cut at every batch size: their
 # subtrees differ in size, so whole roots leave long tails (three raises: 1024 roots 3.96 -> 3.73 ms,
@@ -349,7 +351,7 @@ class HipSparseCFREvaluator:
         split = self.split_small_batches
         if split is None:
             split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
-        self._items = self._split_items(tree, SPLIT_MID_LEVEL if N < SPLIT_ROOTS_BELOW else None) if split else None
+        self._items = self._split_items(tree, SPLIT_MID_LEVEL) if split else None
         # The regret part has no order among families: it runs over the coarser of the two partitions
         # (whole tree tops), which makes fewer and longer workgroups of the same work.
         self._items_regret = (self._split_items(tree) if self._items is not None and len(self._items.tiers) > 2
