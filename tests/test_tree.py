@@ -134,7 +134,7 @@ def test_work_items_partition_the_tree(seed):
     offs = np.asarray(tree.depth_offsets)
     level = np.searchsorted(offs, np.arange(tree.total), side="right") - 1
     has_children = tree.child_count > 0
-    for cut, mid in ((1, None), (2, None), (2, 1), (9, None), (9, 1), (9, 2)):
+    for cut, mid in ((1, None), (2, None), (2, 1), (9, None), (9, 1), (9, 2), (3, (1, 2)), (9, (1, 3))):
         tail = [10 ** 6, 3, 0][(seed + cut) % 3]        # longer than any tier / a few items / none
         it = split_work_items(tree, n, cut, mid, sorted_tail=tail)
         if it is None:
