@@ -205,8 +205,8 @@ class HipSparseCFREvaluator:
         self._skip_t_scalars_update = False
         self._skip_record_stats = True
         self._fused_positive_regrets_buf = None
-        self._fscal = torch.zeros(8, dtype=torch.float32, device=self.device)
-        self._iscal = torch.zeros(8, dtype=torch.int64, device=self.device)
+        self._fscal = self._t_scalars.floats      # the one-kernel iteration reads the first eight
+        self._iscal = self._t_scalars.ints
         self._fscal_host = (ctypes.c_float * 8)()
         self._iscal_host = (ctypes.c_int64 * 8)()
         self._iter_bundles: dict = {}
@@ -481,8 +481,6 @@ class HipSparseCFREvaluator:
         any captured region (fused_sparse_cfr_evaluator.py:535-550)."""
         self.apply_schedules(t)
         mix_old, mix_new = self._get_mixing_weights(t)
-        self._t_scalars.update(t=t, dcfr_alpha=self.dcfr_alpha, dcfr_beta=self.dcfr_beta,
-                               mix_old=float(mix_old), mix_new=float(mix_new))
         apply_dcfr = self.cfr_type in (CFRType.discounted, CFRType.discounted_plus)
         (a, a_den), (b, b_den) = F.discount_pair(t, self.dcfr_alpha), F.discount_pair(t, self.dcfr_beta)
         total = float(mix_old) + float(mix_new)
@@ -497,8 +495,10 @@ class HipSparseCFREvaluator:
         i[0], i[1], i[2] = int(t), int(apply_dcfr), int(self.cfr_plus and not linear)
         i[6], i[7] = int(self.cfr_avg), int(linear)
         i[3], i[4], i[5] = int(self._avg_policy_copies(t)), int(self.enforce_zero_sum), int(not self.use_final_policy_values)
-        _lib.call("p2hip_write_scalars", _lib.ptr(self._fscal), _lib.ptr(self._iscal),
-                  ctypes.cast(f, ctypes.c_void_p), ctypes.cast(i, ctypes.c_void_p), _lib.stream_ptr())
+        # one launch for every scalar of the iteration (the per-operation kernels read the same array
+        # through the 0-D views of ``_t_scalars``); the de-averaging pair only where something reads it
+        needs_pair = self.cfr_avg or not self.fused_iteration
+        self._t_scalars.write(f, i, F.TScalars.deaveraging_factors(mix_old, mix_new) if needs_pair else None)
 
     def _get_sampling_schedule(self) -> torch.Tensor:
         """cfr_evaluator.py:382-404: per-root iteration at which the policy is snapshotted."""

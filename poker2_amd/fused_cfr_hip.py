@@ -12,6 +12,7 @@ be replayed for any ``t``.
 """
 from __future__ import annotations
 
+import ctypes
 from enum import Enum
 
 import torch
@@ -636,40 +637,74 @@ def fused_sample_snapshot_(policy_probs_sample, policy_probs, t_sample, t_tensor
 # --------------------------------------------------------------------------- TScalars
 class TScalars:
     """0-D device tensors holding the iteration-dependent scalars (fused_cfr_triton.py:2100-2158).
-    ``update`` copies host values in and must run outside any captured region."""
+    ``update`` copies host values in and must run outside any captured region.
+
+    On the GPU the float scalars are views into one array (``floats``: alpha and beta numerators,
+    their denominators, mix_old, mix_new, their sum, its reciprocal, then mix_onon and mix_oon) and
+    ``t_tensor`` is element 0 of ``ints``, so that one small launch that carries the values as kernel
+    arguments refreshes all of them (a ``fill_`` per scalar is eleven launches, 50-60 us of an
+    iteration however small the batch).  The first eight floats and the eight ints are the arrays the
+    one-kernel iteration reads."""
+
+    _NAMES = ("t_alpha_num", "t_beta_num", "t_alpha_den", "t_beta_den", "mix_old", "mix_new", "mix_total",
+              "mix_inv_total", "mix_onon", "mix_oon")
 
     def __init__(self, device: torch.device, dtype: torch.dtype = torch.float32) -> None:
-        def _z():
-            return torch.zeros((), dtype=dtype, device=device)
-
-        self.device = device
+        self.device = torch.device(device)
         self.dtype = dtype
-        self.t_alpha_num = _z()
-        self.t_beta_num = _z()
-        self.t_alpha_den = _z()
-        self.t_beta_den = _z()
-        self.mix_old = _z()
-        self.mix_new = _z()
-        self.mix_total = _z()
-        self.mix_inv_total = _z()
-        self.mix_onon = _z()
-        self.mix_oon = _z()
-        self.t_tensor = torch.zeros((), dtype=torch.long, device=device)
+        self._packed = self.device.type == "cuda" and dtype == torch.float32
+        if self._packed:
+            self.floats = torch.zeros(16, dtype=torch.float32, device=device)
+            self.ints = torch.zeros(8, dtype=torch.int64, device=device)
+            for k, name in enumerate(self._NAMES):
+                setattr(self, name, self.floats[k])
+            self.t_tensor = self.ints[0]
+            self._host_f = (ctypes.c_float * 8)()
+            self._host_i = (ctypes.c_int64 * 8)()
+            self._host_x = (ctypes.c_float * 8)()
+        else:
+            for name in self._NAMES:
+                setattr(self, name, torch.zeros((), dtype=dtype, device=device))
+            self.t_tensor = torch.zeros((), dtype=torch.long, device=device)
+
+    def write(self, host_f, host_i, onon_oon: tuple[float, float] | None = None) -> None:
+        """``floats[:8]`` and ``ints[:8]`` from two host arrays of eight (ctypes float / int64), and the
+        two CFR-AVG de-averaging factors if given: one launch, or two."""
+        _req(self._packed, "TScalars.write: float32 scalars on the GPU")
+        _lib.call("p2hip_write_scalars", _lib.ptr(self.floats), _lib.ptr(self.ints),
+                  ctypes.cast(host_f, ctypes.c_void_p), ctypes.cast(host_i, ctypes.c_void_p), _lib.stream_ptr())
+        if onon_oon is not None:
+            x = self._host_x
+            x[0], x[1] = onon_oon
+            _lib.call("p2hip_upload_floats", _lib.ptr(self.floats) + 8 * 4, ctypes.cast(x, ctypes.c_void_p), 2,
+                      _lib.stream_ptr())
+
+    @staticmethod
+    def deaveraging_factors(mix_old: float, mix_new: float) -> tuple[float, float] | None:
+        """(total / new, old / new) of the CFR-AVG de-averaging; None while ``mix_new`` is zero (the
+        scalars then keep their last values, fused_cfr_triton.py:2150-2156)."""
+        if float(mix_new) == 0.0:
+            return None
+        return (float(mix_old) + float(mix_new)) / float(mix_new), float(mix_old) / float(mix_new)
 
     def update(self, t: int, dcfr_alpha: float, dcfr_beta: float, mix_old: float, mix_new: float) -> None:
         (t_alpha_num, t_alpha_den), (t_beta_num, t_beta_den) = discount_pair(t, dcfr_alpha), discount_pair(t, dcfr_beta)
-        self.t_alpha_num.fill_(t_alpha_num)
-        self.t_beta_num.fill_(t_beta_num)
-        self.t_alpha_den.fill_(t_alpha_den)
-        self.t_beta_den.fill_(t_beta_den)
         total = float(mix_old) + float(mix_new)
-        self.mix_old.fill_(float(mix_old))
-        self.mix_new.fill_(float(mix_new))
-        self.mix_total.fill_(total)
-        self.mix_inv_total.fill_(1.0 / total if total != 0.0 else 1.0)
-        if float(mix_new) != 0.0:
-            self.mix_onon.fill_(total / float(mix_new))
-            self.mix_oon.fill_(float(mix_old) / float(mix_new))
+        inv_total = 1.0 / total if total != 0.0 else 1.0
+        extra = self.deaveraging_factors(mix_old, mix_new)
+        if self._packed:
+            f, i = self._host_f, self._host_i
+            f[0], f[1], f[2], f[3] = t_alpha_num, t_beta_num, t_alpha_den, t_beta_den
+            f[4], f[5], f[6], f[7] = float(mix_old), float(mix_new), total, inv_total
+            i[0] = int(t)                      # ints[1:] belong to whoever reads them: zero here
+            self.write(f, i, extra)
+            return
+        for name, value in zip(self._NAMES[:8], (t_alpha_num, t_beta_num, t_alpha_den, t_beta_den, float(mix_old),
+                                                 float(mix_new), total, inv_total)):
+            getattr(self, name).fill_(value)
+        if extra is not None:
+            self.mix_onon.fill_(extra[0])
+            self.mix_oon.fill_(extra[1])
         self.t_tensor.fill_(int(t))
 
 
