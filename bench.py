@@ -79,7 +79,7 @@ def synth_roots(n: int, seed: int):
     return boards, x.astype(np.float32)
 
 
-def make_evaluator(n_roots: int, tree: str, seed: int, iterations: int):
+def make_evaluator(n_roots: int, tree: str, seed: int, iterations: int, spread_state: bool = False):
     import torch
     from poker2_amd.config import river_dcfr_config
     from poker2_amd.evaluator import HipSparseCFREvaluator
@@ -89,7 +89,8 @@ def make_evaluator(n_roots: int, tree: str, seed: int, iterations: int):
     roots = RootStates.at_round_start(3, np.full(n_roots, 200), np.tile([[800, 800]], (n_roots, 1)), boards,
                                       button=np.arange(n_roots) % 2)
     cfg = river_dcfr_config(n_roots, iterations=iterations, depth=depth, dcfr_delay=0)
-    ev = HipSparseCFREvaluator(None, torch.device("cuda"), cfg, fused_iteration=True, max_raises=max_raises)
+    ev = HipSparseCFREvaluator(None, torch.device("cuda"), cfg, fused_iteration=True, max_raises=max_raises,
+                               spread_state=spread_state)
     ev.initialize_subgame(roots, np.arange(n_roots), torch.from_numpy(beliefs))
     ev.prepare_search()
     return ev, boards, beliefs
@@ -290,6 +291,9 @@ def main() -> None:
     ap.add_argument("--mode", choices=sorted(MODES), default="search",
                     help="search: the iterations as a search runs all but its last; plain: every tensor written in full")
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--no-spread", action="store_true",
+                    help="allocate the state tensors back to back (the evaluator's default) instead of each behind "
+                         "a held block of device memory (its spread_state option, made for long searches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -312,7 +316,14 @@ def main() -> None:
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    ev, _, _ = make_evaluator(args.roots, args.tree, args.seed, iterations=args.warmup + args.steps + 1)
+    torch.zeros(1, device="cuda")
+    torch.cuda.synchronize()
+    t_build = time.perf_counter()
+    ev, _, _ = make_evaluator(args.roots, args.tree, args.seed, iterations=args.warmup + args.steps + 1,
+                              spread_state=not args.no_spread)
+    torch.cuda.synchronize()
+    t_build = time.perf_counter() - t_build
+    placed = ev.state_spread_count
     nodes_per_root = ev.total_nodes // ev.root_nodes
     launches = 1 if ev._items is None else 2 * len(ev._items.tiers)
 
@@ -375,7 +386,11 @@ def main() -> None:
                    "roots": args.roots, "nodes_per_root": nodes_per_root, "total_nodes": total_nodes,
                    "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0",
                    "mode": args.mode, "mode_note": mode_text[args.mode],
-                   "launches_per_iteration": launches},
+                   "launches_per_iteration": launches,
+                   "state_placement": {"spread_state": not args.no_spread, "tensors_allocated_behind_a_held_block": placed,
+                                       "subgame_construction_s": t_build,
+                                       "note": "evaluator option for long searches: each state tensor is allocated while a "
+                                               "9 GiB block reserved just before it is held; outside the timed region"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic,

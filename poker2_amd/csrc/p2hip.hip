@@ -11,10 +11,11 @@
 #include "tree.hip"
 #include "datagen.hip"
 #include "stream_probe.hip"
+#include "placement.hip"
 
 extern "C" {
 // Library / ABI version, bumped whenever an exported signature changes.
-int p2hip_abi_version(void) { return 4; }
+int p2hip_abi_version(void) { return 5; }
 // Number of visible HIP devices (0 when there is none); never throws.
 int p2hip_device_count(void) {
   int n = 0;

@@ -77,6 +77,12 @@ _PHASE_LEAN = 16
 # 0.38 -> 0.42; a cut right under the root leaves subtrees whose chain of families is as long as
 # half the tree, deeper cuts put more of the tree into the few top items.
 SPLIT_ROOTS_BELOW = 400
+# Placement of the state tensors (``HipSparseCFREvaluator._new_state``).  The block held while a tensor is
+# allocated: no effect up to 5 GiB, part of it at 6 and 7 GiB, all of it from 8 GiB on (4096 three-raise
+# roots, first process on a machine: 11.18 / 10.68 / 10.57 / 10.49 / 10.47 / 10.50 ms per iteration with
+# 5 / 6 / 7 / 8 / 9 / 12 GiB).  Tensors below the minimum size are allocated as they come.
+STATE_SPREAD_GAP_BYTES = 9 << 30
+STATE_SPREAD_MIN_TENSOR_BYTES = 256 << 20
 SPLIT_CUT_LEVEL = 2
 # The tree tops (one workgroup per root, five families in a row) are few and long: a second cut right under
 # the root makes the root's family one item and each of its children's families another (six launches per
@@ -137,7 +143,8 @@ class HipSparseCFREvaluator:
     def __init__(self, model, device, cfg, generator: torch.Generator | None = None, *,
                  compile_model: bool = True, fused_iteration: bool = True,
                  max_raises: int | None = None, tree_builder: str = "device",
-                 split_small_batches: bool | None = None, lean_search: bool = True) -> None:
+                 split_small_batches: bool | None = None, lean_search: bool = True,
+                 spread_state: bool = False) -> None:
         self.device = torch.device(device)
         if model is not None and not hasattr(model, "leaf_values"):
             # the reference hands its network over as is (cfr_evaluator.py:306-322, 1025-1047): its
@@ -194,6 +201,12 @@ class HipSparseCFREvaluator:
         # iteration are not stored) and lets reach_avg alternate between two buffers; the final state is
         # bit-identical either way.  False: every iteration as ``cfr_iteration`` runs it.
         self.lean_search = bool(lean_search)
+        # True: each large state tensor is allocated while a block of STATE_SPREAD_GAP_BYTES, reserved
+        # just before it, is held (``_new_state``: 5-10 % faster iterations; free in a fresh process,
+        # seconds per subgame once the card's memory has been used and given back, so it is for long
+        # searches).  ``state_spread_count``: for how many tensors of the current subgame that was done
+        self.spread_state = bool(spread_state)
+        self.state_spread_count = 0
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -224,6 +237,43 @@ class HipSparseCFREvaluator:
         if dtype is not None:
             t = t.to(dtype)
         return t.to(self.device)
+
+    def _hold_gap(self, nbytes: int) -> ctypes.c_void_p | None:
+        """A block of device memory to hold while ``nbytes`` are allocated, or None where that would
+        not pay or not fit: small tensors, an allocator that would answer from blocks it has cached
+        (they lie where they lie), or a card too full to take the block without pressure."""
+        if not self.spread_state or nbytes < STATE_SPREAD_MIN_TENSOR_BYTES:
+            return None
+        if torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device) >= nbytes:
+            return None
+        free, total = torch.cuda.mem_get_info(self.device)
+        if free - nbytes - STATE_SPREAD_GAP_BYTES < total // 4:
+            return None
+        block = ctypes.c_void_p()
+        code = _lib.load().p2hip_device_reserve(STATE_SPREAD_GAP_BYTES, ctypes.byref(block))
+        return block if code == 0 and block.value else None
+
+    def _new_state(self, *shape: int) -> torch.Tensor:
+        """Zeros of the float dtype for a state tensor of the search.  Where the tensors lie in the
+        card's memory changes the speed of the iteration kernel by 5-10 % (4096 three-raise river roots:
+        11.1 ms per iteration with the tensors allocated back to back by a fresh process, 10.5 ms this
+        way; the depth-2 tree 1.90 -> 1.71 ms; 1024 three-raise roots 2.67-2.82 -> 2.57 ms): with
+        ``spread_state`` each one is allocated while a block of 9 GiB, reserved just before it and released
+        right after, is held.  One block held during the whole construction, blocks before some of the
+        tensors only, address space reserved without memory behind it, tensor bases aligned to 1 GiB or
+        staggered by 0.2-33 MB: none of these changes anything.  Cost: nothing measurable in a process
+        that is the first to use the memory (4096 roots: 1.19 against 1.15 s of construction); 0.15-0.45 s
+        per tensor once memory has been used and released before (the driver clears what it hands out
+        again: 2.3-5.5 s per subgame), which only a long search earns back.  Hence an option, off by
+        default."""
+        nbytes = 4 * int(np.prod(shape))
+        block = self._hold_gap(nbytes)
+        try:
+            return torch.zeros(*shape, dtype=self.float_dtype, device=self.device)
+        finally:
+            if block is not None:
+                self.state_spread_count += 1
+                _lib.call("p2hip_device_release", block)
 
     def _construct_subgame(self, src_env, src_indices) -> None:
         """Build the sparse tree and allocate the state (sparse_cfr_evaluator.py:142-306)."""
@@ -299,28 +349,30 @@ class HipSparseCFREvaluator:
         self.showdown_potential = d_potential[self.showdown_indices]
         self._potential_all = d_potential.to(torch.float32)
 
+        self.state_spread_count = 0
+
         def z1():
-            return torch.zeros(T, NUM_HANDS, dtype=self.float_dtype, device=dev)
+            return self._new_state(T, NUM_HANDS)
 
         def z2():
-            return torch.zeros(T, 2, NUM_HANDS, dtype=self.float_dtype, device=dev)
+            return self._new_state(T, 2, NUM_HANDS)
 
         self.policy_probs, self.policy_probs_avg, self.policy_probs_sample = z1(), z1(), z1()
         self.cumulative_regrets, self.regret_weight_sums = z1(), z1()
-        self.uniform_policy = z1()
+        self.uniform_policy = torch.zeros(T, NUM_HANDS, dtype=self.float_dtype, device=dev)
         cc_dest = self.child_count[:tree.top].repeat_interleave(self.child_count[:tree.top])
         self.uniform_policy[N:] = (1.0 / cc_dest)[:, None].expand(-1, NUM_HANDS)
         self.beliefs, self.beliefs_avg = z2(), z2()
         self.root_pre_chance_beliefs = torch.zeros(N, 2, NUM_HANDS, dtype=self.float_dtype, device=dev)
         self.self_reach = z2()
         self.self_reach[:N] = 1.0
-        self.self_reach_avg = self.self_reach.clone()
+        self.self_reach_avg = z2().copy_(self.self_reach)
         self.latest_values = z2()
         folded = tt("fold_mask", tree.fold_mask)
         rew = tt("reward", tree.reward)
         self.latest_values[folded, 0] = rew[folded][:, None]
         self.latest_values[folded, 1] = -rew[folded][:, None]
-        self.values_avg = self.latest_values.clone()
+        self.values_avg = z2().copy_(self.latest_values)
         self.last_model_values = None
         self._scratch = z1()
         flags = np.zeros(T, dtype=np.uint8)
@@ -738,7 +790,7 @@ class HipSparseCFREvaluator:
     def _other_reach_avg(self) -> torch.Tensor:
         """The second reach_avg buffer of the alternating scheme (allocated on first use; root rows 1)."""
         if self._reach_avg_alt is None or self._reach_avg_alt.shape != self.self_reach_avg.shape:
-            self._reach_avg_alt = torch.empty_like(self.self_reach_avg)
+            self._reach_avg_alt = self._new_state(*self.self_reach_avg.shape)
             self._reach_avg_alt[:self.root_nodes] = 1.0
         return self._reach_avg_alt
 
