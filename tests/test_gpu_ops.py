@@ -367,6 +367,37 @@ def test_unblocked_mass_at_every_buffer_alignment_and_ragged_row_counts(rows):
     assert np.array_equal(got[0], got[1])
 
 
+def test_tscalars_update_fills_every_scalar_with_one_array_behind_them(F):
+    """TScalars.update (fused_cfr_triton.py:2131-2158): every 0-D tensor holds what the reference's fills
+    would leave, the de-averaging pair keeps its last values while mix_new is zero, and on the GPU all of
+    them are views of one array (refreshed by a launch or two instead of eleven)."""
+    sc = F.TScalars(torch.device("cuda"))
+    expect = {}
+
+    def check(t, alpha, beta, old, new):
+        sc.update(t, alpha, beta, old, new)
+        (an, ad), (bn, bd) = F.discount_pair(t, alpha), F.discount_pair(t, beta)
+        total = float(old) + float(new)
+        expect.update(t_alpha_num=an, t_alpha_den=ad, t_beta_num=bn, t_beta_den=bd, mix_old=old, mix_new=new,
+                      mix_total=total, mix_inv_total=1.0 / total if total else 1.0)
+        if new != 0.0:
+            expect.update(mix_onon=total / new, mix_oon=old / new)
+        for name, value in expect.items():
+            got = getattr(sc, name)
+            assert got.dim() == 0 and got.dtype == torch.float32
+            assert float(got) == np.float32(value), (name, t)
+        assert sc.t_tensor.dim() == 0 and sc.t_tensor.dtype == torch.int64 and int(sc.t_tensor) == t
+
+    expect.update(mix_onon=0.0, mix_oon=0.0)
+    check(0, 1.5, -1.0, 1.0, 0.0)          # mix_new = 0: the pair stays as it was
+    check(7, 1.5, 0.0, 10.5, 3.0)
+    check(8, 1.5, 0.5, 4.0, 0.0)           # and keeps the values of t = 7 here
+    check(50, 2.0, -1.0, 0.0, 2.0)
+    base = sc.floats.data_ptr()
+    assert [getattr(sc, n).data_ptr() - base for n in F.TScalars._NAMES] == [4 * k for k in range(10)]
+    assert sc.t_tensor.data_ptr() == sc.ints.data_ptr()
+
+
 def test_stream_probe_moves_what_it_says():
     """The measurement aid behind bench.py's flat-stream figure: every output array holds the sum of the input
     arrays plus its own number (so every load and every store happens), and unsupported mixes are refused."""
