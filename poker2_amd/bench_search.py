@@ -1,7 +1,7 @@
 """Whole river searches, wall clock: tree construction + state set-up, the DCFR iterations with
 their leaf sampling (``evaluate_cfr``), and the local exploitability afterwards.
 
-    python -m poker2_amd.bench_search [--roots 1024] [--max-raises 3] [--depth 16] [--iterations 200] [--json]
+    python -m poker2_amd.bench_search [--roots 1024] [--max-raises 3] [--depth 16] [--iterations 200] [--spread-state] [--json]
 
 Roots: random 5-card boards, Gamma(0.5) ranges with board-blocked hands removed, pot 200, stacks
 800 each, bet bins {0.5, 1.5} pot, no leaf network (river trees end in folds and showdowns).  The
@@ -46,6 +46,9 @@ def main() -> None:
     ap.add_argument("--depth", type=int, default=16)
     ap.add_argument("--iterations", type=int, default=200)
     ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--spread-state", action="store_true",
+                    help="the evaluator's placement option for long searches: faster iterations from 2048 roots on, "
+                         "set-up seconds longer once the card's memory has been used before")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -57,7 +60,8 @@ def main() -> None:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         cfg = river_dcfr_config(n, iterations=args.iterations, depth=args.depth, dcfr_delay=0)
-        ev = HipSparseCFREvaluator(None, dev, cfg, fused_iteration=True, max_raises=args.max_raises)
+        ev = HipSparseCFREvaluator(None, dev, cfg, fused_iteration=True, max_raises=args.max_raises,
+                                   spread_state=args.spread_state)
         ev.initialize_subgame(roots, np.arange(n), bel)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
@@ -68,13 +72,15 @@ def main() -> None:
         torch.cuda.synchronize()
         t3 = time.perf_counter()
     out = {"roots": n, "nodes": int(ev.total_nodes), "iterations": args.iterations,
+           "spread_state": bool(args.spread_state), "state_tensors_placed": int(ev.state_spread_count),
            "setup_s": t1 - t0, "search_s": t2 - t1, "exploitability_s": t3 - t2,
            "subgame_iterations_per_s": n * args.iterations / (t2 - t1),
            "local_exploitability": float(stats.local_exploitability.mean())}
     if args.json:
         print(json.dumps(out))
     else:
-        print(f"{n} roots, {out['nodes']} nodes: set-up {out['setup_s']:.3f} s, {args.iterations} iterations "
+        placed = f" ({out['state_tensors_placed']} state tensors placed)" if args.spread_state else ""
+        print(f"{n} roots, {out['nodes']} nodes: set-up {out['setup_s']:.3f} s{placed}, {args.iterations} iterations "
               f"{out['search_s']:.3f} s -> {out['subgame_iterations_per_s'] / 1e6:.3f} M subgame-iterations/s, "
               f"exploitability pass {1e3 * out['exploitability_s']:.1f} ms "
               f"(mean local exploitability {out['local_exploitability']:.4g})")
