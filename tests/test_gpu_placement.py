@@ -70,6 +70,7 @@ def test_spread_state_changes_where_the_state_lies_and_nothing_else(monkeypatch)
     assert plain.state_spread_count == 0
     torch.cuda.synchronize()
     free_before, _ = torch.cuda.mem_get_info()
+    cached_before = torch.cuda.memory_reserved()
     spread = _search(True, 0)
     # cached blocks of the allocator may serve some of the tensors; the others went behind a block
     assert 0 <= spread.state_spread_count <= 13
@@ -77,7 +78,8 @@ def test_spread_state_changes_where_the_state_lies_and_nothing_else(monkeypatch)
         assert torch.equal(getattr(plain, name), getattr(spread, name)), name
     torch.cuda.synchronize()
     free_after, _ = torch.cuda.mem_get_info()
-    assert free_before - free_after < 40 << 20, "the held blocks were given back"
+    grown = torch.cuda.memory_reserved() - cached_before          # what the tensors' allocator took meanwhile
+    assert (free_before - free_after) - grown < 16 << 20, "the held blocks were given back"
 
 
 def test_spread_state_places_tensors_when_the_allocator_has_nothing_cached(monkeypatch):
