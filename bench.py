@@ -292,8 +292,8 @@ def main() -> None:
                     help="search: the iterations as a search runs all but its last; plain: every tensor written in full")
     ap.add_argument("--seed", type=int, default=42)
     ap.add_argument("--no-spread", action="store_true",
-                    help="allocate the state tensors back to back (the evaluator's default) instead of each behind "
-                         "a held block of device memory (its spread_state option, made for long searches)")
+                    help="allocate the state tensors as they come (the evaluator's default) instead of dealing them to two "
+                         "slabs in different thirds of the card's memory (its spread_state option, made for long searches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -323,7 +323,7 @@ def main() -> None:
                               spread_state=not args.no_spread)
     torch.cuda.synchronize()
     t_build = time.perf_counter() - t_build
-    placed = ev.state_spread_count
+    placed = dict(ev.state_placement)
     nodes_per_root = ev.total_nodes // ev.root_nodes
     launches = 1 if ev._items is None else 2 * len(ev._items.tiers)
 
@@ -387,10 +387,11 @@ def main() -> None:
                    "cfr": "discounted alpha=1.5 beta=0 gamma=2, cfr_plus=False, delay=0",
                    "mode": args.mode, "mode_note": mode_text[args.mode],
                    "launches_per_iteration": launches,
-                   "state_placement": {"spread_state": not args.no_spread, "tensors_allocated_behind_a_held_block": placed,
+                   "state_placement": {"spread_state": not args.no_spread, **placed,
                                        "subgame_construction_s": t_build,
-                                       "note": "evaluator option for long searches: each state tensor is allocated while a "
-                                               "9 GiB block reserved just before it is held; outside the timed region"}},
+                                       "note": "evaluator option for long searches: the state tensors are dealt to two slabs "
+                                               "in different thirds of the card's memory, the second chosen by a measured "
+                                               "probe; outside the timed region"}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic,

@@ -74,6 +74,7 @@ _SIGNATURES: dict[str, list] = {
     "p2hip_cfr_iteration": [_P, _L, _I, _I, _P],
     "p2hip_write_scalars": [_P, _P, _P, _P, _P],
     "p2hip_stream_probe": [_P, _P, _L, _I, _I, _I, _P],
+    "p2hip_placement_probe": [_P, _P, _L, _I, _P, _P],
     "p2hip_device_reserve": [_L, _P],
     "p2hip_device_release": [_P],
 }

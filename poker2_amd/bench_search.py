@@ -72,14 +72,14 @@ def main() -> None:
         torch.cuda.synchronize()
         t3 = time.perf_counter()
     out = {"roots": n, "nodes": int(ev.total_nodes), "iterations": args.iterations,
-           "spread_state": bool(args.spread_state), "state_tensors_placed": int(ev.state_spread_count),
+           "spread_state": bool(args.spread_state), "state_placed": bool(ev.state_placement.get("placed")),
            "setup_s": t1 - t0, "search_s": t2 - t1, "exploitability_s": t3 - t2,
            "subgame_iterations_per_s": n * args.iterations / (t2 - t1),
            "local_exploitability": float(stats.local_exploitability.mean())}
     if args.json:
         print(json.dumps(out))
     else:
-        placed = f" ({out['state_tensors_placed']} state tensors placed)" if args.spread_state else ""
+        placed = (" (state placed)" if out["state_placed"] else " (state not placed)") if args.spread_state else ""
         print(f"{n} roots, {out['nodes']} nodes: set-up {out['setup_s']:.3f} s{placed}, {args.iterations} iterations "
               f"{out['search_s']:.3f} s -> {out['subgame_iterations_per_s'] / 1e6:.3f} M subgame-iterations/s, "
               f"exploitability pass {1e3 * out['exploitability_s']:.1f} ms "

@@ -77,12 +77,18 @@ _PHASE_LEAN = 16
 # 0.38 -> 0.42; a cut right under the root leaves subtrees whose chain of families is as long as
 # half the tree, deeper cuts put more of the tree into the few top items.
 SPLIT_ROOTS_BELOW = 400
-# Placement of the state tensors (``HipSparseCFREvaluator._new_state``).  The block held while a tensor is
-# allocated: no effect up to 5 GiB, part of it at 6 and 7 GiB, all of it from 8 GiB on (4096 three-raise
-# roots, first process on a machine: 11.18 / 10.68 / 10.57 / 10.49 / 10.47 / 10.50 ms per iteration with
-# 5 / 6 / 7 / 8 / 9 / 12 GiB).  Tensors below the minimum size are allocated as they come.
-STATE_SPREAD_GAP_BYTES = 9 << 30
-STATE_SPREAD_MIN_TENSOR_BYTES = 256 << 20
+# Placement of the state tensors (``HipSparseCFREvaluator._place_state``): slabs below the minimum are allocated
+# as they come; a second slab that the probe finds in the same third of the card's memory as the first is held,
+# together with a block of the step size, while the next candidate is allocated, at most so many times (the
+# thirds are ~89 GiB); a candidate counts as lying elsewhere when the probe runs in under 0.9 of the time it
+# takes on two halves of the first slab (measured: 0.79-0.81 against 1.0).
+STATE_SPREAD_MIN_SLAB_BYTES = 256 << 20
+STATE_SPREAD_STEP_BYTES = 31 << 30         # held as blocks of 16, 8, 4, 2 and 1 GiB: the driver hands out the highest free
+                                           # block of a request's size class, so every class has to be taken out of the way
+STATE_SPREAD_TRIES = 6
+STATE_SPREAD_ACCEPT = 0.9
+_PROBE_PACKED_BYTES = 10 * 12288 * 1326 * 4     # ten of the probe's arrays at their largest, back to back
+_PROBE_MIN_BYTES = 10 * (256 * 1326 * 4 + 256)  # per buffer: the probe refuses arrays of fewer than 256 rows
 SPLIT_CUT_LEVEL = 2
 # The tree tops (one workgroup per root, five families in a row) are few and long: a second cut right under
 # the root makes the root's family one item and each of its children's families another (six launches per
@@ -201,12 +207,13 @@ class HipSparseCFREvaluator:
         # iteration are not stored) and lets reach_avg alternate between two buffers; the final state is
         # bit-identical either way.  False: every iteration as ``cfr_iteration`` runs it.
         self.lean_search = bool(lean_search)
-        # True: each large state tensor is allocated while a block of STATE_SPREAD_GAP_BYTES, reserved
-        # just before it, is held (``_new_state``: 5-10 % faster iterations; free in a fresh process,
-        # seconds per subgame once the card's memory has been used and given back, so it is for long
-        # searches).  ``state_spread_count``: for how many tensors of the current subgame that was done
+        # True: the state tensors are dealt to two slabs that lie in different thirds of the card's physical
+        # memory, found by measurement (``_place_state``): iterations 6-11 % faster from 1024 roots on; costs
+        # a few probe launches in a process that is the first to use the memory and seconds per subgame once
+        # memory has been used and given back, so it is for long searches.  ``state_placement``: what was done
+        # for the current subgame
         self.spread_state = bool(spread_state)
-        self.state_spread_count = 0
+        self.state_placement: dict = {"placed": False}
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -238,42 +245,81 @@ class HipSparseCFREvaluator:
             t = t.to(dtype)
         return t.to(self.device)
 
-    def _hold_gap(self, nbytes: int) -> ctypes.c_void_p | None:
-        """A block of device memory to hold while ``nbytes`` are allocated, or None where that would
-        not pay or not fit: small tensors, an allocator that would answer from blocks it has cached
-        (they lie where they lie), or a card too full to take the block without pressure."""
-        if not self.spread_state or nbytes < STATE_SPREAD_MIN_TENSOR_BYTES:
-            return None
-        if torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device) >= nbytes:
-            return None
-        free, total = torch.cuda.mem_get_info(self.device)
-        if free - nbytes - STATE_SPREAD_GAP_BYTES < total // 4:
-            return None
-        block = ctypes.c_void_p()
-        code = _lib.load().p2hip_device_reserve(STATE_SPREAD_GAP_BYTES, ctypes.byref(block))
-        return block if code == 0 and block.value else None
+    def _probe_ns_per_row(self, a: int, b: int, nbytes: int) -> float:
+        """Time of the placement probe over the first ``nbytes`` of two buffers, per row it streams (the
+        probe takes as many rows as fit, at most 12 288, so launches over buffers of different size compare)."""
+        ms = ctypes.c_float()
+        _lib.call("p2hip_placement_probe", a, b, nbytes, 3, ctypes.byref(ms), _lib.stream_ptr())
+        rows = min(nbytes // 10 // 256 * 256 // (4 * NUM_HANDS), 12288)
+        return float(ms.value) * 1e6 / rows
 
-    def _new_state(self, *shape: int) -> torch.Tensor:
-        """Zeros of the float dtype for a state tensor of the search.  Where the tensors lie in the
-        card's memory changes the speed of the iteration kernel by 5-10 % (4096 three-raise river roots:
-        11.1 ms per iteration with the tensors allocated back to back by a fresh process, 10.5 ms this
-        way; the depth-2 tree 1.90 -> 1.71 ms; 1024 three-raise roots 2.67-2.82 -> 2.57 ms): with
-        ``spread_state`` each one is allocated while a block of 9 GiB, reserved just before it and released
-        right after, is held.  One block held during the whole construction, blocks before some of the
-        tensors only, address space reserved without memory behind it, tensor bases aligned to 1 GiB or
-        staggered by 0.2-33 MB: none of these changes anything.  Cost: nothing measurable in a process
-        that is the first to use the memory (4096 roots: 1.19 against 1.15 s of construction); 0.15-0.45 s
-        per tensor once memory has been used and released before (the driver clears what it hands out
-        again: 2.3-5.5 s per subgame), which only a long search earns back.  Hence an option, off by
-        default."""
-        nbytes = 4 * int(np.prod(shape))
-        block = self._hold_gap(nbytes)
+    def _place_state(self, shapes: list[tuple[int, ...]]) -> list[torch.Tensor]:
+        """Zero-filled float tensors of the given shapes: the state of a search.
+
+        The iteration kernel writes about ten of them at once, and the card's memory takes that faster when
+        the written tensors lie in two different thirds (~89 GiB each) of its physical address space than when
+        all lie in one: 4096 three-raise river roots 11.0 -> 9.9-10.0 ms per iteration, 2048 roots 5.56 ->
+        5.0 ms, the depth-2 tree 1.86 -> 1.65 ms (tensors carved out of one large allocation at chosen offsets;
+        a state allocated back to back by a fresh process lies inside one third).  Virtual addresses play no
+        part and physical ones are not visible, but two buffers in different thirds show in the time of a
+        small row-streaming kernel (``p2hip_placement_probe``: a fifth less than on two halves of one buffer).
+        With ``spread_state`` the tensors are therefore dealt alternately to two slabs, and the second slab is
+        chosen by that measurement: a candidate in the same third as the first slab is held, together with a
+        block of STATE_SPREAD_STEP_BYTES, while the next one is allocated; the fastest candidate stays, the
+        rest goes back.  The arithmetic does not change.  Cost: a handful of probe launches (0.3 ms each) and
+        allocations - nothing measurable in a process that is the first to use the memory, up to seconds once
+        memory has been used and given back (the driver clears what it hands out again).  Off by default."""
+        dev = self.device
+        sizes = [(4 * int(np.prod(sh)) + 255) // 256 * 256 for sh in shapes]
+        side = [k % 2 for k in range(len(shapes))]
+        slab_bytes = [sum(n for n, c in zip(sizes, side) if c == q) for q in (0, 1)]
+        self.state_placement = {"placed": False}
+        if not self.spread_state or min(slab_bytes) < max(STATE_SPREAD_MIN_SLAB_BYTES, 2 * _PROBE_MIN_BYTES):
+            return [torch.zeros(*sh, dtype=self.float_dtype, device=dev) for sh in shapes]
+        first = torch.empty(slab_bytes[0], dtype=torch.uint8, device=dev)
+        # what the probe takes when all of its arrays lie in one third: the arrays packed into the first
+        # 1.2 GiB of the first slab (a stretch that short hardly ever reaches across a boundary)
+        half = min(slab_bytes[0] // 2 // 256 * 256, _PROBE_PACKED_BYTES)
+        same_ns = self._probe_ns_per_row(first.data_ptr(), first.data_ptr() + half, half)
+        probe_bytes = min(slab_bytes)
+        tried: list[tuple[float, torch.Tensor]] = []
+        blocks: list[ctypes.c_void_p] = []
         try:
-            return torch.zeros(*shape, dtype=self.float_dtype, device=self.device)
+            for attempt in range(STATE_SPREAD_TRIES):
+                free, total = torch.cuda.mem_get_info(dev)
+                if tried and free - slab_bytes[1] < total // 8:
+                    break                                    # no room for another candidate without pressure
+                cand = torch.empty(slab_bytes[1], dtype=torch.uint8, device=dev)
+                tried.append((self._probe_ns_per_row(first.data_ptr(), cand.data_ptr(), probe_bytes), cand))
+                if tried[-1][0] < STATE_SPREAD_ACCEPT * same_ns or attempt == STATE_SPREAD_TRIES - 1:
+                    break
+                free, total = torch.cuda.mem_get_info(dev)
+                if free - STATE_SPREAD_STEP_BYTES - slab_bytes[1] >= total // 8:
+                    piece = STATE_SPREAD_STEP_BYTES + (1 << 30)
+                    while piece > 1 << 30:
+                        piece >>= 1
+                        block = ctypes.c_void_p()
+                        if _lib.load().p2hip_device_reserve(piece, ctypes.byref(block)) == 0 and block.value:
+                            blocks.append(block)
         finally:
-            if block is not None:
-                self.state_spread_count += 1
+            for block in blocks:
                 _lib.call("p2hip_device_release", block)
+        best = min(range(len(tried)), key=lambda k: tried[k][0])
+        second = tried[best][1]
+        self.state_placement = {"placed": True, "probe_ns_per_row_inside_first_slab": same_ns,
+                                "probe_ns_per_row_candidates": [t for t, _ in tried], "chosen": best,
+                                "slab_GiB": [b / 2 ** 30 for b in slab_bytes]}
+        rejected = len(tried) > 1
+        del tried, cand
+        if rejected:
+            torch.cuda.empty_cache()                         # the candidates that were not taken go back to the card
+        slabs = (first.zero_(), second.zero_())
+        out, cursor = [], [0, 0]
+        for sh, n, c in zip(shapes, sizes, side):
+            nbytes = 4 * int(np.prod(sh))
+            out.append(slabs[c][cursor[c]:cursor[c] + nbytes].view(self.float_dtype).view(*sh))
+            cursor[c] += n
+        return out
 
     def _construct_subgame(self, src_env, src_indices) -> None:
         """Build the sparse tree and allocate the state (sparse_cfr_evaluator.py:142-306)."""
@@ -349,13 +395,25 @@ class HipSparseCFREvaluator:
         self.showdown_potential = d_potential[self.showdown_indices]
         self._potential_all = d_potential.to(torch.float32)
 
-        self.state_spread_count = 0
+        # the state of the search, in the order it is dealt to the two slabs of ``_place_state``: five [T, H]
+        # tensors, six [T, 2, H], the scratch rows, and the second reach_avg buffer of a lean search
+        one, two = (T, NUM_HANDS), (T, 2, NUM_HANDS)
+        with_alt = self.fused_iteration and self.lean_search
+        pool = self._place_state([one] * 5 + [two] * 6 + [one] + ([two] if with_alt else []))
+        self._reach_avg_alt = pool.pop() if with_alt else None
+        if with_alt:
+            self._reach_avg_alt[:N] = 1.0
+        pool.reverse()
 
         def z1():
-            return self._new_state(T, NUM_HANDS)
+            t = pool.pop()
+            _req(tuple(t.shape) == one, "state pool: a [T, H] tensor is next")
+            return t
 
         def z2():
-            return self._new_state(T, 2, NUM_HANDS)
+            t = pool.pop()
+            _req(tuple(t.shape) == two, "state pool: a [T, 2, H] tensor is next")
+            return t
 
         self.policy_probs, self.policy_probs_avg, self.policy_probs_sample = z1(), z1(), z1()
         self.cumulative_regrets, self.regret_weight_sums = z1(), z1()
@@ -399,7 +457,6 @@ class HipSparseCFREvaluator:
         self._max_children = int(tree.child_count.max()) if T else 1
         self._has_model_leaves = bool(model_mask.any())
         self._iter_bundles = {}
-        self._reach_avg_alt = None
         split = self.split_small_batches
         if split is None:
             split = N < SPLIT_ROOTS_BELOW or T >= SPLIT_NODES_PER_ROOT * N
@@ -790,7 +847,7 @@ class HipSparseCFREvaluator:
     def _other_reach_avg(self) -> torch.Tensor:
         """The second reach_avg buffer of the alternating scheme (allocated on first use; root rows 1)."""
         if self._reach_avg_alt is None or self._reach_avg_alt.shape != self.self_reach_avg.shape:
-            self._reach_avg_alt = self._new_state(*self.self_reach_avg.shape)
+            self._reach_avg_alt = torch.empty_like(self.self_reach_avg)
             self._reach_avg_alt[:self.root_nodes] = 1.0
         return self._reach_avg_alt
 

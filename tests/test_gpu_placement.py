@@ -1,7 +1,7 @@
-"""GPU: the placement aid (``p2hip_device_reserve`` / ``p2hip_device_release``) and the evaluator's
-``spread_state`` option, which allocates each state tensor while such a block is held.  Placement is
-not arithmetic: a search with the option ends in exactly the state of one without it, the blocks are
-given back, and a block that does not fit is an error code, not a fault."""
+"""GPU: the placement aid (``p2hip_placement_probe``, ``p2hip_device_reserve`` / ``p2hip_device_release``)
+and the evaluator's ``spread_state`` option, which deals the state tensors to two slabs and chooses the
+second slab by the probe.  Placement is not arithmetic: a search with the option ends in exactly the state of
+one without it, what was held goes back, and a block that does not fit is an error code, not a fault."""
 import ctypes
 
 import numpy as np
@@ -47,7 +47,7 @@ def _search(spread: bool, seed: int):
     from poker2_amd.evaluator import HipSparseCFREvaluator
     from poker2_amd.tree import RootStates
     rng = np.random.default_rng(7300 + seed)
-    n = 6
+    n = 48                                          # large enough for the probe: slabs of 100 MB and more
     boards = random_boards(rng, n)
     beliefs = random_ranges(rng, boards)
     roots = RootStates.at_round_start(3, rng.integers(40, 900, n), rng.integers(30, 2500, (n, 2)), boards,
@@ -60,39 +60,65 @@ def _search(spread: bool, seed: int):
     return ev
 
 
+def test_placement_probe_through_the_c_abi():
+    from poker2_amd import _lib
+    lib = _lib.load()
+    nbytes = 64 << 20
+    a = torch.full((nbytes // 4,), 0.5, dtype=torch.float32, device="cuda")
+    b = torch.full((nbytes // 4,), 0.25, dtype=torch.float32, device="cuda")
+    ms = ctypes.c_float(-1.0)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.p2hip_placement_probe(a.data_ptr(), b.data_ptr(), nbytes, 2, ctypes.byref(ms), stream) == 0
+    assert 0.0 < ms.value < 50.0
+    # it streams rows of both buffers and overwrites part of them; everything stays finite and inside the buffers
+    torch.cuda.synchronize()
+    assert torch.isfinite(a).all() and torch.isfinite(b).all()
+    assert not torch.equal(a, torch.full_like(a, 0.5)) or not torch.equal(b, torch.full_like(b, 0.25))
+    # refused: no buffers, no result pointer, a repeat count out of range, buffers too small to say anything
+    assert lib.p2hip_placement_probe(None, b.data_ptr(), nbytes, 2, ctypes.byref(ms), stream) != 0
+    assert lib.p2hip_placement_probe(a.data_ptr(), b.data_ptr(), nbytes, 2, None, stream) != 0
+    assert lib.p2hip_placement_probe(a.data_ptr(), b.data_ptr(), nbytes, 0, ctypes.byref(ms), stream) != 0
+    assert lib.p2hip_placement_probe(a.data_ptr(), b.data_ptr(), 1 << 20, 2, ctypes.byref(ms), stream) != 0
+
+
 def test_spread_state_changes_where_the_state_lies_and_nothing_else(monkeypatch):
     import poker2_amd.evaluator as E
-    # the test's tensors are small: let the option apply to them, with a block that fits any card
-    monkeypatch.setattr(E, "STATE_SPREAD_MIN_TENSOR_BYTES", 0)
-    monkeypatch.setattr(E, "STATE_SPREAD_GAP_BYTES", 48 << 20)
+    # the test's state is small: let the option apply to it, with steps that fit any card
+    monkeypatch.setattr(E, "STATE_SPREAD_MIN_SLAB_BYTES", 32 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_STEP_BYTES", 63 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_TRIES", 3)
     torch.cuda.empty_cache()
     plain = _search(False, 0)
-    assert plain.state_spread_count == 0
+    assert plain.state_placement == {"placed": False}
     torch.cuda.synchronize()
     free_before, _ = torch.cuda.mem_get_info()
     cached_before = torch.cuda.memory_reserved()
     spread = _search(True, 0)
-    # cached blocks of the allocator may serve some of the tensors; the others went behind a block
-    assert 0 <= spread.state_spread_count <= 13
+    p = spread.state_placement
+    assert p["placed"] and 1 <= len(p["probe_ns_per_row_candidates"]) <= 3
+    assert p["probe_ns_per_row_inside_first_slab"] > 0 and 0 <= p["chosen"] < len(p["probe_ns_per_row_candidates"])
+    assert p["probe_ns_per_row_candidates"][p["chosen"]] == min(p["probe_ns_per_row_candidates"])
     for name in STATE:
         assert torch.equal(getattr(plain, name), getattr(spread, name)), name
+    # the tensors of a side lie in one slab, neighbours in the dealing order in different slabs
+    base = {spread.policy_probs.untyped_storage().data_ptr(), spread.policy_probs_avg.untyped_storage().data_ptr()}
+    assert len(base) == 2
+    assert spread.policy_probs_sample.untyped_storage().data_ptr() == spread.policy_probs.untyped_storage().data_ptr()
+    assert spread.cumulative_regrets.untyped_storage().data_ptr() == spread.policy_probs_avg.untyped_storage().data_ptr()
     torch.cuda.synchronize()
     free_after, _ = torch.cuda.mem_get_info()
     grown = torch.cuda.memory_reserved() - cached_before          # what the tensors' allocator took meanwhile
     assert (free_before - free_after) - grown < 16 << 20, "the held blocks were given back"
 
 
-def test_spread_state_places_tensors_when_the_allocator_has_nothing_cached(monkeypatch):
+def test_a_second_subgame_on_the_same_evaluator_places_its_state_again(monkeypatch):
     import poker2_amd.evaluator as E
-    monkeypatch.setattr(E, "STATE_SPREAD_MIN_TENSOR_BYTES", 0)
-    monkeypatch.setattr(E, "STATE_SPREAD_GAP_BYTES", 48 << 20)
-    from poker2_amd.config import river_dcfr_config
-    from poker2_amd.evaluator import HipSparseCFREvaluator
-    ev = HipSparseCFREvaluator(None, torch.device("cuda"), river_dcfr_config(1, iterations=2, depth=2), spread_state=True)
-    torch.cuda.empty_cache()
-    # large enough that no cached small-pool block serves it
-    t = ev._new_state(3000, 2, 1326)
-    assert ev.state_spread_count == 1 and float(t.abs().sum()) == 0.0
-    off = HipSparseCFREvaluator(None, torch.device("cuda"), river_dcfr_config(1, iterations=2, depth=2))
-    off._new_state(3000, 2, 1326)
-    assert off.state_spread_count == 0
+    monkeypatch.setattr(E, "STATE_SPREAD_MIN_SLAB_BYTES", 32 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_STEP_BYTES", 63 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_TRIES", 2)
+    a = _search(True, 1)
+    first = {name: getattr(a, name).clone() for name in STATE}
+    b = _search(True, 1)
+    assert a.state_placement["placed"] and b.state_placement["placed"]
+    for name in STATE:
+        assert torch.equal(first[name], getattr(b, name)), name
