@@ -324,6 +324,12 @@ def main() -> None:
     torch.cuda.synchronize()
     t_build = time.perf_counter() - t_build
     placed = dict(ev.state_placement)
+    if placed.get("placed"):
+        # the probe streams 20 rows of 5304 B per node: its rate with all arrays in one third of the card's
+        # memory, and dealt to the two slabs the state lies in
+        per_row = 20 * H * 4
+        placed["probe_GBps_inside_first_slab"] = per_row / placed["probe_ns_per_row_inside_first_slab"]
+        placed["probe_GBps_chosen_slabs"] = per_row / placed["probe_ns_per_row_candidates"][placed["chosen"]]
     nodes_per_root = ev.total_nodes // ev.root_nodes
     launches = 1 if ev._items is None else 2 * len(ev._items.tiers)
 
@@ -415,7 +421,9 @@ def main() -> None:
                      "flat_stream_note": "p2hip_stream_probe: 5 arrays read + 7 written, 512 MiB each, ordinary and "
                                          "non-temporal accesses, measured by this run after the timed region; the "
                                          "kernel's bytes (counted traffic where a counter run exists, else "
-                                         "algorithmic) over its time, as a share of the faster of the two",
+                                         "algorithmic) over its time, as a share of the faster of the two; the probe's "
+                                         "arrays lie back to back, i.e. in one third of the card's memory, so this is "
+                                         "no ceiling for a state placed across two thirds (config.state_placement)",
                      "frac_of_flat_stream": moved / (kernel_ms * 1e-3) / 1e9 / max(flat.values())},
     }
     if not args.no_cpu_baseline:
