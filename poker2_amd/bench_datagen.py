@@ -47,6 +47,9 @@ def main() -> None:
     ap.add_argument("--roots", type=int, default=16384)
     ap.add_argument("--iterations", type=int, default=64)
     ap.add_argument("--max-raises", type=int, default=3)
+    ap.add_argument("--spread-state", action="store_true",
+                    help="the evaluator's placement option: the state tensors dealt to two slabs in different thirds "
+                         "of the card's memory (set-up takes longer)")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -58,7 +61,7 @@ def main() -> None:
     gen = torch.Generator(device=dev)
     gen.manual_seed(1)
     ev = HipSparseCFREvaluator(model, dev, river_dcfr_config(b, iterations=args.iterations, depth=64), generator=gen,
-                               max_raises=args.max_raises)
+                               max_raises=args.max_raises, spread_state=args.spread_state)
 
     def step():
         torch.cuda.synchronize()
@@ -78,7 +81,7 @@ def main() -> None:
     (setup, search, data), nxt, (vb, pvb, pb) = step()
     out = {"roots": b, "nodes": ev.total_nodes, "model_leaves": int(ev.model_indices.numel()),
            "showdown_leaves": int(ev.showdown_indices.numel()), "iterations": args.iterations,
-           "setup_s": setup, "search_s": search, "training_data_s": data, "ms_per_iteration": search / args.iterations * 1e3,
+           "state_placed": bool(ev.state_placement.get("placed")), "setup_s": setup, "search_s": search, "training_data_s": data, "ms_per_iteration": search / args.iterations * 1e3,
            "subgame_iterations_per_s": b * args.iterations / search, "public_states_per_s": b / (setup + search + data),
            "value_samples": len(vb) + len(pvb), "policy_samples": len(pb), "next_roots": nxt.roots.n,
            "peak_GiB": torch.cuda.max_memory_allocated() / 2**30}
