@@ -50,6 +50,8 @@ def main() -> None:
     ap.add_argument("--spread-state", action="store_true",
                     help="the evaluator's placement option: the state tensors dealt to two slabs in different thirds "
                          "of the card's memory (set-up takes longer)")
+    ap.add_argument("--reuse-state", action="store_true",
+                    help="the evaluator keeps its state slabs from step to step (a placement is then paid for once)")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -61,7 +63,8 @@ def main() -> None:
     gen = torch.Generator(device=dev)
     gen.manual_seed(1)
     ev = HipSparseCFREvaluator(model, dev, river_dcfr_config(b, iterations=args.iterations, depth=64), generator=gen,
-                               max_raises=args.max_raises, spread_state=args.spread_state)
+                               max_raises=args.max_raises, spread_state=args.spread_state,
+                               reuse_state=args.reuse_state)
 
     def step():
         torch.cuda.synchronize()

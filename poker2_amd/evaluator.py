@@ -150,7 +150,7 @@ class HipSparseCFREvaluator:
                  compile_model: bool = True, fused_iteration: bool = True,
                  max_raises: int | None = None, tree_builder: str = "device",
                  split_small_batches: bool | None = None, lean_search: bool = True,
-                 spread_state: bool = False) -> None:
+                 spread_state: bool = False, reuse_state: bool = False) -> None:
         self.device = torch.device(device)
         if model is not None and not hasattr(model, "leaf_values"):
             # the reference hands its network over as is (cfr_evaluator.py:306-322, 1025-1047): its
@@ -214,6 +214,12 @@ class HipSparseCFREvaluator:
         # for the current subgame
         self.spread_state = bool(spread_state)
         self.state_placement: dict = {"placed": False}
+        # True: the state tensors of successive subgames are views into the same two slabs (a quarter larger
+        # than the first subgame needs, replaced when one needs more), so a placement is paid for once.  The
+        # reference allocates a fresh state per subgame: with this option every state tensor of an EARLIER
+        # subgame, and any view of one, is overwritten by the next ``initialize_subgame``
+        self.reuse_state = bool(reuse_state)
+        self._arena: tuple[torch.Tensor, torch.Tensor] | None = None
         self.stats: dict = {}
         self.root_nodes = cfg.num_envs
         self.total_nodes = 0
@@ -273,10 +279,41 @@ class HipSparseCFREvaluator:
         sizes = [(4 * int(np.prod(sh)) + 255) // 256 * 256 for sh in shapes]
         side = [k % 2 for k in range(len(shapes))]
         slab_bytes = [sum(n for n, c in zip(sizes, side) if c == q) for q in (0, 1)]
+
+        def carve(slabs):
+            out, cursor = [], [0, 0]
+            for sh, n, c in zip(shapes, sizes, side):
+                nbytes = 4 * int(np.prod(sh))
+                out.append(slabs[c][cursor[c]:cursor[c] + nbytes].view(self.float_dtype).view(*sh))
+                cursor[c] += n
+            for c in (0, 1):
+                slabs[c][:cursor[c]].zero_()
+            return out
+
+        if self.reuse_state and self._arena is not None:
+            if all(self._arena[q].numel() >= slab_bytes[q] for q in (0, 1)):
+                self.state_placement = dict(self.state_placement, reused=True)
+                return carve(self._arena)
+            self._drop_state()                               # the slabs are too small: give them back first
         self.state_placement = {"placed": False}
-        if not self.spread_state or min(slab_bytes) < max(STATE_SPREAD_MIN_SLAB_BYTES, 2 * _PROBE_MIN_BYTES):
+        place = self.spread_state and min(slab_bytes) >= max(STATE_SPREAD_MIN_SLAB_BYTES, 2 * _PROBE_MIN_BYTES)
+        if not place and not self.reuse_state:
             return [torch.zeros(*sh, dtype=self.float_dtype, device=dev) for sh in shapes]
+        if self.reuse_state:
+            slab_bytes = [(b + b // 4 + 255) // 256 * 256 for b in slab_bytes]
         first = torch.empty(slab_bytes[0], dtype=torch.uint8, device=dev)
+        if place:
+            second = self._second_slab_elsewhere(first, slab_bytes)
+        else:
+            second = torch.empty(slab_bytes[1], dtype=torch.uint8, device=dev)
+        if self.reuse_state:
+            self._arena = (first, second)
+        return carve((first, second))
+
+    def _second_slab_elsewhere(self, first: torch.Tensor, slab_bytes: list[int]) -> torch.Tensor:
+        """The second slab of ``_place_state``: of the candidates probed against ``first`` the one with the
+        shortest probe time; candidates that were not taken go back to the card."""
+        dev = self.device
         # what the probe takes when all of its arrays lie in one third: the arrays packed into the first
         # 1.2 GiB of the first slab (a stretch that short hardly ever reaches across a boundary)
         half = min(slab_bytes[0] // 2 // 256 * 256, _PROBE_PACKED_BYTES)
@@ -296,6 +333,7 @@ class HipSparseCFREvaluator:
                         raise
                     break                                    # what was found so far has to do
                 tried.append((self._probe_ns_per_row(first.data_ptr(), cand.data_ptr(), probe_bytes), cand))
+                cand = None
                 if tried[-1][0] < STATE_SPREAD_ACCEPT * same_ns or attempt == STATE_SPREAD_TRIES - 1:
                     break
                 free, total = torch.cuda.mem_get_info(dev)
@@ -316,16 +354,23 @@ class HipSparseCFREvaluator:
                                 "slab_GiB": [b / 2 ** 30 for b in slab_bytes]}
         rejected = len(tried) > 1
         tried.clear()
-        cand = None
         if rejected:
             torch.cuda.empty_cache()                         # the candidates that were not taken go back to the card
-        slabs = (first.zero_(), second.zero_())
-        out, cursor = [], [0, 0]
-        for sh, n, c in zip(shapes, sizes, side):
-            nbytes = 4 * int(np.prod(sh))
-            out.append(slabs[c][cursor[c]:cursor[c] + nbytes].view(self.float_dtype).view(*sh))
-            cursor[c] += n
-        return out
+        return second
+
+    _STATE_TENSORS = ("policy_probs", "policy_probs_avg", "policy_probs_sample", "cumulative_regrets",
+                      "regret_weight_sums", "beliefs", "beliefs_avg", "self_reach", "self_reach_avg", "latest_values",
+                      "values_avg", "_scratch", "_reach_avg_alt")
+
+    def _drop_state(self) -> None:
+        """Let go of the state tensors and their slabs (``reuse_state``), so that larger slabs can take
+        their place on the card."""
+        for name in self._STATE_TENSORS:
+            setattr(self, name, None)
+        self._arena = None
+        self._iter_bundles = {}
+        self.last_model_values = None
+        torch.cuda.empty_cache()
 
     def _construct_subgame(self, src_env, src_indices) -> None:
         """Build the sparse tree and allocate the state (sparse_cfr_evaluator.py:142-306)."""
@@ -1208,6 +1253,9 @@ class HipSparseCFREvaluator:
         actions_root = self.env.actions_this_round[:N]
         if exclude_start:
             value_batch = value_batch[~((street_root == 0) & (actions_root == 0))]
+        elif self.reuse_state:
+            # the features of all roots would be a view of the state, which the next subgame overwrites
+            value_batch = value_batch[torch.arange(N, device=dev)]
         policy_batch = RebelBatch(features=features[valid_top], policy_targets=self._policy_targets(policy_rows, check_rows=False),
                                   legal_masks=legal_masks[:top][valid_top], statistics=policy_statistics)
 

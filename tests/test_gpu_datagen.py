@@ -592,8 +592,9 @@ def compare_generator_batch(g, prefix, batch, cols, every_entry):
         all_close(pt[:, cols, :], g[f"{prefix}/policy_targets"], ok[:, cols, None], "policy_targets", f"{prefix} policy targets")
 
 
+@pytest.mark.parametrize("reuse_state", [False, True])
 @pytest.mark.parametrize("fixture", ["base", "fused"])
-def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
+def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture, reuse_state):
     """The whole self-play loop (rebel_data_generator.py:52-95) against a run of the reference's own
     generator, evaluator and env from the same two seeds: the same hands are dealt, the same
     batches reach the buffers pass by pass, the call returns the same samples and leaves the same
@@ -611,7 +612,8 @@ def test_generator_loop_reproduces_the_reference_run(golden_dir, fixture):
     search_gen.manual_seed(search_seed)
     proto = EnvProto(mean_stack=1000, sb=50, bb=100, randomize_stacks=True, rng=env_gen)
     ev = HipSparseCFREvaluator(NetworkLeafModel(ValueNet(), DEV), torch.device(DEV),
-                               river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0), generator=search_gen)
+                               river_dcfr_config(n, iterations=iters, depth=depth, dcfr_delay=0), generator=search_gen,
+                               reuse_state=reuse_state)         # the buffers keep every pass's batches: nothing may alias the state
 
     class Recorder:
         def __init__(self):

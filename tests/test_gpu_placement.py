@@ -122,3 +122,50 @@ def test_a_second_subgame_on_the_same_evaluator_places_its_state_again(monkeypat
     assert a.state_placement["placed"] and b.state_placement["placed"]
     for name in STATE:
         assert torch.equal(first[name], getattr(b, name)), name
+
+
+def _search_on(ev, seed: int, n: int, iterations: int = 9):
+    from poker2_amd.tree import RootStates
+    rng = np.random.default_rng(7400 + seed)
+    boards = random_boards(rng, n)
+    beliefs = random_ranges(rng, boards)
+    roots = RootStates.at_round_start(3, rng.integers(40, 900, n), rng.integers(30, 2500, (n, 2)), boards,
+                                      button=rng.integers(0, 2, n))
+    ev.generator.manual_seed(5)                     # the sampling schedule is drawn per search
+    ev.initialize_subgame(roots, np.arange(n), torch.from_numpy(beliefs))
+    ev.evaluate_cfr()
+    return {name: getattr(ev, name).clone() for name in STATE}
+
+
+def _evaluator(n: int, **kw):
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    cfg = river_dcfr_config(n, iterations=9, depth=4, dcfr_delay=0)
+    return HipSparseCFREvaluator(None, torch.device("cuda"), cfg, torch.Generator().manual_seed(5), max_raises=2, **kw)
+
+
+@pytest.mark.parametrize("spread", [False, True])
+def test_reuse_state_keeps_the_slabs_across_subgames_and_the_results(monkeypatch, spread):
+    """``reuse_state``: successive subgames of one evaluator live in the same two slabs (replaced when a
+    subgame needs more), and every one of them ends in the state a fresh evaluator reaches."""
+    import poker2_amd.evaluator as E
+    monkeypatch.setattr(E, "STATE_SPREAD_MIN_SLAB_BYTES", 32 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_STEP_BYTES", 63 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_TRIES", 2)
+    sizes = [(0, 40), (1, 24), (2, 44), (3, 96), (4, 30)]        # second and third fit the first slabs; the fourth does not
+    kept = _evaluator(40, reuse_state=True, spread_state=spread)
+    slabs = []
+    for seed, n in sizes:
+        kept.cfg.num_envs = n
+        got = _search_on(kept, seed, n)
+        slabs.append(tuple(t.data_ptr() for t in kept._arena))
+        want = _search_on(_evaluator(n), seed, n)
+        for name in STATE:
+            assert torch.equal(got[name], want[name]), (name, seed)
+        assert kept.policy_probs.untyped_storage().data_ptr() == kept._arena[0].data_ptr()
+        assert kept.policy_probs_avg.untyped_storage().data_ptr() == kept._arena[1].data_ptr()
+    assert slabs[0] == slabs[1] == slabs[2], "subgames that fit keep the slabs"
+    assert kept._arena[0].numel() >= 2 * 96 * 1326 * 4, "the large subgame got larger slabs"
+    assert slabs[3] == slabs[4], "and the next small one stays in them"
+    if spread:
+        assert kept.state_placement["placed"] and kept.state_placement.get("reused")
