@@ -161,7 +161,7 @@ def flat_stream_rate(pairs: int = 1 << 26, reps: int = 5) -> dict:
     return out
 
 
-def side_metrics(skip=()) -> dict:
+def side_metrics(skip=(), spread_state: bool = False) -> dict:
     """Showdown evaluations/s (B=4096 public states) and hands ranked/s (2^20 hands)."""
     import torch
     from poker2_amd import rules_hip
@@ -204,7 +204,8 @@ def side_metrics(skip=()) -> dict:
     out["rank7_ms_per_call_2e20"] = ms
     # the batch the reference's own settings search at a time (num_envs: 192), on the three-raise tree: few roots
     # are cut into work items that get a workgroup each
-    small, _, _ = make_evaluator(192, "raise3", 42, iterations=64)
+    small, _, _ = make_evaluator(192, "raise3", 42, iterations=64, spread_state=spread_state)
+    out["state_placed_B192"] = bool(small.state_placement.get("placed"))
     for mode, kw in MODES.items():
         for t in range(1, 6):
             small.cfr_iteration(t, **kw)
@@ -225,8 +226,12 @@ def side_metrics(skip=()) -> dict:
     for roots, tree in ((4096, "depth2"), (4096, "raise1"), (1024, "depth2"), (1024, "raise3")):
         if (roots, tree) == tuple(skip):
             continue
-        ev, _, _ = make_evaluator(roots, tree, 42, iterations=64)
-        row = {"roots": roots, "tree": tree, "nodes_per_root": ev.total_nodes // roots}
+        ev, _, _ = make_evaluator(roots, tree, 42, iterations=64, spread_state=spread_state)
+        p = ev.state_placement
+        row = {"roots": roots, "tree": tree, "nodes_per_root": ev.total_nodes // roots,
+               "state_placed": bool(p.get("placed")),
+               "probe_ns_per_row": ([p["probe_ns_per_row_inside_first_slab"]] + p["probe_ns_per_row_candidates"])
+               if p.get("placed") else None}
         for mode, kw in MODES.items():
             for t in range(6):
                 ev.cfr_iteration(t, **kw)
@@ -429,7 +434,7 @@ def main() -> None:
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.tree, args.seed)
     if not args.no_extra:
-        result["extra"] = side_metrics(skip=(args.roots, args.tree))
+        result["extra"] = side_metrics(skip=(args.roots, args.tree), spread_state=not args.no_spread)
         if not args.no_cpu_baseline:
             result["extra"]["cpu"] = cpu_side_baselines()
     print(json.dumps(result))
