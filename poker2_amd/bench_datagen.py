@@ -84,7 +84,10 @@ def main() -> None:
     (setup, search, data), nxt, (vb, pvb, pb) = step()
     out = {"roots": b, "nodes": ev.total_nodes, "model_leaves": int(ev.model_indices.numel()),
            "showdown_leaves": int(ev.showdown_indices.numel()), "iterations": args.iterations,
-           "state_placed": bool(ev.state_placement.get("placed")), "setup_s": setup, "search_s": search, "training_data_s": data, "ms_per_iteration": search / args.iterations * 1e3,
+           "state_placed": bool(ev.state_placement.get("placed")),
+           "placement_probe_ns_per_row": ([ev.state_placement["probe_ns_per_row_inside_first_slab"]] +
+                                          ev.state_placement["probe_ns_per_row_candidates"])
+           if ev.state_placement.get("placed") else None, "setup_s": setup, "search_s": search, "training_data_s": data, "ms_per_iteration": search / args.iterations * 1e3,
            "subgame_iterations_per_s": b * args.iterations / search, "public_states_per_s": b / (setup + search + data),
            "value_samples": len(vb) + len(pvb), "policy_samples": len(pb), "next_roots": nxt.roots.n,
            "peak_GiB": torch.cuda.max_memory_allocated() / 2**30}
@@ -92,6 +95,8 @@ def main() -> None:
         print(json.dumps(out))
     else:
         for k, v in out.items():
+            if isinstance(v, list):
+                v = " ".join(f"{x:.1f}" for x in v)
             print(f"{k:28s} {v:.4g}" if isinstance(v, float) else f"{k:28s} {v}")
 
 

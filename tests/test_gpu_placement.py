@@ -169,3 +169,41 @@ def test_reuse_state_keeps_the_slabs_across_subgames_and_the_results(monkeypatch
     assert slabs[3] == slabs[4], "and the next small one stays in them"
     if spread:
         assert kept.state_placement["placed"] and kept.state_placement.get("reused")
+
+
+def test_graph_replay_on_a_placed_state(monkeypatch):
+    """A captured iteration (fused_cfr_triton.py:2359-2451) replays on state tensors that are views into
+    the two slabs exactly as eager iterations run on separately allocated ones."""
+    import poker2_amd.evaluator as E
+    from poker2_amd.fused_cfr_hip import GraphedCFRIteration, _EvaluatorStateSnapshot
+    from poker2_amd.tree import RootStates
+    monkeypatch.setattr(E, "STATE_SPREAD_MIN_SLAB_BYTES", 32 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_STEP_BYTES", 63 << 20)
+    monkeypatch.setattr(E, "STATE_SPREAD_TRIES", 2)
+    n, iters = 48, 8
+    rng = np.random.default_rng(7500)
+    boards = random_boards(rng, n)
+    beliefs = torch.from_numpy(random_ranges(rng, boards))
+    roots = RootStates.at_round_start(3, rng.integers(40, 900, n), rng.integers(30, 2500, (n, 2)), boards,
+                                      button=rng.integers(0, 2, n))
+
+    def ready(**kw):
+        ev = _evaluator(n, **kw)
+        ev.initialize_subgame(roots, np.arange(n), beliefs)
+        ev.prepare_search(t_sample=torch.full((ev.total_nodes,), 5, dtype=torch.long))
+        return ev
+    eager, graphed = ready(), ready(spread_state=True, reuse_state=True)
+    assert graphed.state_placement["placed"] and not eager.state_placement["placed"]
+    for t in range(3):
+        eager.cfr_iteration(t)
+        graphed.cfr_iteration(t)
+    snap = _EvaluatorStateSnapshot.from_evaluator(graphed)
+    runner = GraphedCFRIteration(graphed)
+    runner.capture(t_capture=3, num_warmup=0)
+    snap.restore_to(graphed)
+    for t in range(3, iters):
+        eager.cfr_iteration(t)
+        runner.replay(t)
+        torch.cuda.synchronize()
+    for name in STATE:
+        assert torch.equal(getattr(eager, name), getattr(graphed, name)), name
