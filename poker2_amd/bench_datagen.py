@@ -52,6 +52,8 @@ def main() -> None:
                          "of the card's memory (set-up takes longer)")
     ap.add_argument("--reuse-state", action="store_true",
                     help="the evaluator keeps its state slabs from step to step (a placement is then paid for once)")
+    ap.add_argument("--split", choices=["auto", "on", "off"], default="auto",
+                    help="cut every root's tree into work items (auto: the evaluator's rule)")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -64,7 +66,8 @@ def main() -> None:
     gen.manual_seed(1)
     ev = HipSparseCFREvaluator(model, dev, river_dcfr_config(b, iterations=args.iterations, depth=64), generator=gen,
                                max_raises=args.max_raises, spread_state=args.spread_state,
-                               reuse_state=args.reuse_state)
+                               reuse_state=args.reuse_state,
+                               split_small_batches={"auto": None, "on": True, "off": False}[args.split])
 
     def step():
         torch.cuda.synchronize()
