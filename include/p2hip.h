@@ -452,7 +452,7 @@ int p2hip_stream_probe(const float* in, float* out, int64_t pairs, int n_read, i
 
 /* No counterpart in the reference (PyTorch's allocator places its tensors).  The iteration kernel writes
  * about ten tensors at once, and the card's memory takes that 10 % faster when the written tensors lie in
- * two different thirds (~89 GiB each) of its physical address space instead of one.  Where an allocation
+ * two different thirds (~96 GiB each) of its physical address space instead of one.  Where an allocation
  * lies physically is not visible, but it can be measured and steered:
  *
  * p2hip_placement_probe: time of one launch (ms, mean of `reps`, 1..64) of a row-streaming kernel - 12 rows

@@ -5,7 +5,7 @@
 // address space than when they all lie in one (a row-streaming probe, 12 rows read and 8 written per
 // node from 20 arrays: 4.2 TB/s with all arrays in one third, 5.2-5.3 TB/s with the written ones split
 // between two; moving only read arrays changes nothing; a third region adds 2 %.  4096 three-raise river
-// roots: 11.0 ms per iteration against 9.9-10.0 ms).  The thirds are ~89 GiB each; virtual addresses,
+// roots: 11.0 ms per iteration against 9.9-10.0 ms).  The thirds are ~96 GiB each; virtual addresses,
 // alignment and address translation play no part, and where an allocation lands physically is not visible
 // to a process - but it can be MEASURED: p2hip_placement_probe times that probe with its arrays dealt
 // alternately to two buffers, and two buffers in different thirds show by a time a fifth shorter than two

@@ -80,7 +80,7 @@ SPLIT_ROOTS_BELOW = 400
 # Placement of the state tensors (``HipSparseCFREvaluator._place_state``): slabs below the minimum are allocated
 # as they come; a second slab that the probe finds in the same third of the card's memory as the first is held,
 # together with a block of the step size, while the next candidate is allocated, at most so many times (the
-# thirds are ~89 GiB); a candidate counts as lying elsewhere when the probe runs in under 0.9 of the time it
+# thirds are ~96 GiB); a candidate counts as lying elsewhere when the probe runs in under 0.9 of the time it
 # takes on two halves of the first slab (measured: 0.79-0.81 against 1.0).
 STATE_SPREAD_MIN_SLAB_BYTES = 256 << 20
 STATE_SPREAD_STEP_BYTES = 31 << 30         # held as blocks of 16, 8, 4, 2 and 1 GiB: the driver hands out the highest free
@@ -263,7 +263,7 @@ class HipSparseCFREvaluator:
         """Zero-filled float tensors of the given shapes: the state of a search.
 
         The iteration kernel writes about ten of them at once, and the card's memory takes that faster when
-        the written tensors lie in two different thirds (~89 GiB each) of its physical address space than when
+        the written tensors lie in two different thirds (~96 GiB each) of its physical address space than when
         all lie in one: 4096 three-raise river roots 11.0 -> 9.9-10.0 ms per iteration, 2048 roots 5.56 ->
         5.0 ms, the depth-2 tree 1.86 -> 1.65 ms (tensors carved out of one large allocation at chosen offsets;
         a state allocated back to back by a fresh process lies inside one third).  Virtual addresses play no
