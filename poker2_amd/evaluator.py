@@ -79,9 +79,10 @@ _PHASE_LEAN = 16
 SPLIT_ROOTS_BELOW = 400
 # Placement of the state tensors (``HipSparseCFREvaluator._place_state``): slabs below the minimum are allocated
 # as they come; a second slab that the probe finds in the same third of the card's memory as the first is held,
-# together with a block of the step size, while the next candidate is allocated, at most so many times (the
-# thirds are ~96 GiB); a candidate counts as lying elsewhere when the probe runs in under 0.9 of the time it
-# takes on two halves of the first slab (measured: 0.79-0.81 against 1.0).
+# together with blocks that add up to the step size, while the next candidate is allocated, at most so many
+# times (the thirds are ~96 GiB: three steps cross one); a candidate counts as lying elsewhere when the probe
+# runs in under 0.9 of the time it takes with all of its arrays packed into the start of the first slab
+# (measured: 0.80-0.85 against 1.0).
 STATE_SPREAD_MIN_SLAB_BYTES = 256 << 20
 STATE_SPREAD_STEP_BYTES = 31 << 30         # held as blocks of 16, 8, 4, 2 and 1 GiB: the driver hands out the highest free
                                            # block of a request's size class, so every class has to be taken out of the way
