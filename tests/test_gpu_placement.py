@@ -207,3 +207,42 @@ def test_graph_replay_on_a_placed_state(monkeypatch):
         torch.cuda.synchronize()
     for name in STATE:
         assert torch.equal(getattr(eager, name), getattr(graphed, name)), name
+
+
+def test_placement_at_full_size_B1024_three_raise_tree():
+    """BASELINE configuration 3's shape (1024 river roots, three-raise tree, 105 nodes per root) with the
+    option's real constants - slabs of 5.8 and 4.8 GiB, steps of 31 GiB: the placed search ends in exactly
+    the state of the search on tensors as allocated, and what was held is back on the card."""
+    from poker2_amd.config import river_dcfr_config
+    from poker2_amd.evaluator import HipSparseCFREvaluator
+    from poker2_amd.tree import RootStates
+    n = 1024
+    rng = np.random.default_rng(77)
+    boards = random_boards(rng, n)
+    beliefs = torch.from_numpy(random_ranges(rng, boards))
+    roots = RootStates.at_round_start(3, np.full(n, 200), np.tile([[800, 800]], (n, 1)), boards, button=np.arange(n) % 2)
+    torch.cuda.empty_cache()
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    states = []
+    for spread in (False, True):
+        ev = HipSparseCFREvaluator(None, torch.device("cuda"), river_dcfr_config(n, iterations=24, depth=16, dcfr_delay=0),
+                                   torch.Generator().manual_seed(3), max_raises=3, spread_state=spread)
+        ev.initialize_subgame(roots, np.arange(n), beliefs)
+        assert ev.total_nodes == 105 * n
+        ev.evaluate_cfr()
+        p = ev.state_placement
+        assert p["placed"] == spread
+        if spread:
+            assert 1 <= len(p["probe_ns_per_row_candidates"]) <= 6 and 5.0 < p["probe_ns_per_row_inside_first_slab"] < 200.0
+            assert min(p["probe_ns_per_row_candidates"]) <= 1.05 * p["probe_ns_per_row_inside_first_slab"]
+            print("placement at B=1024:", {k: (round(v, 2) if isinstance(v, float) else v) for k, v in p.items()})
+        states.append({name: getattr(ev, name).clone() for name in STATE})
+        del ev
+    for name in STATE:
+        assert torch.equal(states[0][name], states[1][name]), name
+    del states
+    torch.cuda.empty_cache()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_before - free_after < 1 << 30, "slabs, candidates and held blocks are back on the card"
